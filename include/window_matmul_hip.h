@@ -1,0 +1,119 @@
+/*
+ * C ABI of the MI355X (gfx950) banded-matmul library, libwindow_matmul_hip.so.
+ *
+ * These entry points are what a binding of the reference's native module
+ * `window_matmul_kernel` (reference csrc/window_matmul/window_matmul.cpp:100-106)
+ * calls for tensors that live on the GPU.  They replace the reference's CUDA
+ * launchers (reference csrc/window_matmul/cuda/window_matmul_cuda.h:5-10).
+ *
+ * Conventions
+ *   - All pointers are device pointers on the current HIP device; the caller
+ *     owns every buffer.  The library allocates nothing, never synchronises and
+ *     keeps no mutable state, so it may be called from several host threads.
+ *   - Work is enqueued on `stream` (a hipStream_t passed as void*; NULL is the
+ *     legacy default stream) and the call returns as soon as it is enqueued.
+ *   - Every operand is a rank-3 view described by a base pointer and ELEMENT
+ *     strides for (batch, row, column); any strides are accepted.  The fast
+ *     kernels need unit column stride and 16-byte aligned rows; other layouts
+ *     run on the slower strided kernels, with identical results.
+ *   - Outputs need not be zeroed: every element is written, and band entries
+ *     that fall outside the sequence are written as +0.0.
+ *   - Band convention: column j of band row i addresses source row c = i+j-w,
+ *     valid iff 0 <= c < M.  Invalid entries of an INPUT band are never read.
+ *   - Accumulation is float32 for f32/f16/bf16 storage and float64 for f64.
+ *   - Return value: WM_OK (0) when the work was enqueued, otherwise a wm_status
+ *     code; nothing is enqueued on error.  wm_status_string() names the code.
+ */
+#ifndef WINDOW_MATMUL_HIP_H
+#define WINDOW_MATMUL_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define WM_ABI_VERSION 1
+
+typedef enum wm_dtype {
+  WM_DTYPE_F32 = 0,
+  WM_DTYPE_F16 = 1,
+  WM_DTYPE_BF16 = 2,
+  WM_DTYPE_F64 = 3
+} wm_dtype;
+
+typedef enum wm_status {
+  WM_OK = 0,
+  WM_ERR_NULL_POINTER = 1,     /* a required operand or its data pointer is NULL */
+  WM_ERR_BAD_SHAPE = 2,        /* negative extent, or an extent beyond 2^31-1      */
+  WM_ERR_BAD_DTYPE = 3,        /* dtype is not a wm_dtype value                     */
+  WM_ERR_BAD_FLAGS = 4,        /* unknown bit set in flags                          */
+  WM_ERR_LAUNCH_FAILED = 5,    /* the HIP runtime rejected a kernel launch          */
+  WM_ERR_NO_DEVICE_CODE = 6    /* the library holds no code object for this GPU     */
+} wm_status;
+
+/* Kernel selection.  0 lets the library choose per (shape, dtype, layout). */
+#define WM_FLAG_FORCE_STRIDED 0x1u /* always use the strided fallback kernels (A/B testing) */
+
+/* Rank-3 operand: element (b, r, c) lives at data + b*stride_b + r*stride_r + c*stride_c. */
+typedef struct wm_operand {
+  void *data;
+  int64_t stride_b;
+  int64_t stride_r;
+  int64_t stride_c;
+} wm_operand;
+
+/* A[b,i,j] = sum_h q[b,i,h] * k[b,h,i+j-w]  (0 <= i+j-w < M, else +0.0)
+ *   q (B,M,N), k (B,N,M) -- the reference's orientation: K transposed -- , a (B,M,2w+1).
+ * Replaces window_matmul_fw_cuda (reference cuda/window_matmul_cuda.cu:224-270),
+ * reached from window_matmul_forward (reference window_matmul.cpp:74-78). */
+int wm_window_matmul_forward(const wm_operand *q, const wm_operand *k, const wm_operand *a,
+                             int64_t B, int64_t M, int64_t N, int64_t w, int dtype,
+                             unsigned flags, void *stream);
+
+/* grad_q[b,i,h] = sum_j grad_a[b,i,j] * k[b,h,i+j-w]           (B,M,N)
+ * grad_k[b,h,c] = sum_r q[b,r,h] * grad_a[b,r,c-r+w]            (B,N,M), no atomics
+ *   Either gradient may be skipped by passing NULL for its operand.
+ * Replaces window_matmul_bw_cuda (reference cuda/window_matmul_cuda.cu:272-319),
+ * reached from window_matmul_backward (reference window_matmul.cpp:80-85). */
+int wm_window_matmul_backward(const wm_operand *q, const wm_operand *k, const wm_operand *grad_a,
+                              const wm_operand *grad_q, const wm_operand *grad_k, int64_t B,
+                              int64_t M, int64_t N, int64_t w, int dtype, unsigned flags,
+                              void *stream);
+
+/* o[b,i,h] = sum_{j valid} a[b,i,j] * v[b,i+j-w,h]
+ *   a (B,M,2w+1), v (B,M,N), o (B,M,N).
+ * Replaces unwindow_matmul_fw_cuda (reference cuda/window_matmul_cuda.cu:321-358),
+ * reached from unwindow_matmul_forward (reference window_matmul.cpp:87-91). */
+int wm_unwindow_matmul_forward(const wm_operand *a, const wm_operand *v, const wm_operand *o,
+                               int64_t B, int64_t M, int64_t N, int64_t w, int dtype,
+                               unsigned flags, void *stream);
+
+/* grad_a[b,i,j] = sum_h v[b,i+j-w,h] * grad_o[b,i,h]  (+0.0 where invalid)   (B,M,2w+1)
+ * grad_v[b,c,h] = sum_r a[b,r,c-r+w] * grad_o[b,r,h]                          (B,M,N), no atomics
+ *   Either gradient may be skipped by passing NULL for its operand.
+ * Replaces unwindow_matmul_bw_cuda (reference cuda/window_matmul_cuda.cu:360-416),
+ * reached from unwindow_matmul_backward (reference window_matmul.cpp:93-98). */
+int wm_unwindow_matmul_backward(const wm_operand *a, const wm_operand *v, const wm_operand *grad_o,
+                                const wm_operand *grad_a, const wm_operand *grad_v, int64_t B,
+                                int64_t M, int64_t N, int64_t w, int dtype, unsigned flags,
+                                void *stream);
+
+/* Name of the kernel family the library would pick for one banded product, for
+ * logs and profiles: op is 1 (band-out: window forward, grad_a), 2 (band-in:
+ * unwindow forward, grad_q) or 3 (transposed band-in: grad_k, grad_v);
+ * fast_layout is non-zero when all operands have unit column stride and 16-byte
+ * aligned rows.  Returns a static string.  No counterpart in the reference. */
+const char *wm_kernel_choice(int op, int64_t B, int64_t M, int64_t N, int64_t w, int dtype,
+                             int fast_layout, unsigned flags);
+
+/* Human-readable name of a wm_status code (static string). */
+const char *wm_status_string(int status);
+
+/* WM_ABI_VERSION the library was built with. */
+int wm_abi_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* WINDOW_MATMUL_HIP_H */

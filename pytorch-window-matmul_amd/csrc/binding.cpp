@@ -1,0 +1,185 @@
+// Python module `window_matmul_kernel` for PyTorch-ROCm: the same four functions the
+// reference's native module exports (reference csrc/window_matmul/window_matmul.cpp:100-106),
+// implemented as a thin layer over the C ABI in include/window_matmul_hip.h.
+//
+// What this layer does, and nothing more: argument checks with the reference's error
+// texts (reference cuda/utils.cuh:3-4, cuda/window_matmul_cuda.cu:226-232, 323-329),
+// layout normalisation, output allocation with the input's dtype and device, device
+// guard, current-stream lookup, and the call into libwindow_matmul_hip.so.
+//
+// There is deliberately no CPU implementation behind this module: tensors that do not
+// live on the GPU raise, as the reference does for GPU tensors in a CPU-only build
+// (reference window_matmul.cpp:15).
+#include <torch/extension.h>
+
+#include <ATen/hip/impl/HIPGuardImplMasqueradingAsCUDA.h>
+#include <ATen/hip/impl/HIPStreamMasqueradingAsCUDA.h>
+
+#include <tuple>
+
+#include "../../include/window_matmul_hip.h"
+
+namespace {
+
+void check_gpu(const torch::Tensor &t, const char *name) {
+  TORCH_CHECK(t.device().is_cuda(), name,
+              " must be CUDA tensor (window_matmul_kernel is built for MI355X only and has no CPU path)");
+}
+
+int abi_dtype(const torch::Tensor &t, const char *op) {
+  switch (t.scalar_type()) {
+    case at::kFloat: return WM_DTYPE_F32;
+    case at::kHalf: return WM_DTYPE_F16;
+    case at::kBFloat16: return WM_DTYPE_BF16;
+    case at::kDouble: return WM_DTYPE_F64;
+    default: TORCH_CHECK(false, "\"", op, "\" not implemented for '", c10::toString(t.scalar_type()), "'");
+  }
+  return -1;
+}
+
+// Unit column stride and 16-byte aligned rows/batches, else a contiguous copy.
+torch::Tensor vector_friendly(const torch::Tensor &t) {
+  const int64_t es = t.element_size();
+  const bool ok = t.stride(2) == 1 && (t.stride(1) * es) % 16 == 0 && (t.stride(0) * es) % 16 == 0 &&
+                  reinterpret_cast<uintptr_t>(t.data_ptr()) % 16 == 0;
+  if (ok || t.numel() == 0) return t;
+  if (t.is_contiguous()) return t;  // odd N: the strided kernels take it as it is
+  return t.contiguous();
+}
+
+// Band tensors (rows of odd length 2w+1) only need to be contiguous.
+torch::Tensor band_friendly(const torch::Tensor &t) { return t.contiguous(); }
+
+// K comes as (B,N,M).  The kernels want key rows contiguous, which is what a
+// transposed view of a row-major (B,M,N) tensor already is; anything else is
+// copied into that layout once (the reference always copies: cuda:236).
+torch::Tensor key_rows(const torch::Tensor &k) { return vector_friendly(k.transpose(1, 2)); }
+
+wm_operand operand(const torch::Tensor &t) {
+  return wm_operand{t.data_ptr(), t.stride(0), t.stride(1), t.stride(2)};
+}
+
+void raise_on_error(int status, const char *op) {
+  TORCH_CHECK(status == WM_OK, op, ": ", wm_status_string(status), " (status ", status, ")");
+}
+
+void *current_stream(const torch::Tensor &t) {
+  return c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(t.device().index()).stream();
+}
+
+void check_window_inputs(const torch::Tensor &src, const torch::Tensor &other) {
+  check_gpu(src, "A");
+  check_gpu(other, "B");
+  TORCH_CHECK(src.dim() == 3 && other.dim() == 3, "Input mismatch");
+  TORCH_CHECK(src.size(0) == other.size(0), "Input mismatch");
+  TORCH_CHECK(src.size(2) == other.size(1), "Input mismatch");
+  TORCH_CHECK(src.size(1) == other.size(2), "Input mismatch");
+  TORCH_CHECK(src.scalar_type() == other.scalar_type(), "Input mismatch");
+  TORCH_CHECK(src.device() == other.device(), "Input mismatch");
+}
+
+void check_unwindow_inputs(const torch::Tensor &src, const torch::Tensor &other, int64_t w) {
+  check_gpu(src, "A");
+  check_gpu(other, "B");
+  TORCH_CHECK(src.dim() == 3 && other.dim() == 3, "Input mismatch");
+  TORCH_CHECK(src.size(0) == other.size(0), "Input mismatch");
+  TORCH_CHECK(src.size(2) == 2 * w + 1, "Input mismatch");
+  TORCH_CHECK(src.size(1) == other.size(1), "Input mismatch");
+  TORCH_CHECK(src.scalar_type() == other.scalar_type(), "Input mismatch");
+  TORCH_CHECK(src.device() == other.device(), "Input mismatch");
+}
+
+void check_grad(const torch::Tensor &g, const torch::Tensor &like, std::vector<int64_t> sizes) {
+  check_gpu(g, "grad_C");
+  TORCH_CHECK(g.dim() == 3 && g.sizes().vec() == sizes, "Input mismatch");
+  TORCH_CHECK(g.scalar_type() == like.scalar_type() && g.device() == like.device(), "Input mismatch");
+}
+
+// reference: window_matmul_forward -> window_matmul_fw_cuda (window_matmul.cpp:74-78, cuda:224-270)
+torch::Tensor window_matmul_forward(torch::Tensor src, torch::Tensor other, int64_t window_size) {
+  TORCH_CHECK(window_size >= 0, "Input mismatch");
+  check_window_inputs(src, other);
+  const int dtype = abi_dtype(src, "window_matmul_fw_cuda");
+  at::hip::HIPGuardMasqueradingAsCUDA guard(src.device());
+  const int64_t B = src.size(0), M = src.size(1), N = src.size(2);
+  auto q = vector_friendly(src);
+  auto krows = key_rows(other);  // (B,M,N) view or copy
+  auto kt = krows.transpose(1, 2);
+  auto out = torch::empty({B, M, 2 * window_size + 1}, src.options());
+  wm_operand oq = operand(q), ok = operand(kt), oa = operand(out);
+  raise_on_error(wm_window_matmul_forward(&oq, &ok, &oa, B, M, N, window_size, dtype, 0, current_stream(src)),
+                 "window_matmul_forward");
+  return out;
+}
+
+// reference: window_matmul_backward -> window_matmul_bw_cuda (window_matmul.cpp:80-85, cuda:272-319)
+std::tuple<torch::Tensor, torch::Tensor> window_matmul_backward(torch::Tensor src, torch::Tensor other,
+                                                                 int64_t window_size, torch::Tensor grad_output) {
+  TORCH_CHECK(window_size >= 0, "Input mismatch");
+  check_window_inputs(src, other);
+  const int64_t B = src.size(0), M = src.size(1), N = src.size(2);
+  check_grad(grad_output, src, {B, M, 2 * window_size + 1});
+  const int dtype = abi_dtype(src, "window_matmul_bw_cuda");
+  at::hip::HIPGuardMasqueradingAsCUDA guard(src.device());
+  auto q = vector_friendly(src);
+  auto kt = key_rows(other).transpose(1, 2);
+  auto ga = band_friendly(grad_output);
+  auto grad_q = torch::empty({B, M, N}, src.options());
+  // grad_k is produced row-major per key row and handed back in the (B,N,M)
+  // orientation of `other` as a transposed view, like the reference (cuda:318).
+  auto grad_k = torch::empty({B, M, N}, src.options()).transpose(1, 2);
+  wm_operand oq = operand(q), ok = operand(kt), oga = operand(ga), ogq = operand(grad_q), ogk = operand(grad_k);
+  raise_on_error(wm_window_matmul_backward(&oq, &ok, &oga, &ogq, &ogk, B, M, N, window_size, dtype, 0,
+                                           current_stream(src)),
+                 "window_matmul_backward");
+  return std::make_tuple(grad_q, grad_k);
+}
+
+// reference: unwindow_matmul_forward -> unwindow_matmul_fw_cuda (window_matmul.cpp:87-91, cuda:321-358)
+torch::Tensor unwindow_matmul_forward(torch::Tensor src, torch::Tensor other, int64_t window_size) {
+  TORCH_CHECK(window_size >= 0, "Input mismatch");
+  check_unwindow_inputs(src, other, window_size);
+  const int dtype = abi_dtype(src, "unwindow_matmul_fw_cuda");
+  at::hip::HIPGuardMasqueradingAsCUDA guard(src.device());
+  const int64_t B = other.size(0), M = other.size(1), N = other.size(2);
+  auto a = band_friendly(src);
+  auto v = vector_friendly(other);
+  auto out = torch::empty({B, M, N}, src.options());
+  wm_operand oa = operand(a), ov = operand(v), oo = operand(out);
+  raise_on_error(wm_unwindow_matmul_forward(&oa, &ov, &oo, B, M, N, window_size, dtype, 0, current_stream(src)),
+                 "unwindow_matmul_forward");
+  return out;
+}
+
+// reference: unwindow_matmul_backward -> unwindow_matmul_bw_cuda (window_matmul.cpp:93-98, cuda:360-416)
+std::tuple<torch::Tensor, torch::Tensor> unwindow_matmul_backward(torch::Tensor src, torch::Tensor other,
+                                                                   int64_t window_size,
+                                                                   torch::Tensor grad_output) {
+  TORCH_CHECK(window_size >= 0, "Input mismatch");
+  check_unwindow_inputs(src, other, window_size);
+  const int64_t B = other.size(0), M = other.size(1), N = other.size(2);
+  check_grad(grad_output, src, {B, M, N});
+  const int dtype = abi_dtype(src, "unwindow_matmul_bw_cuda");
+  at::hip::HIPGuardMasqueradingAsCUDA guard(src.device());
+  auto a = band_friendly(src);
+  auto v = vector_friendly(other);
+  auto go = vector_friendly(grad_output);
+  auto grad_a = torch::empty({B, M, 2 * window_size + 1}, src.options());
+  auto grad_v = torch::empty({B, M, N}, src.options());
+  wm_operand oa = operand(a), ov = operand(v), ogo = operand(go), oga = operand(grad_a), ogv = operand(grad_v);
+  raise_on_error(wm_unwindow_matmul_backward(&oa, &ov, &ogo, &oga, &ogv, B, M, N, window_size, dtype, 0,
+                                             current_stream(src)),
+                 "unwindow_matmul_backward");
+  return std::make_tuple(grad_a, grad_v);
+}
+
+}  // namespace
+
+PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
+  m.doc() = "MI355X banded matmul kernels behind the window_matmul package";
+  m.def("window_matmul_forward", &window_matmul_forward, "WindowMatmul forward");
+  m.def("window_matmul_backward", &window_matmul_backward, "WindowMatmul backward");
+  m.def("unwindow_matmul_forward", &unwindow_matmul_forward, "UnwindowMatmul forward");
+  m.def("unwindow_matmul_backward", &unwindow_matmul_backward, "UnwindowMatmul backward");
+  m.def("abi_version", []() { return wm_abi_version(); }, "ABI version of libwindow_matmul_hip.so");
+}

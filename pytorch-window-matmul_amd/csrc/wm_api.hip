@@ -1,0 +1,131 @@
+// extern "C" entry points of libwindow_matmul_hip.so: argument validation and
+// the mapping of the four ops onto the three banded primitives.
+#include "wm_common.hpp"
+
+namespace wm {
+namespace {
+
+int check_common(int64_t B, int64_t M, int64_t N, int64_t w, int dtype, unsigned flags) {
+  if (dtype < WM_DTYPE_F32 || dtype > WM_DTYPE_F64) return WM_ERR_BAD_DTYPE;
+  if (flags & ~WM_FLAG_FORCE_STRIDED) return WM_ERR_BAD_FLAGS;
+  const int64_t lim = 0x7fffffff;
+  if (B < 0 || M < 0 || N < 0 || w < 0) return WM_ERR_BAD_SHAPE;
+  if (B > lim || M > lim || N > lim || w > (lim - 1) / 2) return WM_ERR_BAD_SHAPE;
+  return WM_OK;
+}
+
+bool missing(const wm_operand *op) { return op == nullptr || op->data == nullptr; }
+
+int to_status(hipError_t err) {
+  if (err == hipSuccess) return WM_OK;
+  if (err == hipErrorNoBinaryForGpu || err == hipErrorInvalidDeviceFunction || err == hipErrorSharedObjectInitFailed)
+    return WM_ERR_NO_DEVICE_CODE;
+  return WM_ERR_LAUNCH_FAILED;
+}
+
+typedef bool (*mfma_fn)(const Problem &, const View &, const View &, const View &, hipError_t *);
+typedef hipError_t (*strided_fn)(const Problem &, const View &, const View &, const View &);
+
+int run_primitive(mfma_fn fast, strided_fn slow, const Problem &p, const View &a, const View &y, const View &c) {
+  hipError_t err = hipSuccess;
+  if (!(p.flags & WM_FLAG_FORCE_STRIDED) && fast(p, a, y, c, &err)) return to_status(err);
+  return to_status(slow(p, a, y, c));
+}
+
+int p1(const Problem &p, const View &x, const View &y, const View &c) {
+  return run_primitive(try_launch_mfma_p1, launch_strided_p1, p, x, y, c);
+}
+int p2(const Problem &p, const View &a, const View &y, const View &c) {
+  return run_primitive(try_launch_mfma_p2, launch_strided_p2, p, a, y, c);
+}
+int p3(const Problem &p, const View &a, const View &y, const View &c) {
+  return run_primitive(try_launch_mfma_p3, launch_strided_p3, p, a, y, c);
+}
+
+}  // namespace
+}  // namespace wm
+
+using namespace wm;
+
+extern "C" {
+
+int wm_window_matmul_forward(const wm_operand *q, const wm_operand *k, const wm_operand *a, int64_t B,
+                             int64_t M, int64_t N, int64_t w, int dtype, unsigned flags, void *stream) {
+  if (int st = check_common(B, M, N, w, dtype, flags)) return st;
+  if (B == 0 || M == 0) return WM_OK;  // nothing to write
+  if (missing(a) || (N > 0 && (missing(q) || missing(k)))) return WM_ERR_NULL_POINTER;
+  const Problem p{B, M, N, w, dtype, flags, (hipStream_t)stream};
+  const wm_operand none{a->data, 0, 0, 0};  // N == 0: operands are never dereferenced
+  // K arrives as (B,N,M); the primitives read it as rows c, columns h.
+  return p1(p, make_view(N > 0 ? q : &none), transposed(make_view(N > 0 ? k : &none)), make_view(a));
+}
+
+int wm_window_matmul_backward(const wm_operand *q, const wm_operand *k, const wm_operand *grad_a,
+                              const wm_operand *grad_q, const wm_operand *grad_k, int64_t B, int64_t M,
+                              int64_t N, int64_t w, int dtype, unsigned flags, void *stream) {
+  if (int st = check_common(B, M, N, w, dtype, flags)) return st;
+  if (B == 0 || M == 0 || N == 0) return WM_OK;
+  if (missing(q) || missing(k) || missing(grad_a)) return WM_ERR_NULL_POINTER;
+  if ((grad_q && !grad_q->data) || (grad_k && !grad_k->data)) return WM_ERR_NULL_POINTER;
+  const Problem p{B, M, N, w, dtype, flags, (hipStream_t)stream};
+  if (grad_q)
+    if (int st = p2(p, make_view(grad_a), transposed(make_view(k)), make_view(grad_q))) return st;
+  if (grad_k)
+    if (int st = p3(p, make_view(grad_a), make_view(q), transposed(make_view(grad_k)))) return st;
+  return WM_OK;
+}
+
+int wm_unwindow_matmul_forward(const wm_operand *a, const wm_operand *v, const wm_operand *o, int64_t B,
+                               int64_t M, int64_t N, int64_t w, int dtype, unsigned flags, void *stream) {
+  if (int st = check_common(B, M, N, w, dtype, flags)) return st;
+  if (B == 0 || M == 0 || N == 0) return WM_OK;
+  if (missing(a) || missing(v) || missing(o)) return WM_ERR_NULL_POINTER;
+  const Problem p{B, M, N, w, dtype, flags, (hipStream_t)stream};
+  return p2(p, make_view(a), make_view(v), make_view(o));
+}
+
+int wm_unwindow_matmul_backward(const wm_operand *a, const wm_operand *v, const wm_operand *grad_o,
+                                const wm_operand *grad_a, const wm_operand *grad_v, int64_t B, int64_t M,
+                                int64_t N, int64_t w, int dtype, unsigned flags, void *stream) {
+  if (int st = check_common(B, M, N, w, dtype, flags)) return st;
+  if (B == 0 || M == 0) return WM_OK;
+  if ((grad_a && !grad_a->data) || (grad_v && !grad_v->data)) return WM_ERR_NULL_POINTER;
+  if (N > 0 && (missing(a) || missing(v) || missing(grad_o))) return WM_ERR_NULL_POINTER;
+  const Problem p{B, M, N, w, dtype, flags, (hipStream_t)stream};
+  if (grad_a) {
+    const wm_operand none{grad_a->data, 0, 0, 0};  // N == 0: grad_a is all +0.0
+    if (int st = p1(p, make_view(N > 0 ? grad_o : &none), make_view(N > 0 ? v : &none), make_view(grad_a)))
+      return st;
+  }
+  if (grad_v && N > 0)
+    if (int st = p3(p, make_view(a), make_view(grad_o), make_view(grad_v))) return st;
+  return WM_OK;
+}
+
+const char *wm_kernel_choice(int op, int64_t B, int64_t M, int64_t N, int64_t w, int dtype, int fast,
+                             unsigned flags) {
+  if (op < 1 || op > 3) return "invalid";
+  if (!(flags & WM_FLAG_FORCE_STRIDED) && fast && mfma_supports(op, B, M, N, w, dtype)) {
+    static const char *names[] = {"mfma_p1", "mfma_p2", "mfma_p3"};
+    return names[op - 1];
+  }
+  static const char *names[] = {"strided_p1", "strided_p2", "strided_p3"};
+  return names[op - 1];
+}
+
+const char *wm_status_string(int status) {
+  switch (status) {
+    case WM_OK: return "ok";
+    case WM_ERR_NULL_POINTER: return "null operand or data pointer";
+    case WM_ERR_BAD_SHAPE: return "negative or oversized extent";
+    case WM_ERR_BAD_DTYPE: return "unknown dtype";
+    case WM_ERR_BAD_FLAGS: return "unknown flag bit";
+    case WM_ERR_LAUNCH_FAILED: return "kernel launch failed";
+    case WM_ERR_NO_DEVICE_CODE: return "no device code for this GPU (library is built for gfx950)";
+    default: return "unknown status";
+  }
+}
+
+int wm_abi_version(void) { return WM_ABI_VERSION; }
+
+}  // extern "C"

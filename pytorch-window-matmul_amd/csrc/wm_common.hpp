@@ -1,0 +1,72 @@
+// Shared declarations of the gfx950 banded-matmul kernels.
+//
+// The six products of the path (window forward, grad_q, grad_k, unwindow
+// forward, grad_a, grad_v) are three primitives over row-major views:
+//   P1 band-out            C[b,i,j] = sum_h X[b,i,h] * Y[b,i+j-w,h]      (+0 out of range)
+//   P2 band-in             C[b,i,h] = sum_j A[b,i,j] * Y[b,i+j-w,h]
+//   P3 transposed band-in  C[b,c,h] = sum_r A[b,r,c-r+w] * Y[b,r,h]
+// with X, Y, C(P2,P3) of logical shape (B,M,N) and the band of shape (B,M,2w+1).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <hip/hip_bf16.h>
+#include <hip/hip_fp16.h>
+#include <stdint.h>
+
+#include "../../include/window_matmul_hip.h"
+
+namespace wm {
+
+// Rank-3 view handed to kernels: element strides, 64-bit.
+struct View {
+  void *data;
+  int64_t sb, sr, sc;
+};
+
+inline View make_view(const wm_operand *op) { return View{op->data, op->stride_b, op->stride_r, op->stride_c}; }
+// Same storage seen with rows and columns swapped: (B,N,M) <-> (B,M,N).
+inline View transposed(const View &v) { return View{v.data, v.sb, v.sc, v.sr}; }
+
+struct Problem {
+  int64_t B, M, N, w;
+  int dtype;
+  unsigned flags;
+  hipStream_t stream;
+};
+
+// Launchers return hipSuccess or the launch error.  The strided family accepts
+// any dtype and layout; the MFMA family reports whether it took the problem.
+hipError_t launch_strided_p1(const Problem &p, const View &x, const View &y, const View &c);
+hipError_t launch_strided_p2(const Problem &p, const View &a, const View &y, const View &c);
+hipError_t launch_strided_p3(const Problem &p, const View &a, const View &y, const View &c);
+
+// Returns true and sets *err when the MFMA family handles the problem.
+bool try_launch_mfma_p1(const Problem &p, const View &x, const View &y, const View &c, hipError_t *err);
+bool try_launch_mfma_p2(const Problem &p, const View &a, const View &y, const View &c, hipError_t *err);
+bool try_launch_mfma_p3(const Problem &p, const View &a, const View &y, const View &c, hipError_t *err);
+// Pure predicate behind the three functions above (shape/dtype only).
+bool mfma_supports(int op, int64_t B, int64_t M, int64_t N, int64_t w, int dtype);
+
+inline size_t dtype_size(int dtype) {
+  switch (dtype) {
+    case WM_DTYPE_F32: return 4;
+    case WM_DTYPE_F16: return 2;
+    case WM_DTYPE_BF16: return 2;
+    case WM_DTYPE_F64: return 8;
+    default: return 0;
+  }
+}
+
+// Unit column stride, every row start 16-byte aligned: what the vector paths need.
+inline bool fast_layout(const View &v, int dtype) {
+  const int64_t es = (int64_t)dtype_size(dtype);
+  if (v.sc != 1) return false;
+  if (((uintptr_t)v.data) % 16 != 0) return false;
+  return (v.sr * es) % 16 == 0 && (v.sb * es) % 16 == 0;
+}
+
+// Band operands are only required to be contiguous per batch (rows of odd
+// length 2w+1 are never 16-byte aligned); the kernels realign in LDS.
+inline bool band_layout(const View &v, int64_t W) { return v.sc == 1 && v.sr == W; }
+
+}  // namespace wm

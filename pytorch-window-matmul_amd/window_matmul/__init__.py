@@ -1,0 +1,14 @@
+"""Banded ("windowed") batched matmuls for local attention on MI355X.
+
+Drop-in for the ``window_matmul`` package of webis-de/pytorch-window-matmul
+(reference window_matmul/__init__.py:1-4): same two public functions, same
+autograd behaviour, with gfx950 HIP kernels underneath.
+"""
+from .window_matmul import (
+    UnwindowMatmulFunc,
+    WindowMatmulFunc,
+    unwindow_matmul,
+    window_matmul,
+)
+
+__all__ = ["window_matmul", "unwindow_matmul"]

@@ -1,0 +1,103 @@
+"""ctypes view of libwindow_matmul_hip.so used by the tests (mirrors include/window_matmul_hip.h)."""
+import ctypes
+import os
+import re
+
+import torch
+
+REPO = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+LIB_PATH = os.path.join(REPO, "pytorch-window-matmul_amd", "libwindow_matmul_hip.so")
+HEADER = os.path.join(REPO, "include", "window_matmul_hip.h")
+
+DTYPES = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2, torch.float64: 3}
+FORCE_STRIDED = 0x1
+
+
+class Operand(ctypes.Structure):
+    _fields_ = [
+        ("data", ctypes.c_void_p),
+        ("stride_b", ctypes.c_int64),
+        ("stride_r", ctypes.c_int64),
+        ("stride_c", ctypes.c_int64),
+    ]
+
+
+def declared_symbols():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(wm_[a-z_0-9]+)\s*\(", text)))
+
+
+_LIB = None
+
+
+def lib():
+    global _LIB
+    if _LIB is None:
+        if not os.path.exists(LIB_PATH):
+            raise FileNotFoundError(f"{LIB_PATH} is not built; run python pytorch-window-matmul_amd/build.py")
+        L = ctypes.CDLL(LIB_PATH)
+        P, i64, u32, vp = ctypes.POINTER(Operand), ctypes.c_int64, ctypes.c_uint, ctypes.c_void_p
+        tail = [i64, i64, i64, i64, ctypes.c_int, u32, vp]
+        L.wm_window_matmul_forward.argtypes = [P, P, P] + tail
+        L.wm_unwindow_matmul_forward.argtypes = [P, P, P] + tail
+        L.wm_window_matmul_backward.argtypes = [P, P, P, P, P] + tail
+        L.wm_unwindow_matmul_backward.argtypes = [P, P, P, P, P] + tail
+        L.wm_status_string.restype = ctypes.c_char_p
+        L.wm_status_string.argtypes = [ctypes.c_int]
+        L.wm_kernel_choice.restype = ctypes.c_char_p
+        L.wm_kernel_choice.argtypes = [ctypes.c_int, i64, i64, i64, i64, ctypes.c_int, ctypes.c_int, u32]
+        _LIB = L
+    return _LIB
+
+
+def op(t):
+    """Operand for a rank-3 tensor (None -> NULL pointer)."""
+    if t is None:
+        return None
+    assert t.dim() == 3
+    return ctypes.byref(Operand(t.data_ptr(), t.stride(0), t.stride(1), t.stride(2)))
+
+
+def _stream():
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _check(status, what):
+    if status != 0:
+        raise RuntimeError(f"{what}: {lib().wm_status_string(status).decode()} ({status})")
+
+
+def window_forward(q, k, w, flags=0, out=None):
+    """q (B,M,N), k (B,N,M) (any strides) -> a (B,M,2w+1)."""
+    B, M, N = q.shape
+    a = torch.empty(B, M, 2 * w + 1, dtype=q.dtype, device=q.device) if out is None else out
+    _check(lib().wm_window_matmul_forward(op(q), op(k), op(a), B, M, N, w, DTYPES[q.dtype], flags, _stream()),
+           "wm_window_matmul_forward")
+    return a
+
+
+def window_backward(q, k, w, ga, flags=0, want_q=True, want_k=True):
+    B, M, N = q.shape
+    gq = torch.empty(B, M, N, dtype=q.dtype, device=q.device) if want_q else None
+    gk = torch.empty(B, M, N, dtype=q.dtype, device=q.device).transpose(1, 2) if want_k else None
+    _check(lib().wm_window_matmul_backward(op(q), op(k), op(ga), op(gq), op(gk), B, M, N, w, DTYPES[q.dtype], flags,
+                                          _stream()), "wm_window_matmul_backward")
+    return gq, gk
+
+
+def unwindow_forward(a, v, w, flags=0):
+    B, M, N = v.shape
+    o = torch.empty(B, M, N, dtype=v.dtype, device=v.device)
+    _check(lib().wm_unwindow_matmul_forward(op(a), op(v), op(o), B, M, N, w, DTYPES[v.dtype], flags, _stream()),
+           "wm_unwindow_matmul_forward")
+    return o
+
+
+def unwindow_backward(a, v, w, go, flags=0, want_a=True, want_v=True):
+    B, M, N = v.shape
+    ga = torch.empty(B, M, 2 * w + 1, dtype=v.dtype, device=v.device) if want_a else None
+    gv = torch.empty(B, M, N, dtype=v.dtype, device=v.device) if want_v else None
+    _check(lib().wm_unwindow_matmul_backward(op(a), op(v), op(go), op(ga), op(gv), B, M, N, w, DTYPES[v.dtype], flags,
+                                            _stream()), "wm_unwindow_matmul_backward")
+    return ga, gv

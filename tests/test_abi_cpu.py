@@ -1,0 +1,97 @@
+"""Host-side checks that need no GPU: the library loads, exports what the header
+declares, validates arguments before touching the device, and the Python layer
+mirrors the reference's surface and error behaviour."""
+import ctypes
+import inspect
+
+import pytest
+import torch
+
+import abi
+
+
+def test_library_exports_every_declared_symbol():
+    L = abi.lib()
+    names = abi.declared_symbols()
+    assert {"wm_window_matmul_forward", "wm_window_matmul_backward", "wm_unwindow_matmul_forward",
+            "wm_unwindow_matmul_backward", "wm_kernel_choice", "wm_status_string", "wm_abi_version"} <= set(names)
+    for name in names:
+        assert hasattr(L, name), name
+    assert L.wm_abi_version() == 1
+
+
+def test_argument_validation_happens_on_the_host():
+    L = abi.lib()
+    dummy = abi.Operand(ctypes.c_void_p(16), 0, 0, 0)
+    null = abi.Operand(None, 0, 0, 0)
+    P = ctypes.byref
+    # empty problems are a no-op, whatever the pointers
+    assert L.wm_window_matmul_forward(None, None, None, 0, 4, 4, 1, 0, 0, None) == 0
+    assert L.wm_unwindow_matmul_forward(None, None, None, 2, 0, 4, 1, 0, 0, None) == 0
+    assert L.wm_window_matmul_backward(None, None, None, None, None, 2, 4, 0, 1, 0, 0, None) == 0
+    # status codes from include/window_matmul_hip.h
+    assert L.wm_window_matmul_forward(P(dummy), P(dummy), P(null), 1, 4, 4, 1, 0, 0, None) == 1
+    assert L.wm_window_matmul_forward(None, P(dummy), P(dummy), 1, 4, 4, 1, 0, 0, None) == 1
+    assert L.wm_window_matmul_forward(P(dummy), P(dummy), P(dummy), -1, 4, 4, 1, 0, 0, None) == 2
+    assert L.wm_window_matmul_forward(P(dummy), P(dummy), P(dummy), 1, 4, 4, -3, 0, 0, None) == 2
+    assert L.wm_window_matmul_forward(P(dummy), P(dummy), P(dummy), 1, 2**31, 4, 1, 0, 0, None) == 2
+    assert L.wm_window_matmul_forward(P(dummy), P(dummy), P(dummy), 1, 4, 4, 1, 7, 0, None) == 3
+    assert L.wm_unwindow_matmul_backward(P(dummy), P(dummy), P(dummy), P(dummy), P(dummy), 1, 4, 4, 1, 0, 0x80, None) == 4
+    assert L.wm_unwindow_matmul_backward(P(dummy), P(dummy), None, P(dummy), P(dummy), 1, 4, 4, 1, 0, 0, None) == 1
+    assert b"dtype" in L.wm_status_string(3)
+    assert L.wm_status_string(0) == b"ok"
+
+
+def test_kernel_choice_names():
+    L = abi.lib()
+    assert L.wm_kernel_choice(1, 2, 128, 64, 4, 0, 1, abi.FORCE_STRIDED) == b"strided_p1"
+    assert L.wm_kernel_choice(3, 2, 128, 64, 4, 3, 1, 0) == b"strided_p3"  # float64 has no MFMA path
+    assert L.wm_kernel_choice(9, 2, 128, 64, 4, 0, 1, 0) == b"invalid"
+
+
+def test_python_surface_matches_reference():
+    import window_matmul
+    from window_matmul.window_matmul import UnwindowMatmulFunc, WindowMatmulFunc
+
+    assert window_matmul.__all__ == ["window_matmul", "unwindow_matmul"]
+    for fn in (window_matmul.window_matmul, window_matmul.unwindow_matmul):
+        assert list(inspect.signature(fn).parameters) == ["inp", "other", "window_size"]
+    for cls in (WindowMatmulFunc, UnwindowMatmulFunc):
+        assert issubclass(cls, torch.autograd.Function)
+
+    import window_matmul_kernel as native
+
+    for name in ("window_matmul_forward", "window_matmul_backward", "unwindow_matmul_forward",
+                 "unwindow_matmul_backward"):
+        assert callable(getattr(native, name))
+
+
+def test_window_size_zero_paths_are_plain_torch():
+    """w = 0 never reaches the kernels (reference window_matmul.py:33-34, 69-70; tests/test_attention.py:75-87)."""
+    from window_matmul import unwindow_matmul, window_matmul
+
+    q = torch.randn(2, 3, 5, 4)
+    k = torch.randn(2, 3, 5, 4)
+    v = torch.randn(2, 3, 5, 4)
+    att = window_matmul(q, k.transpose(-1, -2), 0)
+    assert att.shape == (2, 3, 5, 1)
+    torch.testing.assert_close(att[..., 0], (q * k).sum(-1))
+    out = unwindow_matmul(att.softmax(-1), v, None)
+    torch.testing.assert_close(out, v)
+
+
+def test_native_module_rejects_cpu_tensors_and_bad_shapes():
+    """Errors surface as RuntimeError with the reference's texts (reference cuda/utils.cuh:3-4)."""
+    import window_matmul_kernel as native
+
+    with pytest.raises(RuntimeError, match="must be CUDA tensor"):
+        native.window_matmul_forward(torch.zeros(1, 4, 3), torch.zeros(1, 3, 4), 1)
+    with pytest.raises(RuntimeError, match="must be CUDA tensor"):
+        native.unwindow_matmul_backward(torch.zeros(1, 4, 3), torch.zeros(1, 4, 3), 1, torch.zeros(1, 4, 3))
+
+
+def test_only_one_hip_runtime_is_mapped():
+    import window_matmul_kernel  # noqa: F401
+
+    paths = {line.split()[-1] for line in open("/proc/self/maps") if "libamdhip64" in line}
+    assert len(paths) == 1, paths

@@ -1,0 +1,171 @@
+"""GPU tests of the drop-in Python API (window_matmul.window_matmul / unwindow_matmul and
+their autograd Functions), in the manner of the reference's own tests: the custom op
+against an independent torch formulation, outputs and input gradients
+(reference tests/test_window_matmul.py:53-84, tests/test_unwindow_matmul.py:40-79,
+tests/test_attention.py:90-140)."""
+import itertools
+import math
+
+import pytest
+import torch
+
+import oracle
+from conftest import seeded
+
+pytestmark = pytest.mark.gpu
+
+DIMS = [(2, 1, 1, 3), (2, 1, 4, 3), (2, 1, 16, 3), (2, 1, 32, 3), (2, 1, 16, 32), (2, 3, 77, 16)]  # (batch, heads, M, N)
+WINDOWS = [0, 1, 4, 16]
+
+
+def head_major(batch, heads, M, N, seed, device, dtype=torch.float32):
+    """randn(batch, M, heads*N) viewed as (batch, heads, M, N): non-contiguous (reference tests/utils.py:38-44)."""
+    t = seeded((batch, M, heads * N), seed, dtype).to(device)
+    return t.view(batch, M, heads, N).transpose(1, 2)
+
+
+def dense_window(q, kt, w):
+    if not w:
+        return (q * kt.transpose(-1, -2)).sum(-1, keepdim=True)
+    lead = q.shape[:-2]
+    S = torch.matmul(q, kt).reshape(-1, q.shape[-2], q.shape[-2])
+    return oracle.dense_to_band(S, w).reshape(*lead, q.shape[-2], 2 * w + 1)
+
+
+def dense_unwindow(a, v, w):
+    if not w:
+        return a * v
+    lead = v.shape[:-2]
+    D = oracle.band_to_dense(a.reshape(-1, a.shape[-2], a.shape[-1]), w).reshape(*lead, v.shape[-2], v.shape[-2])
+    return torch.matmul(D, v)
+
+
+@pytest.mark.parametrize("dim", DIMS)
+@pytest.mark.parametrize("w", WINDOWS)
+def test_window_matmul_forward_and_grads(device, dim, w):
+    from window_matmul import window_matmul
+
+    q0 = head_major(*dim, 1, device)
+    k0 = head_major(*dim, 2, device)
+    res = {}
+    for name, fn in (("dense", dense_window), ("custom", window_matmul)):
+        q = q0.detach().clone().requires_grad_(True)
+        k = k0.detach().clone().requires_grad_(True)
+        att = fn(q, k.transpose(-1, -2), w)
+        # arange-weighted loss gives a known, non-uniform upstream gradient (reference tests/test_window_matmul.py:71)
+        (att * torch.arange(att.numel(), device=device).to(att).view_as(att)).mean().backward()
+        res[name] = (att, q.grad, k.grad)
+    assert res["custom"][0].shape == (*dim[:3], 2 * w + 1)
+    for x, y in zip(res["custom"], res["dense"]):
+        torch.testing.assert_close(x, y, rtol=1e-4, atol=1e-4)
+
+
+@pytest.mark.parametrize("dim", DIMS)
+@pytest.mark.parametrize("w", WINDOWS)
+def test_unwindow_matmul_forward_and_grads(device, dim, w):
+    from window_matmul import unwindow_matmul
+
+    batch, heads, M, N = dim
+    a0 = seeded((batch, heads, M, 2 * w + 1), 3, torch.float32).to(device)
+    v0 = head_major(*dim, 4, device)
+    res = {}
+    for name, fn in (("dense", dense_unwindow), ("custom", unwindow_matmul)):
+        a = a0.detach().clone().requires_grad_(True)
+        v = v0.detach().clone().requires_grad_(True)
+        out = fn(a, v, w)
+        (out * torch.arange(out.numel(), device=device).to(out).view_as(out)).mean().backward()
+        ga = a.grad
+        if w:
+            mask = oracle.band_mask(M, w, device)
+            # the dense formulation propagates no gradient to invalid entries; ours writes +0.0 there
+            assert torch.equal(ga[..., ~mask], torch.zeros_like(ga[..., ~mask]))
+        res[name] = (out, ga, v.grad)
+    for x, y in zip(res["custom"], res["dense"]):
+        torch.testing.assert_close(x, y, rtol=1e-4, atol=1e-4)
+
+
+@pytest.mark.parametrize("dim", DIMS[:5])
+def test_window_size_zero_on_gpu(device, dim):
+    from window_matmul import unwindow_matmul, window_matmul
+
+    q, k, v = (head_major(*dim, s, device) for s in (1, 2, 3))
+    att = window_matmul(q, k.transpose(-1, -2), 0)
+    out = unwindow_matmul(att.softmax(-1), v, 0)
+    assert att.shape[-1] == 1
+    assert torch.allclose(out, v)  # reference tests/test_attention.py:86-87
+
+
+class Layer(torch.nn.Module):
+    """window -> /sqrt(N) -> softmax over the whole band -> unwindow -> linear -> sigmoid
+    (the caller the reference tests, tests/test_attention.py:48-72)."""
+
+    def __init__(self, w, fns, linear):
+        super().__init__()
+        self.w, self.fns, self.linear = w, fns, linear
+
+    def forward(self, q, k, v):
+        win, unwin = self.fns
+        p = torch.softmax(win(q, k.transpose(-1, -2), self.w) / math.sqrt(q.shape[-1]), dim=-1)
+        return torch.sigmoid(self.linear(unwin(p, v, self.w)))
+
+
+@pytest.mark.parametrize("dim", DIMS)
+@pytest.mark.parametrize("w", WINDOWS)
+def test_three_layer_attention_chain(device, dim, w):
+    from window_matmul import unwindow_matmul, window_matmul
+
+    torch.manual_seed(0)
+    linear = torch.nn.Linear(dim[-1], dim[-1]).to(device)
+    res = {}
+    for name, fns in (("dense", (dense_window, dense_unwindow)), ("custom", (window_matmul, unwindow_matmul))):
+        q, k, v = (head_major(*dim, s, device).detach().clone().requires_grad_(True) for s in (1, 2, 3))
+        x = (q, k, v)
+        for _ in range(3):
+            out = Layer(w, fns, linear)(*x)
+            x = (linear(out), linear(out), linear(out))
+        out.mean().backward()
+        res[name] = (out, q.grad, k.grad, v.grad)
+    for x, y in zip(res["custom"], res["dense"]):
+        torch.testing.assert_close(x, y, rtol=1e-4, atol=1e-5)
+
+
+def test_gradcheck_float64(device):
+    from window_matmul import unwindow_matmul, window_matmul
+
+    B, M, N, w = 2, 7, 3, 2
+    q = seeded((B, M, N), 1, torch.float64).to(device).requires_grad_(True)
+    kt = seeded((B, N, M), 2, torch.float64).to(device).requires_grad_(True)
+    v = seeded((B, M, N), 3, torch.float64).to(device).requires_grad_(True)
+    mask = oracle.band_mask(M, w, device)
+    a = (seeded((B, M, 2 * w + 1), 4, torch.float64).to(device) * mask).requires_grad_(True)
+    assert torch.autograd.gradcheck(lambda x, y: window_matmul(x, y, w), (q, kt))
+    # invalid band entries carry no dependence; restrict the check to valid ones
+    assert torch.autograd.gradcheck(lambda x, y: unwindow_matmul(x * mask, y, w), (a, v))
+
+
+def test_autocast_casts_to_float16(device):
+    """Under autocast the Functions run in float16 (reference window_matmul.py:9,45)."""
+    from window_matmul import unwindow_matmul, window_matmul
+
+    B, M, N, w = 2, 40, 16, 4
+    q, k, v = (seeded((B, M, N), s).to(device) for s in (1, 2, 3))
+    with torch.autocast("cuda", dtype=torch.bfloat16):
+        att = window_matmul(q, k.transpose(1, 2), w)
+        out = unwindow_matmul(att.float().softmax(-1), v, w)
+    assert att.dtype == torch.float16 and out.dtype == torch.float16
+    want = oracle.dense_window_matmul(q.half().cpu(), k.half().cpu().transpose(1, 2), w)
+    torch.testing.assert_close(att.cpu().double(), want, rtol=2e-2, atol=2e-2)
+
+
+def test_error_behaviour(device):
+    import window_matmul_kernel as native
+
+    q = torch.zeros(2, 8, 4, device=device)
+    with pytest.raises(RuntimeError, match="Input mismatch"):
+        native.window_matmul_forward(q, torch.zeros(2, 8, 4, device=device), 1)
+    with pytest.raises(RuntimeError, match="Input mismatch"):
+        native.unwindow_matmul_forward(torch.zeros(2, 8, 4, device=device), q, 1)
+    with pytest.raises(RuntimeError, match="must be CUDA tensor"):
+        native.window_matmul_forward(q, torch.zeros(2, 4, 8), 1)
+    with pytest.raises(RuntimeError, match="not implemented for"):
+        native.window_matmul_forward(q.int(), torch.zeros(2, 4, 8, device=device).int(), 1)
