@@ -1,0 +1,235 @@
+#!/usr/bin/env python3
+"""Benchmark of the banded-matmul hot path on one MI355X.
+
+A step is one pass of the chain the reference's callers run (reference
+tests/test_attention.py:48-72) at the Longformer shape the headline metric is quoted on:
+
+    A = window_matmul(q, k^T, w) -> P = softmax(A, -1) -> O = unwindow_matmul(P, v, w)
+    backward with dO ~ N(0,1)  (grad_a, grad_v, softmax backward, grad_q, grad_k)
+
+bf16 storage, float32 accumulation, B=96 M=4096 N=64 w=256, seeded synthetic inputs that
+are resident in HBM before the timed region starts.  The value reported is whole-step
+throughput on the band FLOPs (6 band units per step; the torch softmax adds no FLOPs to
+the count but its time is inside the step).  Next to it:
+
+  roofline      the slowest of the six kernels, timed alone with HIP events on the stream
+                it is launched on, priced against the 8 TB/s HBM peak on its algorithmic
+                bytes (each operand touched once);
+  cpu_baseline  the reference's own scalar CPU path (oracle/_ref, where built) or its C
+                restatement, one thread, on a slice of the batch.
+
+Usage: python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c2|c4] [--no-cpu]
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+REPO = os.path.dirname(os.path.abspath(__file__))
+PKG = os.path.join(REPO, "pytorch-window-matmul_amd")
+for _p in (REPO, PKG):
+    if _p not in sys.path:
+        sys.path.insert(0, _p)
+
+HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
+
+WORKLOADS = {
+    # name: (B, M, N, w, dtype, qk_scale, backward)
+    "c3": dict(B=96, M=4096, N=64, w=256, dtype="bf16", qk_scale=0.125, backward=True,
+               label="B96 M4096 N64 w256 bf16, window->softmax->unwindow, fwd+bwd"),
+    "c2": dict(B=96, M=16384, N=64, w=8, dtype="bf16", qk_scale=1.0, backward=False,
+               label="B96 M16384 N64 w8 bf16, window->softmax->unwindow, fwd"),
+    "c4": dict(B=16, M=32768, N=128, w=512, dtype="fp16", qk_scale=1.0, backward=True,
+               label="B16 M32768 N128 w512 fp16, window->softmax->unwindow, fwd+bwd"),
+}
+
+
+def band_unit_flops(B, M, N, w):
+    valid = M * (2 * w + 1) - w * (w + 1) if w <= M - 1 else M * M
+    return 2.0 * B * N * valid
+
+
+def kernel_bytes(B, M, N, w, es):
+    """Algorithmic HBM bytes of one launch, every operand touched once."""
+    W = 2 * w + 1
+    band, mat = B * M * W * es, B * M * N * es
+    return band + 2 * mat  # P1: X, Y in, band out;  P2 / P3: band, Y in, C out
+
+
+def time_gpu(fn, iters, warmup):
+    import torch
+
+    for _ in range(warmup):
+        fn()
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    start.record()
+    for _ in range(iters):
+        fn()
+    stop.record()
+    stop.synchronize()
+    return start.elapsed_time(stop) / iters  # ms
+
+
+def cpu_baseline(cfg, seconds_budget=20.0):
+    """Times the reference CPU path (or its restatement) on one thread over a batch slice."""
+    import torch
+
+    import oracle
+
+    torch.set_num_threads(1)
+    ref = oracle.reference_module()
+    kind = "reference" if ref is not None else "port"
+    impl = ref if ref is not None else oracle
+    M, N, w = cfg["M"], cfg["N"], cfg["w"]
+    g = torch.Generator().manual_seed(0)
+    rnd = {"bf16": torch.bfloat16, "fp16": torch.float16}[cfg["dtype"]]
+
+    def rounded(*shape, scale=1.0):
+        return (torch.randn(*shape, generator=g) * scale).to(rnd).float()
+
+    slice_b, done, elapsed = 1, 0, 0.0
+    flops = 0.0
+    while elapsed < seconds_budget * 0.5 and done < cfg["B"]:
+        q, k, v, go = (rounded(slice_b, M, N, scale=s) for s in (cfg["qk_scale"], cfg["qk_scale"], 1.0, 1.0))
+        kt = k.transpose(1, 2).contiguous()
+        t0 = time.perf_counter()
+        att = impl.window_matmul_forward(q, kt, w)
+        probs = att.softmax(-1)
+        impl.unwindow_matmul_forward(probs, v, w)
+        units = 2
+        if cfg["backward"]:
+            ga, _ = impl.unwindow_matmul_backward(probs, v, w, go)
+            impl.window_matmul_backward(q, kt, w, ga)
+            units = 6
+        elapsed += time.perf_counter() - t0
+        done += slice_b
+        flops += units * band_unit_flops(slice_b, M, N, w)
+    return {
+        "value": flops / elapsed / 1e12,
+        "unit": "TFLOP/s",
+        "cores": 1,
+        "kind": kind,
+        "sample": f"{done} of {cfg['B']} batch elements at full M, N, w; float32 copies of the rounded inputs; "
+                  f"{elapsed:.1f} s of CPU time (softmax between the ops included, as on the GPU)",
+        "host_cpus": os.cpu_count(),
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="c3", choices=sorted(WORKLOADS))
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on one GPU; --gpus must be 1 (the path shards over the batch "
+                 "dimension with no communication, which one GPU cannot show)")
+
+    import torch
+
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no GPU visible")
+    import wm_ctypes as abi
+    from window_matmul import unwindow_matmul, window_matmul
+
+    cfg = WORKLOADS[args.workload]
+    B, M, N, w = cfg["B"], cfg["M"], cfg["N"], cfg["w"]
+    dtype = {"bf16": torch.bfloat16, "fp16": torch.float16}[cfg["dtype"]]
+    es = 2
+    dev = torch.device("cuda:0")
+    g = torch.Generator().manual_seed(0)
+
+    def synth(scale=1.0):
+        return (torch.randn(B, M, N, generator=g) * scale).to(dtype).to(dev)
+
+    q, k, v, go = synth(cfg["qk_scale"]), synth(cfg["qk_scale"]), synth(), synth()
+    q.requires_grad_(True), k.requires_grad_(True), v.requires_grad_(True)
+
+    def step():
+        att = window_matmul(q, k.transpose(1, 2), w)
+        probs = torch.softmax(att, dim=-1)
+        out = unwindow_matmul(probs, v, w)
+        if cfg["backward"]:
+            q.grad = k.grad = v.grad = None
+            out.backward(go)
+        return out
+
+    units = 6 if cfg["backward"] else 2
+    flops = units * band_unit_flops(B, M, N, w)
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+
+    # per-kernel timing through the C ABI (one launch per call), same tensors, same stream
+    with torch.no_grad():
+        kt = k.detach().transpose(1, 2)
+        att = abi.window_forward(q.detach(), kt, w)
+        probs = torch.softmax(att, dim=-1)
+        ga = torch.randn(B, M, 2 * w + 1, generator=g).to(dtype).to(dev) if cfg["backward"] else None
+        qd, vd = q.detach(), v.detach()
+        launches = {
+            "window_fwd(P1)": lambda: abi.window_forward(qd, kt, w, out=att),
+            "unwindow_fwd(P2)": lambda: abi.unwindow_forward(probs, vd, w),
+        }
+        if cfg["backward"]:
+            launches.update({
+                "grad_a(P1)": lambda: abi.unwindow_backward(probs, vd, w, go, want_v=False),
+                "grad_v(P3)": lambda: abi.unwindow_backward(probs, vd, w, go, want_a=False),
+                "grad_q(P2)": lambda: abi.window_backward(qd, kt, w, ga, want_k=False),
+                "grad_k(P3)": lambda: abi.window_backward(qd, kt, w, ga, want_q=False),
+            })
+        kb = kernel_bytes(B, M, N, w, es)
+        per_kernel = {}
+        for name, fn in launches.items():
+            ms = time_gpu(fn, max(args.steps, 10), 3)
+            per_kernel[name] = {"ms": round(ms, 4), "GBps": round(kb / ms / 1e6, 1),
+                                "TFLOPs": round(band_unit_flops(B, M, N, w) / ms / 1e9, 1)}
+        softmax_ms = time_gpu(lambda: torch.softmax(att, dim=-1), max(args.steps, 10), 3)
+        # device-to-device copy of the band as the achievable-bandwidth yardstick
+        scratch = torch.empty_like(att)
+        copy_ms = time_gpu(lambda: scratch.copy_(att), 20, 3)
+        copy_gbs = 2 * att.numel() * es / copy_ms / 1e6
+    dom = max(per_kernel, key=lambda n: per_kernel[n]["ms"])
+    achieved = per_kernel[dom]["GBps"]
+    result = {
+        "metric": "fwd+bwd TFLOP/s & HBM GB/s, window+unwindow, B96 M4096 N64 w256 bf16" if args.workload == "c3"
+                  else f"band TFLOP/s, window+unwindow, {cfg['label']}",
+        "value": round(flops / ms_per_step / 1e9, 2),
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": cfg["dtype"],
+        "data": "synthetic",
+        "config": {"workload": cfg["label"], "B": B, "M": M, "N": N, "w": w,
+                   "band_gflop_per_step": round(flops / 1e9, 2)},
+        "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None, "kernel": dom,
+                     "algorithmic_bytes_per_launch": kb, "avg_launch_ms": per_kernel[dom]["ms"]},
+        "kernels": per_kernel,
+        "softmax_fwd_ms": round(softmax_ms, 4),
+        "copy_yardstick_GBps": round(copy_gbs, 1),
+        "kernel_sum_GBps": round(len(per_kernel) * kb / sum(v["ms"] for v in per_kernel.values()) / 1e6, 1),
+    }
+    if not args.no_cpu:
+        result["cpu_baseline"] = cpu_baseline(cfg)
+    else:
+        result["cpu_baseline"] = None
+    print(json.dumps(result), flush=True)
+
+
+if __name__ == "__main__":
+    main()

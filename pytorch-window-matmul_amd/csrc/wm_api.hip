@@ -7,7 +7,7 @@ namespace {
 
 int check_common(int64_t B, int64_t M, int64_t N, int64_t w, int dtype, unsigned flags) {
   if (dtype < WM_DTYPE_F32 || dtype > WM_DTYPE_F64) return WM_ERR_BAD_DTYPE;
-  if (flags & ~WM_FLAG_FORCE_STRIDED) return WM_ERR_BAD_FLAGS;
+  if (flags & ~(WM_FLAG_FORCE_STRIDED | WM_FLAG_NO_ALIGNED_BAND)) return WM_ERR_BAD_FLAGS;
   const int64_t lim = 0x7fffffff;
   if (B < 0 || M < 0 || N < 0 || w < 0) return WM_ERR_BAD_SHAPE;
   if (B > lim || M > lim || N > lim || w > (lim - 1) / 2) return WM_ERR_BAD_SHAPE;

@@ -1,9 +1,618 @@
-// MFMA kernel family (placeholder until the tiled kernels land): declines every problem.
+// MFMA kernel family for 16-bit storage (bf16 / f16, float32 accumulate) on gfx950.
+//
+// All three primitives are tiled GEMMs over a "skewed" tile T of the band:
+//     T[r][c] = band[r, c - r + w]   (row r of the sequence, dense column c)
+// For one block of 128 sequence rows (P1, P2) or 128 output rows (P3) a workgroup
+// of four 64-lane waves walks the dense columns (P1, P2) or the band rows (P3) in
+// chunks of 64, double-buffering the chunk operands in LDS, and feeds
+// v_mfma_f32_32x32x16_{bf16,f16}.  Each wave owns 32 rows of the block.
+//
+//   P1  S^T(c, r) = Y[c,:] . X[r,:]      A-operand Y chunk (LDS, k = h contiguous)
+//                                         B-operand X rows (registers, loaded once)
+//       the 32 x 64 result is staged per wave in LDS and leaves as row-contiguous
+//       16-byte stores straight into the band (band entry (r, c-r+w)).
+//   P2  O^T(h, r) = sum_c Y[c,h] T[r][c]  A-operand Y chunk via ds_read_b64_tr_b16
+//                                         B-operand T tile (LDS, k = c contiguous)
+//   P3  C^T(h, c) = sum_r Y[r,h] T[r][c]  both operands via ds_read_b64_tr_b16
+//       (output-stationary over c: no atomics).
+//
+// Band rows have odd length 2w+1, so a band row is never 16-byte aligned as a
+// whole; but element (r, c) sits at flat index  b*sb + r*2w + c + w, hence when
+// w % 4 == 0 every group of 8 dense columns starting at c8 = -(b*sb + w) (mod 8)
+// is one aligned 16-byte chunk in every row.  The ALIGNED instantiation picks
+// its column groups that way; the other instantiation issues the same 16-byte
+// accesses at 2-byte alignment (legal on gfx950, somewhat slower).
+//
+// Masking is done on bits, never by multiplying with zero: invalid entries of an
+// input band are cleared before they reach LDS, and out-of-sequence entries of an
+// output band are stored as +0.0 whatever the operands hold.
 #include "wm_common.hpp"
+#include "wm_types.hpp"
 
 namespace wm {
-bool mfma_supports(int, int64_t, int64_t, int64_t, int64_t, int) { return false; }
-bool try_launch_mfma_p1(const Problem &, const View &, const View &, const View &, hipError_t *) { return false; }
-bool try_launch_mfma_p2(const Problem &, const View &, const View &, const View &, hipError_t *) { return false; }
-bool try_launch_mfma_p3(const Problem &, const View &, const View &, const View &, hipError_t *) { return false; }
+namespace {
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+
+constexpr int kThreads = 256;
+constexpr int TM = 128;  // rows per workgroup (32 per wave)
+constexpr int KC = 64;   // chunk length along the contraction (P2, P3) / dense columns (P1)
+
+struct __attribute__((packed, aligned(2))) Chunk2 {
+  u32x4 v;
+};
+
+template <bool ALIGNED>
+__device__ __forceinline__ u32x4 load_chunk(const uint16_t *p) {
+  if (ALIGNED) return *reinterpret_cast<const u32x4 *>(p);
+  return reinterpret_cast<const Chunk2 *>(p)->v;
+}
+template <bool ALIGNED>
+__device__ __forceinline__ void store_chunk(uint16_t *p, u32x4 v) {
+  if (ALIGNED)
+    *reinterpret_cast<u32x4 *>(p) = v;
+  else
+    reinterpret_cast<Chunk2 *>(p)->v = v;
+}
+
+// Keeps elements e_lo..e_hi (inclusive, in 0..7) of a chunk of eight 16-bit values, clears the rest.
+__device__ __forceinline__ u32x4 keep_range(u32x4 v, int e_lo, int e_hi) {
+  u32x4 r;
+#pragma unroll
+  for (int d = 0; d < 4; ++d) {
+    const uint32_t lo = (2 * d >= e_lo && 2 * d <= e_hi) ? 0x0000ffffu : 0u;
+    const uint32_t hi = (2 * d + 1 >= e_lo && 2 * d + 1 <= e_hi) ? 0xffff0000u : 0u;
+    r[d] = v[d] & (lo | hi);
+  }
+  return r;
+}
+
+// Loads the 8 band elements of one skewed-tile chunk; only [e_lo, e_hi] is valid.
+// A chunk with no valid element is never touched.  Partial chunks are read whole
+// when that cannot leave the allocation (aligned chunks never straddle a page),
+// element by element otherwise.
+template <bool ALIGNED>
+__device__ __forceinline__ u32x4 load_band_chunk(const uint16_t *p, int e_lo, int e_hi) {
+  u32x4 z = {0u, 0u, 0u, 0u};
+  if (e_hi < 0 || e_lo > 7 || e_lo > e_hi) return z;
+  if (e_lo <= 0 && e_hi >= 7) return load_chunk<ALIGNED>(p);
+  if (ALIGNED) return keep_range(load_chunk<true>(p), e_lo, e_hi);
+  const int lo = e_lo < 0 ? 0 : e_lo, hi = e_hi > 7 ? 7 : e_hi;
+  uint32_t h[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) h[e] = (e >= lo && e <= hi) ? (uint32_t)p[e] : 0u;
+  u32x4 r = {h[0] | (h[1] << 16), h[2] | (h[3] << 16), h[4] | (h[5] << 16), h[6] | (h[7] << 16)};
+  return r;
+}
+
+template <typename T>
+struct Mma;
+template <>
+struct Mma<bf16_t> {
+  static __device__ __forceinline__ f32x16 run(u32x4 a, u32x4 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c,
+                                                   0, 0, 0);
+  }
+  static __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
+    return float_to_bf16_bits(lo) | (float_to_bf16_bits(hi) << 16);
+  }
+};
+template <>
+struct Mma<f16_t> {
+  static __device__ __forceinline__ f32x16 run(u32x4 a, u32x4 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0,
+                                                  0, 0);
+  }
+  static __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
+    const uint16_t l = __builtin_bit_cast(uint16_t, (_Float16)lo), h = __builtin_bit_cast(uint16_t, (_Float16)hi);
+    return (uint32_t)l | ((uint32_t)h << 16);
+  }
+};
+
+// Operand fetch for a matrix stored in LDS as Mat[k][x] (x contiguous) when the MFMA
+// wants, per lane, x = lane % 32 and eight consecutive k starting at 8 * (lane / 32).
+// ds_read_b64_tr_b16 works on 16-lane groups: lane s of a group supplies the address of
+// 4 consecutive x in row s/4 and receives, for x = its own position in the group, the
+// 4 values of rows 0..3.  Two such reads cover the 8 k's.
+__device__ __forceinline__ u32x4 lds_read_transposed(const uint16_t *mat, int stride, int k0, int x0, int lane) {
+  const int s = lane & 15, grp = lane >> 4;
+  const int xb = x0 + 16 * (grp & 1) + 4 * (s & 3);
+  const int kb = k0 + 8 * (grp >> 1) + (s >> 2);
+  typedef s16x4 __attribute__((address_space(3))) * lds_ptr;
+  const uint16_t *p0 = mat + kb * stride + xb;
+  const uint16_t *p1 = p0 + 4 * stride;
+  const s16x4 a = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(p0));
+  const s16x4 b = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(p1));
+  const u32x2 ua = __builtin_bit_cast(u32x2, a), ub = __builtin_bit_cast(u32x2, b);
+  u32x4 r = {ua[0], ua[1], ub[0], ub[1]};
+  return r;
+}
+
+__device__ __forceinline__ void wave_sync_lds() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+// Workgroup -> (batch, block).  Workgroups are dealt round-robin to the 8 XCDs, each with
+// its own L2; all blocks of one batch element are given to one XCD so that neighbouring
+// blocks find the rows they share (the +-w halo) in that L2.
+__device__ __forceinline__ bool decode_block(int nblk, int B, int *b, int *blk) {
+  const int id = blockIdx.x, xcd = id & 7, slot = id >> 3;
+  *b = (slot / nblk) * 8 + xcd;
+  *blk = slot % nblk;
+  return *b < B;
+}
+
+// Row stride (elements) of matrices read with lds_read_transposed: the byte stride must be
+// 32 or 96 (mod 128) so that the 4 rows touched by a 16-lane group fall into distinct banks.
+constexpr int lds_stride_tr(int n_padded) { return n_padded + 16; }
+
+// ------------------------------------------------------------------------------------------
+// P2: C[b,i,h] = sum_c T[i][c] * Y[b,c,h]
+// ------------------------------------------------------------------------------------------
+template <typename T, int NT, bool ALIGNED>
+__global__ __launch_bounds__(kThreads, 2) void mfma_p2_kernel(const uint16_t *__restrict__ A,
+                                                              const uint16_t *__restrict__ Y,
+                                                              uint16_t *__restrict__ C, int B, int M, int N, int w,
+                                                              int nblk, int64_t asb, int64_t ysb, int64_t ysr,
+                                                              int64_t csb, int64_t csr) {
+  constexpr int NP = 32 * NT;
+  constexpr int ST = KC + 8;                         // T tile row stride: 144 B, conflict-free b128 reads
+  constexpr int SY = lds_stride_tr(NP);
+  __shared__ __attribute__((aligned(16))) uint16_t t_lds[2][TM * ST];
+  __shared__ __attribute__((aligned(16))) uint16_t y_lds[2][KC * SY];
+
+  int b, blk;
+  if (!decode_block(nblk, B, &b, &blk)) return;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int W = 2 * w + 1;
+  const int i0 = blk * TM;
+  const int rows = min(TM, M - i0);
+  const int c_lo = max(i0 - w, 0), c_hi = min(i0 + rows - 1 + w, M - 1);
+  const uint16_t *Ab = A + (int64_t)b * asb;
+  const uint16_t *Yb = Y + (int64_t)b * ysb;
+  const int c_start = ALIGNED ? c_lo - (int)(((int64_t)c_lo + (int64_t)b * asb + w) & 7) : c_lo;
+  const int nk = (c_hi - c_start + KC) / KC;
+
+  // per-thread chunk coordinates (loop invariant)
+  int t_lo[4], t_hi[4];        // valid dense-column range of the chunk's row
+  const uint16_t *t_ptr[4];    // address of dense column 0 of the row (may be virtual)
+#pragma unroll
+  for (int s = 0; s < 4; ++s) {
+    const int q = tid + kThreads * s, r = q >> 3;
+    const int i = i0 + r;
+    t_lo[s] = max(i - w, 0);
+    t_hi[s] = i < M ? min(i + w, M - 1) : -1;
+    t_ptr[s] = Ab + (int64_t)i * W + (w - i);
+  }
+  const int ychunks = KC * (N >> 3), ncg = N >> 3;
+  int y_r[NT], y_h[NT];
+#pragma unroll
+  for (int s = 0; s < NT; ++s) {
+    const int q = tid + kThreads * s;
+    y_r[s] = q < ychunks ? q / ncg : -1;
+    y_h[s] = q < ychunks ? (q % ncg) * 8 : 0;
+  }
+
+  u32x4 t_reg[4], y_reg[NT];
+  auto fetch = [&](int k) {
+    const int cb = c_start + k * KC;
+#pragma unroll
+    for (int s = 0; s < 4; ++s) {
+      const int g = (tid + kThreads * s) & 7;
+      const int c8 = cb + 8 * g;
+      t_reg[s] = load_band_chunk<ALIGNED>(t_ptr[s] + c8, t_lo[s] - c8, t_hi[s] - c8);
+    }
+#pragma unroll
+    for (int s = 0; s < NT; ++s) {
+      const int c = cb + y_r[s];
+      u32x4 z = {0u, 0u, 0u, 0u};
+      y_reg[s] = (y_r[s] >= 0 && c >= 0 && c < M) ? *reinterpret_cast<const u32x4 *>(Yb + (int64_t)c * ysr + y_h[s]) : z;
+    }
+  };
+  auto stash = [&](int buf) {
+#pragma unroll
+    for (int s = 0; s < 4; ++s) {
+      const int q = tid + kThreads * s;
+      *reinterpret_cast<u32x4 *>(&t_lds[buf][(q >> 3) * ST + (q & 7) * 8]) = t_reg[s];
+    }
+#pragma unroll
+    for (int s = 0; s < NT; ++s)
+      if (y_r[s] >= 0) *reinterpret_cast<u32x4 *>(&y_lds[buf][y_r[s] * SY + y_h[s]]) = y_reg[s];
+  };
+
+  f32x16 acc[NT];
+#pragma unroll
+  for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) acc[nt][v] = 0.f;
+
+  fetch(0);
+  stash(0);
+  __syncthreads();
+  for (int k = 0; k < nk; ++k) {
+    const int buf = k & 1;
+    if (k + 1 < nk) fetch(k + 1);
+    const uint16_t *tl = &t_lds[buf][(wave * 32 + (lane & 31)) * ST + 8 * (lane >> 5)];
+#pragma unroll
+    for (int ks = 0; ks < KC / 16; ++ks) {
+      const u32x4 bop = *reinterpret_cast<const u32x4 *>(tl + ks * 16);
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt) {
+        const u32x4 aop = lds_read_transposed(y_lds[buf], SY, ks * 16, 32 * nt, lane);
+        acc[nt] = Mma<T>::run(aop, bop, acc[nt]);
+      }
+    }
+    if (k + 1 < nk) stash(buf ^ 1);
+    __syncthreads();
+  }
+
+  // acc[nt][v]: h = 32 nt + 8 (v / 4) + 4 (lane / 32) + v % 4, row = wave * 32 + lane % 32
+  const int i = i0 + wave * 32 + (lane & 31);
+  if (i < M) {
+    uint16_t *crow = C + (int64_t)b * csb + (int64_t)i * csr;
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+      for (int q4 = 0; q4 < 4; ++q4) {
+        const int h = 32 * nt + 8 * q4 + 4 * (lane >> 5);
+        if (h < N) {
+          u32x2 o = {Mma<T>::pack2(acc[nt][4 * q4], acc[nt][4 * q4 + 1]),
+                     Mma<T>::pack2(acc[nt][4 * q4 + 2], acc[nt][4 * q4 + 3])};
+          *reinterpret_cast<u32x2 *>(crow + h) = o;
+        }
+      }
+  }
+}
+
+// ------------------------------------------------------------------------------------------
+// P3: C[b,c,h] = sum_r T[r][c] * Y[b,r,h]
+// ------------------------------------------------------------------------------------------
+template <typename T, int NT, bool ALIGNED>
+__global__ __launch_bounds__(kThreads, 2) void mfma_p3_kernel(const uint16_t *__restrict__ A,
+                                                              const uint16_t *__restrict__ Y,
+                                                              uint16_t *__restrict__ C, int B, int M, int N, int w,
+                                                              int nblk, int64_t asb, int64_t ysb, int64_t ysr,
+                                                              int64_t csb, int64_t csr) {
+  constexpr int NP = 32 * NT;
+  constexpr int ST = lds_stride_tr(TM);  // T tile [KC rows r][TM cols c]
+  constexpr int SY = lds_stride_tr(NP);
+  __shared__ __attribute__((aligned(16))) uint16_t t_lds[2][KC * ST];
+  __shared__ __attribute__((aligned(16))) uint16_t y_lds[2][KC * SY];
+
+  int b, blk;
+  if (!decode_block(nblk, B, &b, &blk)) return;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int W = 2 * w + 1;
+  // block origin: aligned variant shifts it left so that every 8-column group is an aligned chunk
+  const int c0 = blk * TM - (ALIGNED ? (int)(((int64_t)b * asb + w) & 7) : 0);
+  const int c_first = max(c0, 0), c_last = min(c0 + TM, M) - 1;
+  if (c_first > c_last) return;
+  const int r_lo = max(c_first - w, 0), r_hi = min(c_last + w, M - 1);
+  const int nk = (r_hi - r_lo + KC) / KC;
+  const uint16_t *Ab = A + (int64_t)b * asb;
+  const uint16_t *Yb = Y + (int64_t)b * ysb;
+
+  const int ychunks = KC * (N >> 3), ncg = N >> 3;
+  int y_r[NT], y_h[NT];
+#pragma unroll
+  for (int s = 0; s < NT; ++s) {
+    const int q = tid + kThreads * s;
+    y_r[s] = q < ychunks ? q / ncg : -1;
+    y_h[s] = q < ychunks ? (q % ncg) * 8 : 0;
+  }
+
+  u32x4 t_reg[4], y_reg[NT];
+  auto fetch = [&](int k) {
+    const int rb = r_lo + k * KC;
+#pragma unroll
+    for (int s = 0; s < 4; ++s) {
+      const int q = tid + kThreads * s;
+      const int r = rb + (q >> 4), c8 = c0 + 8 * (q & 15);
+      const int lo = max(r - w, 0), hi = r <= r_hi ? min(r + w, M - 1) : -1;
+      t_reg[s] = load_band_chunk<ALIGNED>(Ab + (int64_t)r * W + (w - r) + c8, lo - c8, hi - c8);
+    }
+#pragma unroll
+    for (int s = 0; s < NT; ++s) {
+      const int r = rb + y_r[s];
+      u32x4 z = {0u, 0u, 0u, 0u};
+      y_reg[s] = (y_r[s] >= 0 && r <= r_hi) ? *reinterpret_cast<const u32x4 *>(Yb + (int64_t)r * ysr + y_h[s]) : z;
+    }
+  };
+  auto stash = [&](int buf) {
+#pragma unroll
+    for (int s = 0; s < 4; ++s) {
+      const int q = tid + kThreads * s;
+      *reinterpret_cast<u32x4 *>(&t_lds[buf][(q >> 4) * ST + (q & 15) * 8]) = t_reg[s];
+    }
+#pragma unroll
+    for (int s = 0; s < NT; ++s)
+      if (y_r[s] >= 0) *reinterpret_cast<u32x4 *>(&y_lds[buf][y_r[s] * SY + y_h[s]]) = y_reg[s];
+  };
+
+  f32x16 acc[NT];
+#pragma unroll
+  for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) acc[nt][v] = 0.f;
+
+  fetch(0);
+  stash(0);
+  __syncthreads();
+  for (int k = 0; k < nk; ++k) {
+    const int buf = k & 1;
+    if (k + 1 < nk) fetch(k + 1);
+#pragma unroll
+    for (int ks = 0; ks < KC / 16; ++ks) {
+      const u32x4 bop = lds_read_transposed(t_lds[buf], ST, ks * 16, wave * 32, lane);
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt) {
+        const u32x4 aop = lds_read_transposed(y_lds[buf], SY, ks * 16, 32 * nt, lane);
+        acc[nt] = Mma<T>::run(aop, bop, acc[nt]);
+      }
+    }
+    if (k + 1 < nk) stash(buf ^ 1);
+    __syncthreads();
+  }
+
+  const int c = c0 + wave * 32 + (lane & 31);
+  if (c >= 0 && c < M) {
+    uint16_t *crow = C + (int64_t)b * csb + (int64_t)c * csr;
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+      for (int q4 = 0; q4 < 4; ++q4) {
+        const int h = 32 * nt + 8 * q4 + 4 * (lane >> 5);
+        if (h < N) {
+          u32x2 o = {Mma<T>::pack2(acc[nt][4 * q4], acc[nt][4 * q4 + 1]),
+                     Mma<T>::pack2(acc[nt][4 * q4 + 2], acc[nt][4 * q4 + 3])};
+          *reinterpret_cast<u32x2 *>(crow + h) = o;
+        }
+      }
+  }
+}
+
+// ------------------------------------------------------------------------------------------
+// P1: band[b,i,c-i+w] = sum_h X[b,i,h] * Y[b,c,h]   (+0.0 where c is outside the sequence)
+// ------------------------------------------------------------------------------------------
+template <typename T, int NK, bool ALIGNED>  // NK = N / 16
+__global__ __launch_bounds__(kThreads, 2) void mfma_p1_kernel(const uint16_t *__restrict__ X,
+                                                              const uint16_t *__restrict__ Y,
+                                                              uint16_t *__restrict__ C, int B, int M, int w,
+                                                              int nblk, int64_t xsb, int64_t xsr, int64_t ysb,
+                                                              int64_t ysr, int64_t csb) {
+  constexpr int N = 16 * NK;
+  constexpr int SY = N + 8;   // Y chunk rows: 16 (mod 128) bytes apart in banks -> conflict-free b128 reads
+  constexpr int SS = KC + 8;  // per-wave staging rows
+  constexpr int YS = (KC * N / 8 + kThreads - 1) / kThreads;
+  __shared__ __attribute__((aligned(16))) uint16_t y_lds[2][KC * SY];
+  __shared__ __attribute__((aligned(16))) uint16_t s_lds[4][32 * SS];
+
+  int b, blk;
+  if (!decode_block(nblk, B, &b, &blk)) return;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int W = 2 * w + 1;
+  const int i0 = blk * TM;
+  const int rows = min(TM, M - i0);
+  const int c_lo = i0 - w, c_hi = i0 + rows - 1 + w;  // not clipped: out-of-sequence entries are written as zeros
+  const int c_start = ALIGNED ? c_lo - (int)(((int64_t)c_lo + (int64_t)b * csb + w) & 7) : c_lo;
+  const int nk = (c_hi - c_start + KC) / KC;
+  const uint16_t *Yb = Y + (int64_t)b * ysb;
+  uint16_t *Cb = C + (int64_t)b * csb;
+
+  // B-operand: this wave's 32 rows of X, all of N, kept in registers
+  u32x4 xop[NK];
+  {
+    const int i = i0 + wave * 32 + (lane & 31);
+    const uint16_t *xr = X + (int64_t)b * xsb + (int64_t)i * xsr + 8 * (lane >> 5);
+#pragma unroll
+    for (int ks = 0; ks < NK; ++ks) {
+      u32x4 z = {0u, 0u, 0u, 0u};
+      xop[ks] = i < M ? *reinterpret_cast<const u32x4 *>(xr + 16 * ks) : z;
+    }
+  }
+
+  u32x4 y_reg[YS];
+  auto fetch = [&](int k) {
+    const int cb = c_start + k * KC;
+#pragma unroll
+    for (int s = 0; s < YS; ++s) {
+      const int q = tid + kThreads * s;
+      const int c = cb + q / (N / 8);
+      u32x4 z = {0u, 0u, 0u, 0u};
+      y_reg[s] = (q < KC * N / 8 && c >= 0 && c < M)
+                     ? *reinterpret_cast<const u32x4 *>(Yb + (int64_t)c * ysr + (q % (N / 8)) * 8)
+                     : z;
+    }
+  };
+  auto stash = [&](int buf) {
+#pragma unroll
+    for (int s = 0; s < YS; ++s) {
+      const int q = tid + kThreads * s;
+      if (q < KC * N / 8) *reinterpret_cast<u32x4 *>(&y_lds[buf][(q / (N / 8)) * SY + (q % (N / 8)) * 8]) = y_reg[s];
+    }
+  };
+
+  fetch(0);
+  stash(0);
+  __syncthreads();
+  uint16_t *stage = s_lds[wave];
+  for (int k = 0; k < nk; ++k) {
+    const int buf = k & 1;
+    const int cb = c_start + k * KC;
+    if (k + 1 < nk) fetch(k + 1);
+#pragma unroll
+    for (int mt = 0; mt < KC / 32; ++mt) {
+      f32x16 acc;
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[v] = 0.f;
+      const uint16_t *yl = &y_lds[buf][(32 * mt + (lane & 31)) * SY + 8 * (lane >> 5)];
+#pragma unroll
+      for (int ks = 0; ks < NK; ++ks)
+        acc = Mma<T>::run(*reinterpret_cast<const u32x4 *>(yl + 16 * ks), xop[ks], acc);
+      // acc[v]: dense column = 32 mt + 8 (v / 4) + 4 (lane / 32) + v % 4, row = lane % 32
+#pragma unroll
+      for (int q4 = 0; q4 < 4; ++q4) {
+        const int cl = 32 * mt + 8 * q4 + 4 * (lane >> 5);
+        const int c = cb + cl;
+        uint32_t lo = Mma<T>::pack2(acc[4 * q4], acc[4 * q4 + 1]);
+        uint32_t hi = Mma<T>::pack2(acc[4 * q4 + 2], acc[4 * q4 + 3]);
+        // columns outside the sequence are +0.0 by definition, whatever X holds
+        if (c < 0 || c >= M) lo &= 0xffff0000u;
+        if (c + 1 < 0 || c + 1 >= M) lo &= 0x0000ffffu;
+        if (c + 2 < 0 || c + 2 >= M) hi &= 0xffff0000u;
+        if (c + 3 < 0 || c + 3 >= M) hi &= 0x0000ffffu;
+        u32x2 o = {lo, hi};
+        *reinterpret_cast<u32x2 *>(&stage[(lane & 31) * SS + cl]) = o;
+      }
+    }
+    wave_sync_lds();
+    // row-contiguous stores: 8 lanes cover the 64 dense columns of one row
+#pragma unroll
+    for (int s = 0; s < 4; ++s) {
+      const int q = lane + 64 * s, r = q >> 3, g = q & 7;
+      const int i = i0 + wave * 32 + r;
+      const int c8 = cb + 8 * g;
+      const int e_lo = (i - w) - c8, e_hi = (i + w) - c8;
+      if (i < M && e_hi >= 0 && e_lo <= 7) {
+        const u32x4 v = *reinterpret_cast<const u32x4 *>(&stage[r * SS + 8 * g]);
+        uint16_t *dst = Cb + (int64_t)i * W + (c8 - i + w);
+        if (e_lo <= 0 && e_hi >= 7) {
+          store_chunk<ALIGNED>(dst, v);
+        } else {
+#pragma unroll
+          for (int e = 0; e < 8; ++e)
+            if (e >= e_lo && e <= e_hi) dst[e] = (uint16_t)(v[e >> 1] >> (16 * (e & 1)));
+        }
+      }
+    }
+    wave_sync_lds();
+    if (k + 1 < nk) stash(buf ^ 1);
+    __syncthreads();
+  }
+}
+
+// ------------------------------------------------------------------------------------------
+// host side
+// ------------------------------------------------------------------------------------------
+bool shape_ok(int64_t M, int64_t N, int64_t w, int dtype) {
+  if (dtype != WM_DTYPE_BF16 && dtype != WM_DTYPE_F16) return false;
+  if (N < 16 || N > 128 || N % 16 != 0) return false;
+  if (M < 1 || w < 1) return false;
+  if (M > (1 << 30) || w > (1 << 28)) return false;
+  return true;
+}
+
+bool band_ok(const View &v, int64_t W) { return v.sc == 1 && v.sr == W && ((uintptr_t)v.data % 2) == 0; }
+bool band_aligned(const View &v, int64_t w, unsigned flags) {
+  return !(flags & WM_FLAG_NO_ALIGNED_BAND) && (w % 4 == 0) && ((uintptr_t)v.data % 16) == 0;
+}
+
+unsigned grid_size(int64_t B, int64_t nblk) { return (unsigned)(((B + 7) / 8) * 8 * nblk); }
+
+template <typename T, bool ALIGNED>
+hipError_t launch_p2(const Problem &p, const View &a, const View &y, const View &c) {
+  const int nblk = (int)((p.M + TM - 1) / TM);
+  const dim3 grid(grid_size(p.B, nblk)), block(kThreads);
+#define WM_P2(NT)                                                                                              \
+  hipLaunchKernelGGL((mfma_p2_kernel<T, NT, ALIGNED>), grid, block, 0, p.stream, (const uint16_t *)a.data,     \
+                     (const uint16_t *)y.data, (uint16_t *)c.data, (int)p.B, (int)p.M, (int)p.N, (int)p.w, nblk, \
+                     a.sb, y.sb, y.sr, c.sb, c.sr)
+  switch ((p.N + 31) / 32) {
+    case 1: WM_P2(1); break;
+    case 2: WM_P2(2); break;
+    case 3: WM_P2(3); break;
+    default: WM_P2(4); break;
+  }
+#undef WM_P2
+  return hipGetLastError();
+}
+
+template <typename T, bool ALIGNED>
+hipError_t launch_p3(const Problem &p, const View &a, const View &y, const View &c) {
+  const int nblk = (int)((p.M + 7 + TM - 1) / TM);
+  const dim3 grid(grid_size(p.B, nblk)), block(kThreads);
+#define WM_P3(NT)                                                                                              \
+  hipLaunchKernelGGL((mfma_p3_kernel<T, NT, ALIGNED>), grid, block, 0, p.stream, (const uint16_t *)a.data,     \
+                     (const uint16_t *)y.data, (uint16_t *)c.data, (int)p.B, (int)p.M, (int)p.N, (int)p.w, nblk, \
+                     a.sb, y.sb, y.sr, c.sb, c.sr)
+  switch ((p.N + 31) / 32) {
+    case 1: WM_P3(1); break;
+    case 2: WM_P3(2); break;
+    case 3: WM_P3(3); break;
+    default: WM_P3(4); break;
+  }
+#undef WM_P3
+  return hipGetLastError();
+}
+
+template <typename T, bool ALIGNED>
+hipError_t launch_p1(const Problem &p, const View &x, const View &y, const View &c) {
+  const int nblk = (int)((p.M + TM - 1) / TM);
+  const dim3 grid(grid_size(p.B, nblk)), block(kThreads);
+#define WM_P1(NK)                                                                                            \
+  hipLaunchKernelGGL((mfma_p1_kernel<T, NK, ALIGNED>), grid, block, 0, p.stream, (const uint16_t *)x.data,   \
+                     (const uint16_t *)y.data, (uint16_t *)c.data, (int)p.B, (int)p.M, (int)p.w, nblk, x.sb, \
+                     x.sr, y.sb, y.sr, c.sb)
+  switch (p.N / 16) {
+    case 1: WM_P1(1); break;
+    case 2: WM_P1(2); break;
+    case 3: WM_P1(3); break;
+    case 4: WM_P1(4); break;
+    case 5: WM_P1(5); break;
+    case 6: WM_P1(6); break;
+    case 7: WM_P1(7); break;
+    default: WM_P1(8); break;
+  }
+#undef WM_P1
+  return hipGetLastError();
+}
+
+template <bool ALIGNED>
+hipError_t by_dtype(int op, const Problem &p, const View &a, const View &y, const View &c) {
+  if (p.dtype == WM_DTYPE_BF16) {
+    if (op == 1) return launch_p1<bf16_t, ALIGNED>(p, a, y, c);
+    if (op == 2) return launch_p2<bf16_t, ALIGNED>(p, a, y, c);
+    return launch_p3<bf16_t, ALIGNED>(p, a, y, c);
+  }
+  if (op == 1) return launch_p1<f16_t, ALIGNED>(p, a, y, c);
+  if (op == 2) return launch_p2<f16_t, ALIGNED>(p, a, y, c);
+  return launch_p3<f16_t, ALIGNED>(p, a, y, c);
+}
+
+}  // namespace
+
+bool mfma_supports(int op, int64_t B, int64_t M, int64_t N, int64_t w, int dtype) {
+  (void)op;
+  (void)B;
+  return shape_ok(M, N, w, dtype);
+}
+
+bool try_launch_mfma_p1(const Problem &p, const View &x, const View &y, const View &c, hipError_t *err) {
+  if (!shape_ok(p.M, p.N, p.w, p.dtype)) return false;
+  if (!fast_layout(x, p.dtype) || !fast_layout(y, p.dtype) || !band_ok(c, 2 * p.w + 1)) return false;
+  *err = band_aligned(c, p.w, p.flags) ? by_dtype<true>(1, p, x, y, c) : by_dtype<false>(1, p, x, y, c);
+  return true;
+}
+
+bool try_launch_mfma_p2(const Problem &p, const View &a, const View &y, const View &c, hipError_t *err) {
+  if (!shape_ok(p.M, p.N, p.w, p.dtype)) return false;
+  if (!band_ok(a, 2 * p.w + 1) || !fast_layout(y, p.dtype) || !fast_layout(c, p.dtype)) return false;
+  *err = band_aligned(a, p.w, p.flags) ? by_dtype<true>(2, p, a, y, c) : by_dtype<false>(2, p, a, y, c);
+  return true;
+}
+
+bool try_launch_mfma_p3(const Problem &p, const View &a, const View &y, const View &c, hipError_t *err) {
+  if (!shape_ok(p.M, p.N, p.w, p.dtype)) return false;
+  if (!band_ok(a, 2 * p.w + 1) || !fast_layout(y, p.dtype) || !fast_layout(c, p.dtype)) return false;
+  *err = band_aligned(a, p.w, p.flags) ? by_dtype<true>(3, p, a, y, c) : by_dtype<false>(3, p, a, y, c);
+  return true;
+}
+
 }  // namespace wm

@@ -1,16 +1,23 @@
-"""ctypes view of libwindow_matmul_hip.so used by the tests (mirrors include/window_matmul_hip.h)."""
+"""ctypes binding of libwindow_matmul_hip.so (mirrors include/window_matmul_hip.h).
+
+For callers that want the C ABI without the PyTorch extension in between: the tests,
+the benchmark's per-kernel timing, and as a template for bindings from other hosts.
+Tensors are only used as (pointer, strides) carriers; work is enqueued on torch's
+current stream."""
 import ctypes
 import os
 import re
 
 import torch
 
-REPO = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-LIB_PATH = os.path.join(REPO, "pytorch-window-matmul_amd", "libwindow_matmul_hip.so")
+HERE = os.path.dirname(os.path.abspath(__file__))
+REPO = os.path.dirname(HERE)
+LIB_PATH = os.path.join(HERE, "libwindow_matmul_hip.so")
 HEADER = os.path.join(REPO, "include", "window_matmul_hip.h")
 
 DTYPES = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2, torch.float64: 3}
 FORCE_STRIDED = 0x1
+NO_ALIGNED_BAND = 0x2
 
 
 class Operand(ctypes.Structure):

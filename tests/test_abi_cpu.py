@@ -7,7 +7,7 @@ import inspect
 import pytest
 import torch
 
-import abi
+import wm_ctypes as abi
 
 
 def test_library_exports_every_declared_symbol():

@@ -10,7 +10,7 @@ import itertools
 import pytest
 import torch
 
-import abi
+import wm_ctypes as abi
 import oracle
 from conftest import seeded
 
