@@ -124,6 +124,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="c3", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--kernels-only", action="store_true",
+                    help="launch each of the six kernels --steps times and a reference copy, nothing else "
+                         "(for rocprofv3 counter passes)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU; --gpus must be 1 (the path shards over the batch "
@@ -160,14 +163,16 @@ def main():
 
     units = 6 if cfg["backward"] else 2
     flops = units * band_unit_flops(B, M, N, w)
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        step()
-    torch.cuda.synchronize()
-    ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+    ms_per_step = float("nan")
+    if not args.kernels_only:
+        for _ in range(args.warmup):
+            step()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            step()
+        torch.cuda.synchronize()
+        ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
 
     # per-kernel timing through the C ABI (one launch per call), same tensors, same stream
     with torch.no_grad():
@@ -224,6 +229,10 @@ def main():
         "copy_yardstick_GBps": round(copy_gbs, 1),
         "kernel_sum_GBps": round(len(per_kernel) * kb / sum(v["ms"] for v in per_kernel.values()) / 1e6, 1),
     }
+    if args.kernels_only:
+        print(json.dumps({"kernels": per_kernel, "copy_yardstick_GBps": round(copy_gbs, 1),
+                          "copy_bytes_each_way": att.numel() * es}), flush=True)
+        return
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(cfg)
     else:

@@ -38,6 +38,8 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 typedef short s16x4 __attribute__((ext_vector_type(4)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 
 constexpr int kThreads = 256;
 constexpr int TM = 128;  // rows per workgroup (32 per wave)
@@ -99,7 +101,8 @@ struct Mma<bf16_t> {
                                                    0, 0, 0);
   }
   static __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
-    return float_to_bf16_bits(lo) | (float_to_bf16_bits(hi) << 16);
+    f32x2 v = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2));  // v_cvt_pk_bf16_f32, RNE
   }
 };
 template <>
@@ -160,8 +163,8 @@ template <typename T, int NT, bool ALIGNED>
 __global__ __launch_bounds__(kThreads, 2) void mfma_p2_kernel(const uint16_t *__restrict__ A,
                                                               const uint16_t *__restrict__ Y,
                                                               uint16_t *__restrict__ C, int B, int M, int N, int w,
-                                                              int nblk, int64_t asb, int64_t ysb, int64_t ysr,
-                                                              int64_t csb, int64_t csr) {
+                                                              int nblk, int galign, int64_t asb, int64_t ysb,
+                                                              int64_t ysr, int64_t csb, int64_t csr) {
   constexpr int NP = 32 * NT;
   constexpr int ST = KC + 8;                         // T tile row stride: 144 B, conflict-free b128 reads
   constexpr int SY = lds_stride_tr(NP);
@@ -177,7 +180,7 @@ __global__ __launch_bounds__(kThreads, 2) void mfma_p2_kernel(const uint16_t *__
   const int c_lo = max(i0 - w, 0), c_hi = min(i0 + rows - 1 + w, M - 1);
   const uint16_t *Ab = A + (int64_t)b * asb;
   const uint16_t *Yb = Y + (int64_t)b * ysb;
-  const int c_start = ALIGNED ? c_lo - (int)(((int64_t)c_lo + (int64_t)b * asb + w) & 7) : c_lo;
+  const int c_start = ALIGNED ? c_lo - (int)(((int64_t)c_lo + (int64_t)b * asb + w) & (galign - 1)) : c_lo;
   const int nk = (c_hi - c_start + KC) / KC;
 
   // per-thread chunk coordinates (loop invariant)
@@ -278,8 +281,8 @@ template <typename T, int NT, bool ALIGNED>
 __global__ __launch_bounds__(kThreads, 2) void mfma_p3_kernel(const uint16_t *__restrict__ A,
                                                               const uint16_t *__restrict__ Y,
                                                               uint16_t *__restrict__ C, int B, int M, int N, int w,
-                                                              int nblk, int64_t asb, int64_t ysb, int64_t ysr,
-                                                              int64_t csb, int64_t csr) {
+                                                              int nblk, int galign, int64_t asb, int64_t ysb,
+                                                              int64_t ysr, int64_t csb, int64_t csr) {
   constexpr int NP = 32 * NT;
   constexpr int ST = lds_stride_tr(TM);  // T tile [KC rows r][TM cols c]
   constexpr int SY = lds_stride_tr(NP);
@@ -291,7 +294,7 @@ __global__ __launch_bounds__(kThreads, 2) void mfma_p3_kernel(const uint16_t *__
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int W = 2 * w + 1;
   // block origin: aligned variant shifts it left so that every 8-column group is an aligned chunk
-  const int c0 = blk * TM - (ALIGNED ? (int)(((int64_t)b * asb + w) & 7) : 0);
+  const int c0 = blk * TM - (ALIGNED ? (int)(((int64_t)b * asb + w) & (galign - 1)) : 0);
   const int c_first = max(c0, 0), c_last = min(c0 + TM, M) - 1;
   if (c_first > c_last) return;
   const int r_lo = max(c_first - w, 0), r_hi = min(c_last + w, M - 1);
@@ -385,8 +388,8 @@ template <typename T, int NK, bool ALIGNED>  // NK = N / 16
 __global__ __launch_bounds__(kThreads, 2) void mfma_p1_kernel(const uint16_t *__restrict__ X,
                                                               const uint16_t *__restrict__ Y,
                                                               uint16_t *__restrict__ C, int B, int M, int w,
-                                                              int nblk, int64_t xsb, int64_t xsr, int64_t ysb,
-                                                              int64_t ysr, int64_t csb) {
+                                                              int nblk, int galign, int64_t xsb, int64_t xsr,
+                                                              int64_t ysb, int64_t ysr, int64_t csb) {
   constexpr int N = 16 * NK;
   constexpr int SY = N + 8;   // Y chunk rows: 16 (mod 128) bytes apart in banks -> conflict-free b128 reads
   constexpr int SS = KC + 8;  // per-wave staging rows
@@ -401,7 +404,7 @@ __global__ __launch_bounds__(kThreads, 2) void mfma_p1_kernel(const uint16_t *__
   const int i0 = blk * TM;
   const int rows = min(TM, M - i0);
   const int c_lo = i0 - w, c_hi = i0 + rows - 1 + w;  // not clipped: out-of-sequence entries are written as zeros
-  const int c_start = ALIGNED ? c_lo - (int)(((int64_t)c_lo + (int64_t)b * csb + w) & 7) : c_lo;
+  const int c_start = ALIGNED ? c_lo - (int)(((int64_t)c_lo + (int64_t)b * csb + w) & (galign - 1)) : c_lo;
   const int nk = (c_hi - c_start + KC) / KC;
   const uint16_t *Yb = Y + (int64_t)b * ysb;
   uint16_t *Cb = C + (int64_t)b * csb;
@@ -513,17 +516,21 @@ bool band_ok(const View &v, int64_t W) { return v.sc == 1 && v.sr == W && ((uint
 bool band_aligned(const View &v, int64_t w, unsigned flags) {
   return !(flags & WM_FLAG_NO_ALIGNED_BAND) && (w % 4 == 0) && ((uintptr_t)v.data % 16) == 0;
 }
+// Column-group alignment (elements) of the ALIGNED kernels: whole 128-byte lines when the
+// skew per row (2w elements) keeps them aligned, 16-byte chunks otherwise.
+int band_group(const View &v, int64_t w) { return (w % 32 == 0 && ((uintptr_t)v.data % 128) == 0) ? 64 : 8; }
 
 unsigned grid_size(int64_t B, int64_t nblk) { return (unsigned)(((B + 7) / 8) * 8 * nblk); }
 
 template <typename T, bool ALIGNED>
 hipError_t launch_p2(const Problem &p, const View &a, const View &y, const View &c) {
   const int nblk = (int)((p.M + TM - 1) / TM);
+  const int galign = band_group(a, p.w);
   const dim3 grid(grid_size(p.B, nblk)), block(kThreads);
 #define WM_P2(NT)                                                                                              \
   hipLaunchKernelGGL((mfma_p2_kernel<T, NT, ALIGNED>), grid, block, 0, p.stream, (const uint16_t *)a.data,     \
                      (const uint16_t *)y.data, (uint16_t *)c.data, (int)p.B, (int)p.M, (int)p.N, (int)p.w, nblk, \
-                     a.sb, y.sb, y.sr, c.sb, c.sr)
+                     galign, a.sb, y.sb, y.sr, c.sb, c.sr)
   switch ((p.N + 31) / 32) {
     case 1: WM_P2(1); break;
     case 2: WM_P2(2); break;
@@ -536,12 +543,13 @@ hipError_t launch_p2(const Problem &p, const View &a, const View &y, const View 
 
 template <typename T, bool ALIGNED>
 hipError_t launch_p3(const Problem &p, const View &a, const View &y, const View &c) {
-  const int nblk = (int)((p.M + 7 + TM - 1) / TM);
+  const int galign = band_group(a, p.w);
+  const int nblk = (int)((p.M + (ALIGNED ? galign - 1 : 0) + TM - 1) / TM);
   const dim3 grid(grid_size(p.B, nblk)), block(kThreads);
 #define WM_P3(NT)                                                                                              \
   hipLaunchKernelGGL((mfma_p3_kernel<T, NT, ALIGNED>), grid, block, 0, p.stream, (const uint16_t *)a.data,     \
                      (const uint16_t *)y.data, (uint16_t *)c.data, (int)p.B, (int)p.M, (int)p.N, (int)p.w, nblk, \
-                     a.sb, y.sb, y.sr, c.sb, c.sr)
+                     galign, a.sb, y.sb, y.sr, c.sb, c.sr)
   switch ((p.N + 31) / 32) {
     case 1: WM_P3(1); break;
     case 2: WM_P3(2); break;
@@ -555,11 +563,12 @@ hipError_t launch_p3(const Problem &p, const View &a, const View &y, const View 
 template <typename T, bool ALIGNED>
 hipError_t launch_p1(const Problem &p, const View &x, const View &y, const View &c) {
   const int nblk = (int)((p.M + TM - 1) / TM);
+  const int galign = band_group(c, p.w);
   const dim3 grid(grid_size(p.B, nblk)), block(kThreads);
 #define WM_P1(NK)                                                                                            \
   hipLaunchKernelGGL((mfma_p1_kernel<T, NK, ALIGNED>), grid, block, 0, p.stream, (const uint16_t *)x.data,   \
-                     (const uint16_t *)y.data, (uint16_t *)c.data, (int)p.B, (int)p.M, (int)p.w, nblk, x.sb, \
-                     x.sr, y.sb, y.sr, c.sb)
+                     (const uint16_t *)y.data, (uint16_t *)c.data, (int)p.B, (int)p.M, (int)p.w, nblk, galign, \
+                     x.sb, x.sr, y.sb, y.sr, c.sb)
   switch (p.N / 16) {
     case 1: WM_P1(1); break;
     case 2: WM_P1(2); break;

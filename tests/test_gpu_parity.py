@@ -29,7 +29,7 @@ REF_GRID = [(2, M, N, w) for (M, N), w in itertools.product([(1, 3), (4, 3), (16
 EDGE = [
     (3, 37, 5, 6), (1, 1, 8, 3), (2, 129, 64, 4), (2, 130, 64, 64), (1, 257, 80, 33), (2, 100, 128, 49),
     (1, 300, 64, 150), (2, 65, 16, 100), (1, 513, 72, 256), (2, 96, 64, 8), (1, 200, 40, 12), (3, 64, 64, 1),
-    (1, 1000, 64, 32), (2, 333, 24, 7),
+    (1, 1000, 64, 32), (2, 333, 24, 7), (3, 700, 64, 32), (1, 1100, 32, 256), (2, 900, 128, 64), (9, 260, 16, 96),
 ]
 CASES = REF_GRID + EDGE
 DTYPES = [torch.float32, torch.bfloat16, torch.float16, torch.float64]
