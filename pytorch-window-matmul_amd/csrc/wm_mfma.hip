@@ -44,6 +44,7 @@ typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 constexpr int kThreads = 256;
 constexpr int TM = 128;  // rows per workgroup (32 per wave)
 constexpr int KC = 64;   // chunk length along the contraction (P2, P3) / dense columns (P1)
+constexpr int PF = 2;    // chunks requested ahead of the one being multiplied (P2, P3)
 
 struct __attribute__((packed, aligned(2))) Chunk2 {
   u32x4 v;
@@ -74,22 +75,36 @@ __device__ __forceinline__ u32x4 keep_range(u32x4 v, int e_lo, int e_hi) {
   return r;
 }
 
-// Loads the 8 band elements of one skewed-tile chunk; only [e_lo, e_hi] is valid.
-// A chunk with no valid element is never touched.  Partial chunks are read whole
-// when that cannot leave the allocation (aligned chunks never straddle a page),
-// element by element otherwise.
+// Band chunk = 8 consecutive dense columns of one row of the skewed tile, of which only
+// elements [e_lo, e_hi] are valid.  Loading is split in two branch-free halves so that the
+// prefetch contains nothing but loads (a use of the loaded value, or a load inside a branch,
+// makes the compiler wait for memory on the spot and serialises the pipeline):
+//   fetch_band_chunk  issues the 16-byte load; from `safe` (any readable, suitably aligned
+//                     address) when no element is valid;
+//   mask_band_chunk   clears the invalid elements, later, when the chunk goes to LDS.
+// A partially valid chunk is read whole: with w >= 7 the up-to-7 elements on either side of a
+// row's valid range are band entries of the same or the neighbouring row, i.e. inside the
+// tensor (the kernels are only used for w >= 8).
+__device__ __forceinline__ bool band_chunk_any(int e_lo, int e_hi) { return (e_hi >= 0) & (e_lo <= 7) & (e_lo <= e_hi); }
 template <bool ALIGNED>
-__device__ __forceinline__ u32x4 load_band_chunk(const uint16_t *p, int e_lo, int e_hi) {
-  u32x4 z = {0u, 0u, 0u, 0u};
-  if (e_hi < 0 || e_lo > 7 || e_lo > e_hi) return z;
-  if (e_lo <= 0 && e_hi >= 7) return load_chunk<ALIGNED>(p);
-  if (ALIGNED) return keep_range(load_chunk<true>(p), e_lo, e_hi);
-  const int lo = e_lo < 0 ? 0 : e_lo, hi = e_hi > 7 ? 7 : e_hi;
-  uint32_t h[8];
-#pragma unroll
-  for (int e = 0; e < 8; ++e) h[e] = (e >= lo && e <= hi) ? (uint32_t)p[e] : 0u;
-  u32x4 r = {h[0] | (h[1] << 16), h[2] | (h[3] << 16), h[4] | (h[5] << 16), h[6] | (h[7] << 16)};
+__device__ __forceinline__ u32x4 fetch_band_chunk(const uint16_t *p, const uint16_t *safe, int e_lo, int e_hi) {
+  return load_chunk<ALIGNED>(band_chunk_any(e_lo, e_hi) ? p : safe);
+}
+__device__ __forceinline__ u32x4 mask_band_chunk(u32x4 v, int e_lo, int e_hi) {
+  return keep_range(v, band_chunk_any(e_lo, e_hi) ? e_lo : 8, e_hi);
+}
+
+// Row chunk of a dense operand; rows outside the sequence are fetched from `safe` and zeroed later.
+__device__ __forceinline__ u32x4 fetch_row_chunk(const uint16_t *p, const uint16_t *safe, bool valid) {
+  return *reinterpret_cast<const u32x4 *>(valid ? p : safe);
+}
+__device__ __forceinline__ u32x4 mask_row_chunk(u32x4 v, bool valid) {
+  const uint32_t m = valid ? 0xffffffffu : 0u;
+  u32x4 r = {v[0] & m, v[1] & m, v[2] & m, v[3] & m};
   return r;
+}
+__device__ __forceinline__ u32x4 load_row_chunk(const uint16_t *p, const uint16_t *safe, bool valid) {
+  return mask_row_chunk(fetch_row_chunk(p, safe, valid), valid);
 }
 
 template <typename T>
@@ -136,6 +151,13 @@ __device__ __forceinline__ u32x4 lds_read_transposed(const uint16_t *mat, int st
   return r;
 }
 
+// Pins a prefetched register at this point of the program: the compiler may not use the value
+// (and therefore may not wait for its load) any earlier than here.
+__device__ __forceinline__ u32x4 pin(u32x4 v) {
+  asm volatile("" : "+v"(v));
+  return v;
+}
+
 __device__ __forceinline__ void wave_sync_lds() {
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
   __builtin_amdgcn_wave_barrier();
@@ -169,7 +191,7 @@ __global__ __launch_bounds__(kThreads, 2) void mfma_p2_kernel(const uint16_t *__
   constexpr int ST = KC + 8;                         // T tile row stride: 144 B, conflict-free b128 reads
   constexpr int SY = lds_stride_tr(NP);
   __shared__ __attribute__((aligned(16))) uint16_t t_lds[2][TM * ST];
-  __shared__ __attribute__((aligned(16))) uint16_t y_lds[2][KC * SY];
+  __shared__ __attribute__((aligned(16))) uint16_t y_lds[2][(KC + 1) * SY];  // row KC: sink for idle loader slots
 
   int b, blk;
   if (!decode_block(nblk, B, &b, &blk)) return;
@@ -199,35 +221,40 @@ __global__ __launch_bounds__(kThreads, 2) void mfma_p2_kernel(const uint16_t *__
 #pragma unroll
   for (int s = 0; s < NT; ++s) {
     const int q = tid + kThreads * s;
-    y_r[s] = q < ychunks ? q / ncg : -1;
+    y_r[s] = q < ychunks ? q / ncg : KC;  // KC = no row: loads nothing real, writes to the sink row
     y_h[s] = q < ychunks ? (q % ncg) * 8 : 0;
   }
 
-  u32x4 t_reg[4], y_reg[NT];
-  auto fetch = [&](int k) {
+  // Register-staged prefetch PF chunks deep: chunk k+PF is requested before chunk k is
+  // multiplied, so PF chunks of band and Y rows are in flight per workgroup at any time.
+  u32x4 t_reg[PF][4], y_reg[PF][NT];
+  auto fetch = [&](int k, u32x4(&tr)[4], u32x4(&yr)[NT]) {  // loads only
     const int cb = c_start + k * KC;
 #pragma unroll
     for (int s = 0; s < 4; ++s) {
-      const int g = (tid + kThreads * s) & 7;
-      const int c8 = cb + 8 * g;
-      t_reg[s] = load_band_chunk<ALIGNED>(t_ptr[s] + c8, t_lo[s] - c8, t_hi[s] - c8);
+      const int c8 = cb + 8 * ((tid + kThreads * s) & 7);
+      tr[s] = fetch_band_chunk<ALIGNED>(t_ptr[s] + c8, A, t_lo[s] - c8, t_hi[s] - c8);
     }
 #pragma unroll
     for (int s = 0; s < NT; ++s) {
       const int c = cb + y_r[s];
-      u32x4 z = {0u, 0u, 0u, 0u};
-      y_reg[s] = (y_r[s] >= 0 && c >= 0 && c < M) ? *reinterpret_cast<const u32x4 *>(Yb + (int64_t)c * ysr + y_h[s]) : z;
+      yr[s] = fetch_row_chunk(Yb + (int64_t)c * ysr + y_h[s], Y, (y_r[s] < KC) & (c >= 0) & (c <= c_hi));
     }
   };
-  auto stash = [&](int buf) {
+  auto stash = [&](int k, const u32x4(&tr)[4], const u32x4(&yr)[NT]) {  // mask, then to LDS buffer k & 1
+    const int cb = c_start + k * KC, buf = k & 1;
 #pragma unroll
     for (int s = 0; s < 4; ++s) {
       const int q = tid + kThreads * s;
-      *reinterpret_cast<u32x4 *>(&t_lds[buf][(q >> 3) * ST + (q & 7) * 8]) = t_reg[s];
+      const int c8 = cb + 8 * (q & 7);
+      *reinterpret_cast<u32x4 *>(&t_lds[buf][(q >> 3) * ST + (q & 7) * 8]) =
+          mask_band_chunk(pin(tr[s]), t_lo[s] - c8, t_hi[s] - c8);
     }
 #pragma unroll
-    for (int s = 0; s < NT; ++s)
-      if (y_r[s] >= 0) *reinterpret_cast<u32x4 *>(&y_lds[buf][y_r[s] * SY + y_h[s]]) = y_reg[s];
+    for (int s = 0; s < NT; ++s) {
+      const int c = cb + y_r[s];
+      *reinterpret_cast<u32x4 *>(&y_lds[buf][y_r[s] * SY + y_h[s]]) = mask_row_chunk(pin(yr[s]), (c >= 0) & (c <= c_hi));
+    }
   };
 
   f32x16 acc[NT];
@@ -236,12 +263,20 @@ __global__ __launch_bounds__(kThreads, 2) void mfma_p2_kernel(const uint16_t *__
 #pragma unroll
     for (int v = 0; v < 16; ++v) acc[nt][v] = 0.f;
 
-  fetch(0);
-  stash(0);
+#pragma unroll
+  for (int s = 0; s < PF; ++s) fetch(s, t_reg[s], y_reg[s]);
+  __builtin_amdgcn_sched_barrier(0);
+  stash(0, t_reg[0], y_reg[0]);
   __syncthreads();
-  for (int k = 0; k < nk; ++k) {
+  // One pipeline slot: request chunk k+PF into register set `mine`, multiply chunk k out of
+  // LDS, then move chunk k+1 (register set `next`, requested PF-1 slots ago) into LDS.
+  // The prefetch is unconditional -- chunks past the end are invalid by their coordinates and
+  // read the safe address -- and the slots are chained by explicit loop exits, so that the
+  // compiler can count outstanding loads exactly and waits only for the set it stores.
+  auto slot = [&](int k, u32x4(&mine_t)[4], u32x4(&mine_y)[NT], u32x4(&next_t)[4], u32x4(&next_y)[NT]) {
     const int buf = k & 1;
-    if (k + 1 < nk) fetch(k + 1);
+    fetch(k + PF, mine_t, mine_y);
+    __builtin_amdgcn_sched_barrier(0);
     const uint16_t *tl = &t_lds[buf][(wave * 32 + (lane & 31)) * ST + 8 * (lane >> 5)];
 #pragma unroll
     for (int ks = 0; ks < KC / 16; ++ks) {
@@ -252,8 +287,16 @@ __global__ __launch_bounds__(kThreads, 2) void mfma_p2_kernel(const uint16_t *__
         acc[nt] = Mma<T>::run(aop, bop, acc[nt]);
       }
     }
-    if (k + 1 < nk) stash(buf ^ 1);
+    __builtin_amdgcn_sched_barrier(0);
+    stash(k + 1, next_t, next_y);
     __syncthreads();
+  };
+  static_assert(PF == 2, "the slot chain below is written out for two register sets");
+  for (int k = 0;;) {
+    slot(k, t_reg[0], y_reg[0], t_reg[1], y_reg[1]);
+    if (++k >= nk) break;
+    slot(k, t_reg[1], y_reg[1], t_reg[0], y_reg[0]);
+    if (++k >= nk) break;
   }
 
   // acc[nt][v]: h = 32 nt + 8 (v / 4) + 4 (lane / 32) + v % 4, row = wave * 32 + lane % 32
@@ -287,7 +330,7 @@ __global__ __launch_bounds__(kThreads, 2) void mfma_p3_kernel(const uint16_t *__
   constexpr int ST = lds_stride_tr(TM);  // T tile [KC rows r][TM cols c]
   constexpr int SY = lds_stride_tr(NP);
   __shared__ __attribute__((aligned(16))) uint16_t t_lds[2][KC * ST];
-  __shared__ __attribute__((aligned(16))) uint16_t y_lds[2][KC * SY];
+  __shared__ __attribute__((aligned(16))) uint16_t y_lds[2][(KC + 1) * SY];  // row KC: sink for idle loader slots
 
   int b, blk;
   if (!decode_block(nblk, B, &b, &blk)) return;
@@ -307,36 +350,39 @@ __global__ __launch_bounds__(kThreads, 2) void mfma_p3_kernel(const uint16_t *__
 #pragma unroll
   for (int s = 0; s < NT; ++s) {
     const int q = tid + kThreads * s;
-    y_r[s] = q < ychunks ? q / ncg : -1;
+    y_r[s] = q < ychunks ? q / ncg : KC;  // KC = no row: loads nothing real, writes to the sink row
     y_h[s] = q < ychunks ? (q % ncg) * 8 : 0;
   }
 
-  u32x4 t_reg[4], y_reg[NT];
-  auto fetch = [&](int k) {
+  u32x4 t_reg[PF][4], y_reg[PF][NT];
+  auto fetch = [&](int k, u32x4(&tr)[4], u32x4(&yr)[NT]) {  // loads only
     const int rb = r_lo + k * KC;
 #pragma unroll
     for (int s = 0; s < 4; ++s) {
       const int q = tid + kThreads * s;
       const int r = rb + (q >> 4), c8 = c0 + 8 * (q & 15);
-      const int lo = max(r - w, 0), hi = r <= r_hi ? min(r + w, M - 1) : -1;
-      t_reg[s] = load_band_chunk<ALIGNED>(Ab + (int64_t)r * W + (w - r) + c8, lo - c8, hi - c8);
+      const int lo = max(r - w, 0), hi = r <= r_hi ? min(r + w, M - 1) : -1;  // r > r_hi also covers k >= nk
+      tr[s] = fetch_band_chunk<ALIGNED>(Ab + (int64_t)r * W + (w - r) + c8, A, lo - c8, hi - c8);
     }
 #pragma unroll
     for (int s = 0; s < NT; ++s) {
       const int r = rb + y_r[s];
-      u32x4 z = {0u, 0u, 0u, 0u};
-      y_reg[s] = (y_r[s] >= 0 && r <= r_hi) ? *reinterpret_cast<const u32x4 *>(Yb + (int64_t)r * ysr + y_h[s]) : z;
+      yr[s] = fetch_row_chunk(Yb + (int64_t)r * ysr + y_h[s], Y, (y_r[s] < KC) & (r <= r_hi));
     }
   };
-  auto stash = [&](int buf) {
+  auto stash = [&](int k, const u32x4(&tr)[4], const u32x4(&yr)[NT]) {  // mask, then to LDS buffer k & 1
+    const int rb = r_lo + k * KC, buf = k & 1;
 #pragma unroll
     for (int s = 0; s < 4; ++s) {
       const int q = tid + kThreads * s;
-      *reinterpret_cast<u32x4 *>(&t_lds[buf][(q >> 4) * ST + (q & 15) * 8]) = t_reg[s];
+      const int r = rb + (q >> 4), c8 = c0 + 8 * (q & 15);
+      const int lo = max(r - w, 0), hi = r <= r_hi ? min(r + w, M - 1) : -1;
+      *reinterpret_cast<u32x4 *>(&t_lds[buf][(q >> 4) * ST + (q & 15) * 8]) =
+          mask_band_chunk(pin(tr[s]), lo - c8, hi - c8);
     }
 #pragma unroll
     for (int s = 0; s < NT; ++s)
-      if (y_r[s] >= 0) *reinterpret_cast<u32x4 *>(&y_lds[buf][y_r[s] * SY + y_h[s]]) = y_reg[s];
+      *reinterpret_cast<u32x4 *>(&y_lds[buf][y_r[s] * SY + y_h[s]]) = mask_row_chunk(pin(yr[s]), rb + y_r[s] <= r_hi);
   };
 
   f32x16 acc[NT];
@@ -345,12 +391,16 @@ __global__ __launch_bounds__(kThreads, 2) void mfma_p3_kernel(const uint16_t *__
 #pragma unroll
     for (int v = 0; v < 16; ++v) acc[nt][v] = 0.f;
 
-  fetch(0);
-  stash(0);
+#pragma unroll
+  for (int s = 0; s < PF; ++s) fetch(s, t_reg[s], y_reg[s]);
+  __builtin_amdgcn_sched_barrier(0);
+  stash(0, t_reg[0], y_reg[0]);
   __syncthreads();
-  for (int k = 0; k < nk; ++k) {
+  // same slot chain as in the band-in kernel above
+  auto slot = [&](int k, u32x4(&mine_t)[4], u32x4(&mine_y)[NT], u32x4(&next_t)[4], u32x4(&next_y)[NT]) {
     const int buf = k & 1;
-    if (k + 1 < nk) fetch(k + 1);
+    fetch(k + PF, mine_t, mine_y);
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int ks = 0; ks < KC / 16; ++ks) {
       const u32x4 bop = lds_read_transposed(t_lds[buf], ST, ks * 16, wave * 32, lane);
@@ -360,8 +410,16 @@ __global__ __launch_bounds__(kThreads, 2) void mfma_p3_kernel(const uint16_t *__
         acc[nt] = Mma<T>::run(aop, bop, acc[nt]);
       }
     }
-    if (k + 1 < nk) stash(buf ^ 1);
+    __builtin_amdgcn_sched_barrier(0);
+    stash(k + 1, next_t, next_y);
     __syncthreads();
+  };
+  static_assert(PF == 2, "the slot chain below is written out for two register sets");
+  for (int k = 0;;) {
+    slot(k, t_reg[0], y_reg[0], t_reg[1], y_reg[1]);
+    if (++k >= nk) break;
+    slot(k, t_reg[1], y_reg[1], t_reg[0], y_reg[0]);
+    if (++k >= nk) break;
   }
 
   const int c = c0 + wave * 32 + (lane & 31);
@@ -415,10 +473,7 @@ __global__ __launch_bounds__(kThreads, 2) void mfma_p1_kernel(const uint16_t *__
     const int i = i0 + wave * 32 + (lane & 31);
     const uint16_t *xr = X + (int64_t)b * xsb + (int64_t)i * xsr + 8 * (lane >> 5);
 #pragma unroll
-    for (int ks = 0; ks < NK; ++ks) {
-      u32x4 z = {0u, 0u, 0u, 0u};
-      xop[ks] = i < M ? *reinterpret_cast<const u32x4 *>(xr + 16 * ks) : z;
-    }
+    for (int ks = 0; ks < NK; ++ks) xop[ks] = load_row_chunk(xr + 16 * ks, X, i < M);
   }
 
   u32x4 y_reg[YS];
@@ -428,17 +483,18 @@ __global__ __launch_bounds__(kThreads, 2) void mfma_p1_kernel(const uint16_t *__
     for (int s = 0; s < YS; ++s) {
       const int q = tid + kThreads * s;
       const int c = cb + q / (N / 8);
-      u32x4 z = {0u, 0u, 0u, 0u};
-      y_reg[s] = (q < KC * N / 8 && c >= 0 && c < M)
-                     ? *reinterpret_cast<const u32x4 *>(Yb + (int64_t)c * ysr + (q % (N / 8)) * 8)
-                     : z;
+      y_reg[s] = fetch_row_chunk(Yb + (int64_t)c * ysr + (q % (N / 8)) * 8, Y, q < KC * N / 8 && c >= 0 && c < M);
     }
   };
-  auto stash = [&](int buf) {
+  auto stash = [&](int k) {
+    const int cb = c_start + k * KC, buf = k & 1;
 #pragma unroll
     for (int s = 0; s < YS; ++s) {
       const int q = tid + kThreads * s;
-      if (q < KC * N / 8) *reinterpret_cast<u32x4 *>(&y_lds[buf][(q / (N / 8)) * SY + (q % (N / 8)) * 8]) = y_reg[s];
+      const int c = cb + q / (N / 8);
+      if (q < KC * N / 8)
+        *reinterpret_cast<u32x4 *>(&y_lds[buf][(q / (N / 8)) * SY + (q % (N / 8)) * 8]) =
+            mask_row_chunk(y_reg[s], c >= 0 && c < M);
     }
   };
 
@@ -496,7 +552,7 @@ __global__ __launch_bounds__(kThreads, 2) void mfma_p1_kernel(const uint16_t *__
       }
     }
     wave_sync_lds();
-    if (k + 1 < nk) stash(buf ^ 1);
+    if (k + 1 < nk) stash(k + 1);
     __syncthreads();
   }
 }
@@ -507,7 +563,7 @@ __global__ __launch_bounds__(kThreads, 2) void mfma_p1_kernel(const uint16_t *__
 bool shape_ok(int64_t M, int64_t N, int64_t w, int dtype) {
   if (dtype != WM_DTYPE_BF16 && dtype != WM_DTYPE_F16) return false;
   if (N < 16 || N > 128 || N % 16 != 0) return false;
-  if (M < 1 || w < 1) return false;
+  if (M < 1 || w < 8) return false;  // partial band chunks are read whole, which needs w >= 7
   if (M > (1 << 30) || w > (1 << 28)) return false;
   return true;
 }
