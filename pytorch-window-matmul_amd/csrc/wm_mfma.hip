@@ -442,6 +442,14 @@ __global__ __launch_bounds__(kThreads, 2) void mfma_p3_kernel(const uint16_t *__
 // ------------------------------------------------------------------------------------------
 // P1: band[b,i,c-i+w] = sum_h X[b,i,h] * Y[b,c,h]   (+0.0 where c is outside the sequence)
 // ------------------------------------------------------------------------------------------
+// Element-wise store of elements [e_lo, e_hi] of a chunk (the slow path for chunk pieces that
+// cannot be completed with their neighbour row's piece).
+__device__ __forceinline__ void store_chunk_elements(uint16_t *dst, u32x4 v, int e_lo, int e_hi) {
+#pragma unroll
+  for (int e = 0; e < 8; ++e)
+    if (e >= e_lo && e <= e_hi) dst[e] = (uint16_t)(v[e >> 1] >> (16 * (e & 1)));
+}
+
 template <typename T, int NK, bool ALIGNED>  // NK = N / 16
 __global__ __launch_bounds__(kThreads, 2) void mfma_p1_kernel(const uint16_t *__restrict__ X,
                                                               const uint16_t *__restrict__ Y,
@@ -452,8 +460,13 @@ __global__ __launch_bounds__(kThreads, 2) void mfma_p1_kernel(const uint16_t *__
   constexpr int SY = N + 8;   // Y chunk rows: 16 (mod 128) bytes apart in banks -> conflict-free b128 reads
   constexpr int SS = KC + 8;  // per-wave staging rows
   constexpr int YS = (KC * N / 8 + kThreads - 1) / kThreads;
-  __shared__ __attribute__((aligned(16))) uint16_t y_lds[2][KC * SY];
+  __shared__ __attribute__((aligned(16))) uint16_t y_lds[2][(KC + 1) * SY];  // row KC: sink for idle loader slots
   __shared__ __attribute__((aligned(16))) uint16_t s_lds[4][32 * SS];
+  // Seam buffer.  The 16-byte chunk that holds the first band entries of row i also holds the
+  // last entries of row i-1 (band rows have odd length).  The head piece is parked here when
+  // its tile is produced; when the tail piece of the row above turns up, many column chunks
+  // later, the two are merged and leave as one aligned 16-byte store.
+  __shared__ __attribute__((aligned(16))) uint16_t seam[TM * 8];
 
   int b, blk;
   if (!decode_block(nblk, B, &b, &blk)) return;
@@ -466,6 +479,10 @@ __global__ __launch_bounds__(kThreads, 2) void mfma_p1_kernel(const uint16_t *__
   const int nk = (c_hi - c_start + KC) / KC;
   const uint16_t *Yb = Y + (int64_t)b * ysb;
   uint16_t *Cb = C + (int64_t)b * csb;
+  // Head and tail pieces of neighbouring rows meet through the seam buffer when both rows belong
+  // to this wave, or to any wave of the workgroup if a workgroup barrier is certain to separate
+  // the two tiles (the tail is produced 2w-1 columns after the head: at least two chunks later).
+  const bool seam_across_waves = ALIGNED && (2 * w - 1 >= 2 * KC);
 
   // B-operand: this wave's 32 rows of X, all of N, kept in registers
   u32x4 xop[NK];
@@ -476,36 +493,41 @@ __global__ __launch_bounds__(kThreads, 2) void mfma_p1_kernel(const uint16_t *__
     for (int ks = 0; ks < NK; ++ks) xop[ks] = load_row_chunk(xr + 16 * ks, X, i < M);
   }
 
-  u32x4 y_reg[YS];
-  auto fetch = [&](int k) {
+  int y_r[YS], y_h[YS];
+#pragma unroll
+  for (int s = 0; s < YS; ++s) {
+    const int q = tid + kThreads * s;
+    y_r[s] = q < KC * N / 8 ? q / (N / 8) : KC;  // KC = no row: loads nothing real, writes to the sink row
+    y_h[s] = q < KC * N / 8 ? (q % (N / 8)) * 8 : 0;
+  }
+  u32x4 y_reg[PF][YS];
+  auto fetch = [&](int k, u32x4(&yr)[YS]) {  // loads only; chunks past c_hi read the safe address
     const int cb = c_start + k * KC;
 #pragma unroll
     for (int s = 0; s < YS; ++s) {
-      const int q = tid + kThreads * s;
-      const int c = cb + q / (N / 8);
-      y_reg[s] = fetch_row_chunk(Yb + (int64_t)c * ysr + (q % (N / 8)) * 8, Y, q < KC * N / 8 && c >= 0 && c < M);
+      const int c = cb + y_r[s];
+      yr[s] = fetch_row_chunk(Yb + (int64_t)c * ysr + y_h[s], Y, (y_r[s] < KC) & (c >= 0) & (c < M) & (c <= c_hi));
     }
   };
-  auto stash = [&](int k) {
+  auto stash = [&](int k, const u32x4(&yr)[YS]) {
     const int cb = c_start + k * KC, buf = k & 1;
 #pragma unroll
     for (int s = 0; s < YS; ++s) {
-      const int q = tid + kThreads * s;
-      const int c = cb + q / (N / 8);
-      if (q < KC * N / 8)
-        *reinterpret_cast<u32x4 *>(&y_lds[buf][(q / (N / 8)) * SY + (q % (N / 8)) * 8]) =
-            mask_row_chunk(y_reg[s], c >= 0 && c < M);
+      const int c = cb + y_r[s];
+      *reinterpret_cast<u32x4 *>(&y_lds[buf][y_r[s] * SY + y_h[s]]) =
+          mask_row_chunk(pin(yr[s]), (c >= 0) & (c < M) & (c <= c_hi));
     }
   };
 
-  fetch(0);
-  stash(0);
-  __syncthreads();
   uint16_t *stage = s_lds[wave];
-  for (int k = 0; k < nk; ++k) {
+  // One slot: request Y chunk k+PF, multiply chunk k, stage the 32 x 64 result, store it, then move
+  // chunk k+1 into LDS.  The stores are issued before the wait for chunk k+1, which was requested
+  // a whole slot earlier, so the wait leaves them (and the newest loads) in flight.
+  auto slot = [&](int k, u32x4(&mine)[YS], u32x4(&next)[YS]) {
     const int buf = k & 1;
     const int cb = c_start + k * KC;
-    if (k + 1 < nk) fetch(k + 1);
+    fetch(k + PF, mine);
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int mt = 0; mt < KC / 32; ++mt) {
       f32x16 acc;
@@ -532,28 +554,69 @@ __global__ __launch_bounds__(kThreads, 2) void mfma_p1_kernel(const uint16_t *__
       }
     }
     wave_sync_lds();
-    // row-contiguous stores: 8 lanes cover the 64 dense columns of one row
+    // Row-contiguous stores: 8 lanes cover the 64 dense columns of one row.
+    // pass A: whole chunks go out; head pieces are parked in the seam buffer.
+    u32x4 v[4];
+    int tail_hi[4];  // >= 0: this slot holds a tail piece with elements 0..tail_hi, handled in pass B
 #pragma unroll
     for (int s = 0; s < 4; ++s) {
       const int q = lane + 64 * s, r = q >> 3, g = q & 7;
-      const int i = i0 + wave * 32 + r;
+      const int rw = wave * 32 + r, i = i0 + rw;
       const int c8 = cb + 8 * g;
       const int e_lo = (i - w) - c8, e_hi = (i + w) - c8;
+      tail_hi[s] = -1;
       if (i < M && e_hi >= 0 && e_lo <= 7) {
-        const u32x4 v = *reinterpret_cast<const u32x4 *>(&stage[r * SS + 8 * g]);
+        v[s] = *reinterpret_cast<const u32x4 *>(&stage[r * SS + 8 * g]);
         uint16_t *dst = Cb + (int64_t)i * W + (c8 - i + w);
         if (e_lo <= 0 && e_hi >= 7) {
-          store_chunk<ALIGNED>(dst, v);
+          store_chunk<ALIGNED>(dst, v[s]);
+        } else if (e_lo > 0) {  // head piece: elements e_lo..7 (W >= 17, so it reaches the chunk's end)
+          if (ALIGNED && rw > 0 && (r > 0 || seam_across_waves))
+            *reinterpret_cast<u32x4 *>(&seam[rw * 8]) = v[s];
+          else
+            store_chunk_elements(dst, v[s], e_lo, 7);
         } else {
-#pragma unroll
-          for (int e = 0; e < 8; ++e)
-            if (e >= e_lo && e <= e_hi) dst[e] = (uint16_t)(v[e >> 1] >> (16 * (e & 1)));
+          tail_hi[s] = e_hi;
         }
       }
     }
     wave_sync_lds();
-    if (k + 1 < nk) stash(k + 1);
+    // pass B: tail pieces pick up the head piece of the row below and leave as whole chunks.
+#pragma unroll
+    for (int s = 0; s < 4; ++s) {
+      if (tail_hi[s] >= 0) {
+        const int q = lane + 64 * s, r = q >> 3, g = q & 7;
+        const int rw = wave * 32 + r, i = i0 + rw;
+        const int c8 = cb + 8 * g;
+        uint16_t *dst = Cb + (int64_t)i * W + (c8 - i + w);
+        if (ALIGNED && rw + 1 < TM && i + 1 < M && (r < 31 || seam_across_waves)) {
+          const u32x4 head = *reinterpret_cast<const u32x4 *>(&seam[(rw + 1) * 8]);
+          const u32x4 mine_part = keep_range(v[s], 0, tail_hi[s]);
+          const u32x4 head_part = keep_range(head, tail_hi[s] + 1, 7);
+          u32x4 merged = {mine_part[0] | head_part[0], mine_part[1] | head_part[1], mine_part[2] | head_part[2],
+                          mine_part[3] | head_part[3]};
+          store_chunk<true>(dst, merged);
+        } else {
+          store_chunk_elements(dst, v[s], 0, tail_hi[s]);
+        }
+      }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    stash(k + 1, next);
     __syncthreads();
+  };
+
+#pragma unroll
+  for (int s = 0; s < PF; ++s) fetch(s, y_reg[s]);
+  __builtin_amdgcn_sched_barrier(0);
+  stash(0, y_reg[0]);
+  __syncthreads();
+  static_assert(PF == 2, "the slot chain below is written out for two register sets");
+  for (int k = 0;;) {
+    slot(k, y_reg[0], y_reg[1]);
+    if (++k >= nk) break;
+    slot(k, y_reg[1], y_reg[0]);
+    if (++k >= nk) break;
   }
 }
 
