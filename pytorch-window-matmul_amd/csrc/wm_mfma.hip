@@ -241,20 +241,35 @@ __global__ __launch_bounds__(kThreads, 2) void mfma_p2_kernel(const uint16_t *__
       yr[s] = fetch_row_chunk(Yb + (int64_t)c * ysr + y_h[s], Y, (y_r[s] < KC) & (c >= 0) & (c <= c_hi));
     }
   };
+  // A chunk is interior when every element of its T tile and every Y row is valid; its masks
+  // are skipped (most chunks of a wide band).
+  const int in_lo = rows == TM ? max(i0 + TM - 1 - w, 0) : 0x7fffffff, in_hi = min(i0 + w, c_hi);
   auto stash = [&](int k, const u32x4(&tr)[4], const u32x4(&yr)[NT]) {  // mask, then to LDS buffer k & 1
     const int cb = c_start + k * KC, buf = k & 1;
+    u32x4 tv[4], yv[NT];
+#pragma unroll
+    for (int s = 0; s < 4; ++s) tv[s] = pin(tr[s]);
+#pragma unroll
+    for (int s = 0; s < NT; ++s) yv[s] = pin(yr[s]);
+    if (!(cb >= in_lo && cb + KC - 1 <= in_hi)) {
+#pragma unroll
+      for (int s = 0; s < 4; ++s) {
+        const int c8 = cb + 8 * ((tid + kThreads * s) & 7);
+        tv[s] = mask_band_chunk(tv[s], t_lo[s] - c8, t_hi[s] - c8);
+      }
+#pragma unroll
+      for (int s = 0; s < NT; ++s) {
+        const int c = cb + y_r[s];
+        yv[s] = mask_row_chunk(yv[s], (c >= 0) & (c <= c_hi));
+      }
+    }
 #pragma unroll
     for (int s = 0; s < 4; ++s) {
       const int q = tid + kThreads * s;
-      const int c8 = cb + 8 * (q & 7);
-      *reinterpret_cast<u32x4 *>(&t_lds[buf][(q >> 3) * ST + (q & 7) * 8]) =
-          mask_band_chunk(pin(tr[s]), t_lo[s] - c8, t_hi[s] - c8);
+      *reinterpret_cast<u32x4 *>(&t_lds[buf][(q >> 3) * ST + (q & 7) * 8]) = tv[s];
     }
 #pragma unroll
-    for (int s = 0; s < NT; ++s) {
-      const int c = cb + y_r[s];
-      *reinterpret_cast<u32x4 *>(&y_lds[buf][y_r[s] * SY + y_h[s]]) = mask_row_chunk(pin(yr[s]), (c >= 0) & (c <= c_hi));
-    }
+    for (int s = 0; s < NT; ++s) *reinterpret_cast<u32x4 *>(&y_lds[buf][y_r[s] * SY + y_h[s]]) = yv[s];
   };
 
   f32x16 acc[NT];
@@ -292,12 +307,14 @@ __global__ __launch_bounds__(kThreads, 2) void mfma_p2_kernel(const uint16_t *__
     __syncthreads();
   };
   static_assert(PF == 2, "the slot chain below is written out for two register sets");
-  for (int k = 0;;) {
+  // Slots run in pairs inside the loop, an odd last one after it: one loop exit, one back edge,
+  // so the state of the memory counters is the same on every way into a slot.
+  int k = 0;
+  for (; k + 1 < nk; k += 2) {
     slot(k, t_reg[0], y_reg[0], t_reg[1], y_reg[1]);
-    if (++k >= nk) break;
-    slot(k, t_reg[1], y_reg[1], t_reg[0], y_reg[0]);
-    if (++k >= nk) break;
+    slot(k + 1, t_reg[1], y_reg[1], t_reg[0], y_reg[0]);
   }
+  if (k < nk) slot(k, t_reg[0], y_reg[0], t_reg[1], y_reg[1]);
 
   // acc[nt][v]: h = 32 nt + 8 (v / 4) + 4 (lane / 32) + v % 4, row = wave * 32 + lane % 32
   const int i = i0 + wave * 32 + (lane & 31);
@@ -370,19 +387,33 @@ __global__ __launch_bounds__(kThreads, 2) void mfma_p3_kernel(const uint16_t *__
       yr[s] = fetch_row_chunk(Yb + (int64_t)r * ysr + y_h[s], Y, (y_r[s] < KC) & (r <= r_hi));
     }
   };
+  // Interior chunk: all KC band rows exist and each covers all TM columns of the block.
+  const bool block_whole = c0 >= 0 && c0 + TM <= M;
   auto stash = [&](int k, const u32x4(&tr)[4], const u32x4(&yr)[NT]) {  // mask, then to LDS buffer k & 1
     const int rb = r_lo + k * KC, buf = k & 1;
+    u32x4 tv[4], yv[NT];
+#pragma unroll
+    for (int s = 0; s < 4; ++s) tv[s] = pin(tr[s]);
+#pragma unroll
+    for (int s = 0; s < NT; ++s) yv[s] = pin(yr[s]);
+    if (!(block_whole && rb + KC - 1 <= r_hi && rb + KC - 1 - w <= c0 && c0 + TM - 1 <= rb + w)) {
+#pragma unroll
+      for (int s = 0; s < 4; ++s) {
+        const int q = tid + kThreads * s;
+        const int r = rb + (q >> 4), c8 = c0 + 8 * (q & 15);
+        const int lo = max(r - w, 0), hi = r <= r_hi ? min(r + w, M - 1) : -1;
+        tv[s] = mask_band_chunk(tv[s], lo - c8, hi - c8);
+      }
+#pragma unroll
+      for (int s = 0; s < NT; ++s) yv[s] = mask_row_chunk(yv[s], rb + y_r[s] <= r_hi);
+    }
 #pragma unroll
     for (int s = 0; s < 4; ++s) {
       const int q = tid + kThreads * s;
-      const int r = rb + (q >> 4), c8 = c0 + 8 * (q & 15);
-      const int lo = max(r - w, 0), hi = r <= r_hi ? min(r + w, M - 1) : -1;
-      *reinterpret_cast<u32x4 *>(&t_lds[buf][(q >> 4) * ST + (q & 15) * 8]) =
-          mask_band_chunk(pin(tr[s]), lo - c8, hi - c8);
+      *reinterpret_cast<u32x4 *>(&t_lds[buf][(q >> 4) * ST + (q & 15) * 8]) = tv[s];
     }
 #pragma unroll
-    for (int s = 0; s < NT; ++s)
-      *reinterpret_cast<u32x4 *>(&y_lds[buf][y_r[s] * SY + y_h[s]]) = mask_row_chunk(pin(yr[s]), rb + y_r[s] <= r_hi);
+    for (int s = 0; s < NT; ++s) *reinterpret_cast<u32x4 *>(&y_lds[buf][y_r[s] * SY + y_h[s]]) = yv[s];
   };
 
   f32x16 acc[NT];
@@ -415,12 +446,14 @@ __global__ __launch_bounds__(kThreads, 2) void mfma_p3_kernel(const uint16_t *__
     __syncthreads();
   };
   static_assert(PF == 2, "the slot chain below is written out for two register sets");
-  for (int k = 0;;) {
+  // Slots run in pairs inside the loop, an odd last one after it: one loop exit, one back edge,
+  // so the state of the memory counters is the same on every way into a slot.
+  int k = 0;
+  for (; k + 1 < nk; k += 2) {
     slot(k, t_reg[0], y_reg[0], t_reg[1], y_reg[1]);
-    if (++k >= nk) break;
-    slot(k, t_reg[1], y_reg[1], t_reg[0], y_reg[0]);
-    if (++k >= nk) break;
+    slot(k + 1, t_reg[1], y_reg[1], t_reg[0], y_reg[0]);
   }
+  if (k < nk) slot(k, t_reg[0], y_reg[0], t_reg[1], y_reg[1]);
 
   const int c = c0 + wave * 32 + (lane & 31);
   if (c >= 0 && c < M) {
@@ -612,12 +645,12 @@ __global__ __launch_bounds__(kThreads, 2) void mfma_p1_kernel(const uint16_t *__
   stash(0, y_reg[0]);
   __syncthreads();
   static_assert(PF == 2, "the slot chain below is written out for two register sets");
-  for (int k = 0;;) {
+  int k = 0;
+  for (; k + 1 < nk; k += 2) {
     slot(k, y_reg[0], y_reg[1]);
-    if (++k >= nk) break;
-    slot(k, y_reg[1], y_reg[0]);
-    if (++k >= nk) break;
+    slot(k + 1, y_reg[1], y_reg[0]);
   }
+  if (k < nk) slot(k, y_reg[0], y_reg[1]);
 }
 
 // ------------------------------------------------------------------------------------------
