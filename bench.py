@@ -58,18 +58,20 @@ def kernel_bytes(B, M, N, w, es):
 
 
 def time_gpu(fn, iters, warmup):
+    """Mean duration of one launch, each launch bracketed by its own pair of HIP events on the
+    current stream (so that the gap between dependent launches is not counted as kernel time)."""
     import torch
 
     for _ in range(warmup):
         fn()
-    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    pairs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(iters)]
     torch.cuda.synchronize()
-    start.record()
-    for _ in range(iters):
+    for start, stop in pairs:
+        start.record()
         fn()
-    stop.record()
-    stop.synchronize()
-    return start.elapsed_time(stop) / iters  # ms
+        stop.record()
+    torch.cuda.synchronize()
+    return sum(a.elapsed_time(b) for a, b in pairs) / iters  # ms
 
 
 def cpu_baseline(cfg, seconds_budget=20.0):
