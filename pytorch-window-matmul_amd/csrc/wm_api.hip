@@ -7,7 +7,7 @@ namespace {
 
 int check_common(int64_t B, int64_t M, int64_t N, int64_t w, int dtype, unsigned flags) {
   if (dtype < WM_DTYPE_F32 || dtype > WM_DTYPE_F64) return WM_ERR_BAD_DTYPE;
-  if (flags & ~(WM_FLAG_FORCE_STRIDED | WM_FLAG_NO_ALIGNED_BAND)) return WM_ERR_BAD_FLAGS;
+  if (flags & ~(WM_FLAG_FORCE_STRIDED | WM_FLAG_NO_ALIGNED_BAND | WM_FLAG_NO_NARROW_BAND)) return WM_ERR_BAD_FLAGS;
   const int64_t lim = 0x7fffffff;
   if (B < 0 || M < 0 || N < 0 || w < 0) return WM_ERR_BAD_SHAPE;
   if (B > lim || M > lim || N > lim || w > (lim - 1) / 2) return WM_ERR_BAD_SHAPE;
@@ -26,20 +26,25 @@ int to_status(hipError_t err) {
 typedef bool (*mfma_fn)(const Problem &, const View &, const View &, const View &, hipError_t *);
 typedef hipError_t (*strided_fn)(const Problem &, const View &, const View &, const View &);
 
-int run_primitive(mfma_fn fast, strided_fn slow, const Problem &p, const View &a, const View &y, const View &c) {
+// Kernel choice per primitive: narrow-band family, else wide-band MFMA family, else strided.
+int run_primitive(mfma_fn narrow, mfma_fn fast, strided_fn slow, const Problem &p, const View &a, const View &y,
+                  const View &c) {
   hipError_t err = hipSuccess;
-  if (!(p.flags & WM_FLAG_FORCE_STRIDED) && fast(p, a, y, c, &err)) return to_status(err);
+  if (!(p.flags & WM_FLAG_FORCE_STRIDED)) {
+    if (narrow && !(p.flags & WM_FLAG_NO_NARROW_BAND) && narrow(p, a, y, c, &err)) return to_status(err);
+    if (fast(p, a, y, c, &err)) return to_status(err);
+  }
   return to_status(slow(p, a, y, c));
 }
 
 int p1(const Problem &p, const View &x, const View &y, const View &c) {
-  return run_primitive(try_launch_mfma_p1, launch_strided_p1, p, x, y, c);
+  return run_primitive(try_launch_small_p1, try_launch_mfma_p1, launch_strided_p1, p, x, y, c);
 }
 int p2(const Problem &p, const View &a, const View &y, const View &c) {
-  return run_primitive(try_launch_mfma_p2, launch_strided_p2, p, a, y, c);
+  return run_primitive(try_launch_small_p2, try_launch_mfma_p2, launch_strided_p2, p, a, y, c);
 }
 int p3(const Problem &p, const View &a, const View &y, const View &c) {
-  return run_primitive(try_launch_mfma_p3, launch_strided_p3, p, a, y, c);
+  return run_primitive(nullptr, try_launch_mfma_p3, launch_strided_p3, p, a, y, c);
 }
 
 }  // namespace
@@ -105,9 +110,15 @@ int wm_unwindow_matmul_backward(const wm_operand *a, const wm_operand *v, const 
 const char *wm_kernel_choice(int op, int64_t B, int64_t M, int64_t N, int64_t w, int dtype, int fast,
                              unsigned flags) {
   if (op < 1 || op > 3) return "invalid";
-  if (!(flags & WM_FLAG_FORCE_STRIDED) && fast && mfma_supports(op, B, M, N, w, dtype)) {
-    static const char *names[] = {"mfma_p1", "mfma_p2", "mfma_p3"};
-    return names[op - 1];
+  if (!(flags & WM_FLAG_FORCE_STRIDED) && fast) {
+    if (!(flags & WM_FLAG_NO_NARROW_BAND) && small_supports(op, M, N, w, dtype)) {
+      static const char *names[] = {"narrow_p1", "narrow_p2", "narrow_p3"};
+      return names[op - 1];
+    }
+    if (mfma_supports(op, B, M, N, w, dtype)) {
+      static const char *names[] = {"mfma_p1", "mfma_p2", "mfma_p3"};
+      return names[op - 1];
+    }
   }
   static const char *names[] = {"strided_p1", "strided_p2", "strided_p3"};
   return names[op - 1];

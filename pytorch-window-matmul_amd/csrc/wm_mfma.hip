@@ -26,157 +26,10 @@
 // Masking is done on bits, never by multiplying with zero: invalid entries of an
 // input band are cleared before they reach LDS, and out-of-sequence entries of an
 // output band are stored as +0.0 whatever the operands hold.
-#include "wm_common.hpp"
-#include "wm_types.hpp"
+#include "wm_mfma_common.hpp"
 
 namespace wm {
 namespace {
-
-typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
-typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
-typedef float f32x16 __attribute__((ext_vector_type(16)));
-typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
-typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
-typedef short s16x4 __attribute__((ext_vector_type(4)));
-typedef float f32x2 __attribute__((ext_vector_type(2)));
-typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
-
-constexpr int kThreads = 256;
-constexpr int TM = 128;  // rows per workgroup (32 per wave)
-constexpr int KC = 64;   // chunk length along the contraction (P2, P3) / dense columns (P1)
-constexpr int PF = 2;    // chunks requested ahead of the one being multiplied (P2, P3)
-
-struct __attribute__((packed, aligned(2))) Chunk2 {
-  u32x4 v;
-};
-
-template <bool ALIGNED>
-__device__ __forceinline__ u32x4 load_chunk(const uint16_t *p) {
-  if (ALIGNED) return *reinterpret_cast<const u32x4 *>(p);
-  return reinterpret_cast<const Chunk2 *>(p)->v;
-}
-template <bool ALIGNED>
-__device__ __forceinline__ void store_chunk(uint16_t *p, u32x4 v) {
-  if (ALIGNED)
-    *reinterpret_cast<u32x4 *>(p) = v;
-  else
-    reinterpret_cast<Chunk2 *>(p)->v = v;
-}
-
-// Keeps elements e_lo..e_hi (inclusive, in 0..7) of a chunk of eight 16-bit values, clears the rest.
-__device__ __forceinline__ u32x4 keep_range(u32x4 v, int e_lo, int e_hi) {
-  u32x4 r;
-#pragma unroll
-  for (int d = 0; d < 4; ++d) {
-    const uint32_t lo = (2 * d >= e_lo && 2 * d <= e_hi) ? 0x0000ffffu : 0u;
-    const uint32_t hi = (2 * d + 1 >= e_lo && 2 * d + 1 <= e_hi) ? 0xffff0000u : 0u;
-    r[d] = v[d] & (lo | hi);
-  }
-  return r;
-}
-
-// Band chunk = 8 consecutive dense columns of one row of the skewed tile, of which only
-// elements [e_lo, e_hi] are valid.  Loading is split in two branch-free halves so that the
-// prefetch contains nothing but loads (a use of the loaded value, or a load inside a branch,
-// makes the compiler wait for memory on the spot and serialises the pipeline):
-//   fetch_band_chunk  issues the 16-byte load; from `safe` (any readable, suitably aligned
-//                     address) when no element is valid;
-//   mask_band_chunk   clears the invalid elements, later, when the chunk goes to LDS.
-// A partially valid chunk is read whole: with w >= 7 the up-to-7 elements on either side of a
-// row's valid range are band entries of the same or the neighbouring row, i.e. inside the
-// tensor (the kernels are only used for w >= 8).
-__device__ __forceinline__ bool band_chunk_any(int e_lo, int e_hi) { return (e_hi >= 0) & (e_lo <= 7) & (e_lo <= e_hi); }
-template <bool ALIGNED>
-__device__ __forceinline__ u32x4 fetch_band_chunk(const uint16_t *p, const uint16_t *safe, int e_lo, int e_hi) {
-  return load_chunk<ALIGNED>(band_chunk_any(e_lo, e_hi) ? p : safe);
-}
-__device__ __forceinline__ u32x4 mask_band_chunk(u32x4 v, int e_lo, int e_hi) {
-  return keep_range(v, band_chunk_any(e_lo, e_hi) ? e_lo : 8, e_hi);
-}
-
-// Row chunk of a dense operand; rows outside the sequence are fetched from `safe` and zeroed later.
-__device__ __forceinline__ u32x4 fetch_row_chunk(const uint16_t *p, const uint16_t *safe, bool valid) {
-  return *reinterpret_cast<const u32x4 *>(valid ? p : safe);
-}
-__device__ __forceinline__ u32x4 mask_row_chunk(u32x4 v, bool valid) {
-  const uint32_t m = valid ? 0xffffffffu : 0u;
-  u32x4 r = {v[0] & m, v[1] & m, v[2] & m, v[3] & m};
-  return r;
-}
-__device__ __forceinline__ u32x4 load_row_chunk(const uint16_t *p, const uint16_t *safe, bool valid) {
-  return mask_row_chunk(fetch_row_chunk(p, safe, valid), valid);
-}
-
-template <typename T>
-struct Mma;
-template <>
-struct Mma<bf16_t> {
-  static __device__ __forceinline__ f32x16 run(u32x4 a, u32x4 b, f32x16 c) {
-    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c,
-                                                   0, 0, 0);
-  }
-  static __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
-    f32x2 v = {lo, hi};
-    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2));  // v_cvt_pk_bf16_f32, RNE
-  }
-};
-template <>
-struct Mma<f16_t> {
-  static __device__ __forceinline__ f32x16 run(u32x4 a, u32x4 b, f32x16 c) {
-    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0,
-                                                  0, 0);
-  }
-  static __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
-    const uint16_t l = __builtin_bit_cast(uint16_t, (_Float16)lo), h = __builtin_bit_cast(uint16_t, (_Float16)hi);
-    return (uint32_t)l | ((uint32_t)h << 16);
-  }
-};
-
-// Operand fetch for a matrix stored in LDS as Mat[k][x] (x contiguous) when the MFMA
-// wants, per lane, x = lane % 32 and eight consecutive k starting at 8 * (lane / 32).
-// ds_read_b64_tr_b16 works on 16-lane groups: lane s of a group supplies the address of
-// 4 consecutive x in row s/4 and receives, for x = its own position in the group, the
-// 4 values of rows 0..3.  Two such reads cover the 8 k's.
-__device__ __forceinline__ u32x4 lds_read_transposed(const uint16_t *mat, int stride, int k0, int x0, int lane) {
-  const int s = lane & 15, grp = lane >> 4;
-  const int xb = x0 + 16 * (grp & 1) + 4 * (s & 3);
-  const int kb = k0 + 8 * (grp >> 1) + (s >> 2);
-  typedef s16x4 __attribute__((address_space(3))) * lds_ptr;
-  const uint16_t *p0 = mat + kb * stride + xb;
-  const uint16_t *p1 = p0 + 4 * stride;
-  const s16x4 a = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(p0));
-  const s16x4 b = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(p1));
-  const u32x2 ua = __builtin_bit_cast(u32x2, a), ub = __builtin_bit_cast(u32x2, b);
-  u32x4 r = {ua[0], ua[1], ub[0], ub[1]};
-  return r;
-}
-
-// Pins a prefetched register at this point of the program: the compiler may not use the value
-// (and therefore may not wait for its load) any earlier than here.
-__device__ __forceinline__ u32x4 pin(u32x4 v) {
-  asm volatile("" : "+v"(v));
-  return v;
-}
-
-__device__ __forceinline__ void wave_sync_lds() {
-  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-  __builtin_amdgcn_wave_barrier();
-  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-}
-
-// Workgroup -> (batch, block).  Workgroups are dealt round-robin to the 8 XCDs, each with
-// its own L2; all blocks of one batch element are given to one XCD so that neighbouring
-// blocks find the rows they share (the +-w halo) in that L2.
-__device__ __forceinline__ bool decode_block(int nblk, int B, int *b, int *blk) {
-  const int id = blockIdx.x, xcd = id & 7, slot = id >> 3;
-  *b = (slot / nblk) * 8 + xcd;
-  *blk = slot % nblk;
-  return *b < B;
-}
-
-// Row stride (elements) of matrices read with lds_read_transposed: the byte stride must be
-// 32 or 96 (mod 128) so that the 4 rows touched by a 16-lane group fall into distinct banks.
-constexpr int lds_stride_tr(int n_padded) { return n_padded + 16; }
 
 // ------------------------------------------------------------------------------------------
 // P2: C[b,i,h] = sum_c T[i][c] * Y[b,c,h]
@@ -475,14 +328,6 @@ __global__ __launch_bounds__(kThreads, 2) void mfma_p3_kernel(const uint16_t *__
 // ------------------------------------------------------------------------------------------
 // P1: band[b,i,c-i+w] = sum_h X[b,i,h] * Y[b,c,h]   (+0.0 where c is outside the sequence)
 // ------------------------------------------------------------------------------------------
-// Element-wise store of elements [e_lo, e_hi] of a chunk (the slow path for chunk pieces that
-// cannot be completed with their neighbour row's piece).
-__device__ __forceinline__ void store_chunk_elements(uint16_t *dst, u32x4 v, int e_lo, int e_hi) {
-#pragma unroll
-  for (int e = 0; e < 8; ++e)
-    if (e >= e_lo && e <= e_hi) dst[e] = (uint16_t)(v[e >> 1] >> (16 * (e & 1)));
-}
-
 template <typename T, int NK, bool ALIGNED>  // NK = N / 16
 __global__ __launch_bounds__(kThreads, 2) void mfma_p1_kernel(const uint16_t *__restrict__ X,
                                                               const uint16_t *__restrict__ Y,

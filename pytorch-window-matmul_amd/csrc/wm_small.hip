@@ -1,0 +1,340 @@
+// Narrow-band kernels (w <= 32) for 16-bit storage on gfx950.
+//
+// With a narrow band the whole band of a block of rows is small (256 rows x 17 entries =
+// 8.7 KB at w = 8), the op is a pure stream over Q/K (P1) or V/O (P2), and the dense tiles of
+// the wide-band kernels would waste most of their work and all of their barriers.  Here a
+// wave owns 64 (or 32) consecutive rows and everything it needs:
+//
+//   P1  the wave loads its rows of X and the rows [r0-w, r0+64+w) of Y straight from HBM
+//       into MFMA operand registers (no LDS, no barrier), forms the 32x32 tiles that touch
+//       the band, and scatters the band entries into a flat LDS image of the workgroup's
+//       band rows, which then leaves as aligned 16-byte stores.
+//   P2  the workgroup copies its band rows flat into LDS (aligned 16-byte loads) and the
+//       rows [i0-w, i0+rows+w) of Y row-major into LDS; each wave then multiplies its rows:
+//       the skewed tile is read back with ds_read_b128 (the flat image keeps 8-column groups
+//       16-byte aligned when w % 4 == 0) and masked on bits, Y is read transposed with
+//       ds_read_b64_tr_b16.
+//
+// One workgroup barrier per kernel; results are written exactly once; out-of-sequence band
+// entries are stored as +0.0.
+#include "wm_mfma_common.hpp"
+
+namespace wm {
+namespace {
+
+constexpr int SMALL_MAX_W = 32;
+
+// ------------------------------------------------------------------------------------------
+// P1 narrow: band[b,i,j] = sum_h X[b,i,h] * Y[b,i+j-w,h]
+// ------------------------------------------------------------------------------------------
+template <typename T, int NK, int NMT>  // N = 16 NK; NMT 32-column tiles cover 64 + 2w columns
+__global__ __launch_bounds__(kThreads) void small_p1_kernel(const uint16_t *__restrict__ X,
+                                                            const uint16_t *__restrict__ Y,
+                                                            uint16_t *__restrict__ C, int B, int M, int w, int nblk,
+                                                            int64_t xsb, int64_t xsr, int64_t ysb, int64_t ysr,
+                                                            int64_t csb) {
+  constexpr int ROWS = 256;  // band rows per workgroup, 64 per wave
+  extern __shared__ __attribute__((aligned(16))) uint16_t flat[];  // 8 + ROWS * W (+ slack) elements
+
+  int b, blk;
+  if (!decode_block(nblk, B, &b, &blk)) return;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int W = 2 * w + 1;
+  const int i0 = blk * ROWS, iw0 = i0 + 64 * wave;
+  const int nrows = min(ROWS, M - i0);
+  uint16_t *Cb = C + (int64_t)b * csb + (int64_t)i0 * W;  // first band entry of this workgroup
+  const int delta = (int)((reinterpret_cast<uintptr_t>(Cb) >> 1) & 7);  // elements past a 16-byte boundary
+
+  if (iw0 < M) {
+    // operands straight into registers: all loads are issued before the first use
+    u32x4 xop[2][NK], yop[NMT][NK];
+    const uint16_t *Xb = X + (int64_t)b * xsb, *Yb = Y + (int64_t)b * ysb;
+#pragma unroll
+    for (int nt = 0; nt < 2; ++nt) {
+      const int i = iw0 + 32 * nt + (lane & 31);
+#pragma unroll
+      for (int ks = 0; ks < NK; ++ks)
+        xop[nt][ks] = fetch_row_chunk(Xb + (int64_t)i * xsr + 16 * ks + 8 * (lane >> 5), X, i < M);
+    }
+#pragma unroll
+    for (int mt = 0; mt < NMT; ++mt) {
+      const int c = iw0 - w + 32 * mt + (lane & 31);
+#pragma unroll
+      for (int ks = 0; ks < NK; ++ks)
+        yop[mt][ks] = fetch_row_chunk(Yb + (int64_t)c * ysr + 16 * ks + 8 * (lane >> 5), Y, (c >= 0) & (c < M));
+    }
+#pragma unroll
+    for (int nt = 0; nt < 2; ++nt) {
+      const int i = iw0 + 32 * nt + (lane & 31);
+#pragma unroll
+      for (int ks = 0; ks < NK; ++ks) xop[nt][ks] = mask_row_chunk(xop[nt][ks], i < M);
+    }
+#pragma unroll
+    for (int mt = 0; mt < NMT; ++mt) {
+      const int c = iw0 - w + 32 * mt + (lane & 31);
+#pragma unroll
+      for (int ks = 0; ks < NK; ++ks) yop[mt][ks] = mask_row_chunk(yop[mt][ks], (c >= 0) & (c < M));
+    }
+
+    uint16_t *img = flat + delta + (64 * wave) * W;  // this wave's 64 rows of the flat band image
+#pragma unroll
+    for (int nt = 0; nt < 2; ++nt) {
+#pragma unroll
+      for (int mt = 0; mt < NMT; ++mt) {
+        // tile columns c_rel in [32 mt, 32 mt + 32), rows r_rel in [32 nt, 32 nt + 32); j = c_rel - r_rel
+        if (32 * (mt - nt) + 31 < 0 || 32 * (mt - nt) - 31 > 2 * w) continue;
+        f32x16 acc;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[v] = 0.f;
+#pragma unroll
+        for (int ks = 0; ks < NK; ++ks) acc = Mma<T>::run(yop[mt][ks], xop[nt][ks], acc);
+        // acc[v]: c_rel = 32 mt + 8 (v / 4) + 4 (lane / 32) + v % 4, r_rel = 32 nt + lane % 32
+        const int r_rel = 32 * nt + (lane & 31);
+        uint16_t *row = img + r_rel * W;
+#pragma unroll
+        for (int q4 = 0; q4 < 4; ++q4) {
+          const int c_rel = 32 * mt + 8 * q4 + 4 * (lane >> 5);
+          const int j = c_rel - r_rel;     // band column of the first of 4 consecutive entries
+          const int c = iw0 - w + c_rel;   // their sequence positions c .. c + 3
+          const uint32_t lo = Mma<T>::pack2(acc[4 * q4], acc[4 * q4 + 1]);
+          const uint32_t hi = Mma<T>::pack2(acc[4 * q4 + 2], acc[4 * q4 + 3]);
+          // entries outside the sequence are +0.0 by definition, whatever X holds
+          if (j >= 0 && j <= 2 * w) row[j] = (c >= 0 && c < M) ? (uint16_t)lo : (uint16_t)0;
+          if (j + 1 >= 0 && j + 1 <= 2 * w) row[j + 1] = (c + 1 >= 0 && c + 1 < M) ? (uint16_t)(lo >> 16) : (uint16_t)0;
+          if (j + 2 >= 0 && j + 2 <= 2 * w) row[j + 2] = (c + 2 >= 0 && c + 2 < M) ? (uint16_t)hi : (uint16_t)0;
+          if (j + 3 >= 0 && j + 3 <= 2 * w) row[j + 3] = (c + 3 >= 0 && c + 3 < M) ? (uint16_t)(hi >> 16) : (uint16_t)0;
+        }
+      }
+    }
+  }
+  __syncthreads();
+
+  // flat image -> HBM: chunk q holds image elements [8q, 8q+8), i.e. band elements [8q - delta, ...)
+  const int n_el = nrows * W;
+  const int chunks = (delta + n_el + 7) >> 3;
+  for (int q = tid; q < chunks; q += kThreads) {
+    const u32x4 v = *reinterpret_cast<const u32x4 *>(flat + 8 * q);
+    const int first = 8 * q - delta;  // band element index of the chunk's element 0
+    uint16_t *dst = Cb + first;
+    if (first >= 0 && first + 8 <= n_el)
+      *reinterpret_cast<u32x4 *>(dst) = v;
+    else
+      store_chunk_elements(dst, v, -first, n_el - 1 - first);  // only the workgroup's first and last chunk
+  }
+}
+
+// ------------------------------------------------------------------------------------------
+// P2 narrow: C[b,i,h] = sum_j A[b,i,j] * Y[b,i+j-w,h]      (w % 4 == 0)
+// ------------------------------------------------------------------------------------------
+template <typename T, int NT, int RW>  // N <= 32 NT; RW rows per wave (64 or 32)
+__global__ __launch_bounds__(kThreads) void small_p2_kernel(const uint16_t *__restrict__ A,
+                                                            const uint16_t *__restrict__ Y,
+                                                            uint16_t *__restrict__ C, int B, int M, int N, int w,
+                                                            int nblk, int64_t asb, int64_t ysb, int64_t ysr,
+                                                            int64_t csb, int64_t csr) {
+  constexpr int ROWS = 4 * RW;
+  constexpr int SY = lds_stride_tr(32 * NT);
+  extern __shared__ __attribute__((aligned(16))) uint16_t lds[];
+  const int W = 2 * w + 1;
+  const int a_elems = ((ROWS * W + 16 + 7) >> 3) << 3;  // flat band image, whole 16-byte chunks
+  uint16_t *aimg = lds;
+  uint16_t *yimg = lds + a_elems;  // rows c = cv0 .. cv0 + ROWS + 2w + 32, stride SY; all initialised
+
+  int b, blk;
+  if (!decode_block(nblk, B, &b, &blk)) return;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int i0 = blk * ROWS;
+  const int nrows = min(ROWS, M - i0);
+  const uint16_t *Ab = A + (int64_t)b * asb + (int64_t)i0 * W;
+  const uint16_t *Yb = Y + (int64_t)b * ysb;
+  const int delta = (int)((reinterpret_cast<uintptr_t>(Ab) >> 1) & 7);
+
+  // band rows, flat: aligned chunks; the first and last chunk may hold neighbours' entries
+  // (inside the tensor's pages: aligned 16-byte chunks never straddle a page)
+  const int n_el = nrows * W;
+  const int chunks = (delta + n_el + 7) >> 3;
+  // Y rows, row-major, zero outside the sequence
+  const int cv0 = i0 - w - 8;
+  const int yrows = ROWS + 2 * w + 32, ncg = N >> 3;  // every row a 16-column step can reach
+  const int ychunks = yrows * ncg;
+  // loads go out in batches of 8 per thread before any of them is used
+  constexpr int BATCH = 8;
+  for (int base = 0; base < chunks + ychunks; base += BATCH * kThreads) {
+    u32x4 reg[BATCH];
+#pragma unroll
+    for (int s = 0; s < BATCH; ++s) {
+      const int q = base + s * kThreads + tid;
+      const int qy = q - chunks, yr = qy / ncg, hg = qy - yr * ncg, c = cv0 + yr;
+      const uint16_t *src = q < chunks ? Ab - delta + 8 * q : Yb + (int64_t)c * ysr + 8 * hg;
+      const bool ok = q < chunks || (q < chunks + ychunks && c >= 0 && c < M);
+      reg[s] = *reinterpret_cast<const u32x4 *>(ok ? src : A);
+    }
+#pragma unroll
+    for (int s = 0; s < BATCH; ++s) {
+      const int q = base + s * kThreads + tid;
+      const int qy = q - chunks, yr = qy / ncg, hg = qy - yr * ncg, c = cv0 + yr;
+      if (q < chunks)
+        *reinterpret_cast<u32x4 *>(aimg + 8 * q) = reg[s];
+      else if (q < chunks + ychunks)
+        *reinterpret_cast<u32x4 *>(yimg + yr * SY + 8 * hg) = mask_row_chunk(reg[s], (c >= 0) & (c < M));
+    }
+  }
+  __syncthreads();
+
+  const int nks = (32 + 2 * w + delta + 15) >> 4;  // 16-column steps covering one 32-row tile's band
+  u32x2 outp[RW / 32][NT][4];
+#pragma unroll
+  for (int nt = 0; nt < RW / 32; ++nt) {
+    const int r0 = RW * wave + 32 * nt;  // first row of the tile, relative to i0 (multiple of 32)
+    const int r = lane & 31, i = i0 + r0 + r;
+    f32x16 acc[NT];
+#pragma unroll
+    for (int t = 0; t < NT; ++t)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[t][v] = 0.f;
+    // dense columns start at c_al = i0 + r0 - w - delta, which makes every 8-column group of every
+    // row an aligned chunk of the flat image: element index (r0 + r) 2w + r0 + 16 ks + 8 kg
+    const uint16_t *trow = aimg + (r0 + r) * 2 * w + r0 + 8 * (lane >> 5);
+    for (int ks = 0; ks < nks; ++ks) {
+      const int off = 16 * ks + 8 * (lane >> 5);    // column offset of this lane's group from c_al
+      const int c_g = i0 + r0 - w - delta + off;     // sequence position of its first element
+      u32x4 bop = *reinterpret_cast<const u32x4 *>(trow + 16 * ks);
+      // element e is band column j = off + e - delta - r of row i: valid iff 0 <= j <= 2w and 0 <= c < M
+      const int e_lo = max(delta + r - off, -c_g);
+      const int e_hi = i < M ? min(2 * w + delta + r - off, M - 1 - c_g) : -1;
+      bop = mask_band_chunk(bop, e_lo, e_hi);
+      const int k0 = r0 - delta + 8 + 16 * ks;  // row of yimg holding sequence position c_al + 16 ks
+#pragma unroll
+      for (int t = 0; t < NT; ++t) {
+        const u32x4 aop = lds_read_transposed(yimg, SY, k0, 32 * t, lane);
+        acc[t] = Mma<T>::run(aop, bop, acc[t]);
+      }
+    }
+    // park the tile's result in registers until every wave is done with the LDS images
+#pragma unroll
+    for (int t = 0; t < NT; ++t)
+#pragma unroll
+      for (int q4 = 0; q4 < 4; ++q4) {
+        outp[nt][t][q4][0] = Mma<T>::pack2(acc[t][4 * q4], acc[t][4 * q4 + 1]);
+        outp[nt][t][q4][1] = Mma<T>::pack2(acc[t][4 * q4 + 2], acc[t][4 * q4 + 3]);
+      }
+  }
+  // results leave through LDS as row-contiguous 16-byte stores (whole 128-byte lines) instead
+  // of 8 bytes per lane scattered over 32 rows; the staging area reuses the images
+  __syncthreads();
+  constexpr int SO = 32 * NT + 8;
+  uint16_t *stage = lds + wave * (RW * SO);
+#pragma unroll
+  for (int nt = 0; nt < RW / 32; ++nt)
+#pragma unroll
+    for (int t = 0; t < NT; ++t)
+#pragma unroll
+      for (int q4 = 0; q4 < 4; ++q4)
+        *reinterpret_cast<u32x2 *>(stage + (32 * nt + (lane & 31)) * SO + 32 * t + 8 * q4 + 4 * (lane >> 5)) =
+            outp[nt][t][q4];
+  wave_sync_lds();
+  const int per_row = N >> 3;  // 16-byte chunks per output row
+  for (int q = lane; q < RW * per_row; q += 64) {
+    const int r = q / per_row, hg = q - r * per_row;
+    const int i = i0 + RW * wave + r;
+    if (i < M)
+      *reinterpret_cast<u32x4 *>(C + (int64_t)b * csb + (int64_t)i * csr + 8 * hg) =
+          *reinterpret_cast<const u32x4 *>(stage + r * SO + 8 * hg);
+  }
+}
+
+// ------------------------------------------------------------------------------------------
+// host side
+// ------------------------------------------------------------------------------------------
+bool small_shape_ok(int64_t M, int64_t N, int64_t w, int dtype) {
+  if (dtype != WM_DTYPE_BF16 && dtype != WM_DTYPE_F16) return false;
+  if (N < 16 || N > 128 || N % 16 != 0) return false;
+  return M >= 1 && M <= (1 << 30) && w >= 1 && w <= SMALL_MAX_W;
+}
+
+unsigned small_grid(int64_t B, int64_t nblk) { return (unsigned)(((B + 7) / 8) * 8 * nblk); }
+
+template <typename T>
+hipError_t launch_small_p1(const Problem &p, const View &x, const View &y, const View &c) {
+  const int nblk = (int)((p.M + 255) / 256);
+  const dim3 grid(small_grid(p.B, nblk)), block(kThreads);
+  const size_t lds = (size_t)(256 * (2 * p.w + 1) + 24) * 2;
+#define WM_SP1(NK, NMT)                                                                                        \
+  hipLaunchKernelGGL((small_p1_kernel<T, NK, NMT>), grid, block, lds, p.stream, (const uint16_t *)x.data,      \
+                     (const uint16_t *)y.data, (uint16_t *)c.data, (int)p.B, (int)p.M, (int)p.w, nblk, x.sb,   \
+                     x.sr, y.sb, y.sr, c.sb)
+#define WM_SP1_N(NMT)                    \
+  switch (p.N / 16) {                    \
+    case 1: WM_SP1(1, NMT); break;       \
+    case 2: WM_SP1(2, NMT); break;       \
+    case 3: WM_SP1(3, NMT); break;       \
+    case 4: WM_SP1(4, NMT); break;       \
+    case 5: WM_SP1(5, NMT); break;       \
+    case 6: WM_SP1(6, NMT); break;       \
+    case 7: WM_SP1(7, NMT); break;       \
+    default: WM_SP1(8, NMT); break;      \
+  }
+  if (p.w <= 16) {
+    WM_SP1_N(3)
+  } else {
+    WM_SP1_N(4)
+  }
+#undef WM_SP1_N
+#undef WM_SP1
+  return hipGetLastError();
+}
+
+template <typename T>
+hipError_t launch_small_p2(const Problem &p, const View &a, const View &y, const View &c) {
+  const int NT = (int)((p.N + 31) / 32);
+  const int RW = NT <= 2 ? 64 : 32;
+  const int rows = 4 * RW;
+  const int nblk = (int)((p.M + rows - 1) / rows);
+  const dim3 grid(small_grid(p.B, nblk)), block(kThreads);
+  const int64_t W = 2 * p.w + 1;
+  const size_t a_elems = (size_t)(((rows * W + 16 + 7) >> 3) << 3);
+  const size_t lds = (a_elems + (size_t)(rows + 2 * p.w + 32) * (32 * NT + 16)) * 2;
+#define WM_SP2(NT_, RW_)                                                                                       \
+  hipLaunchKernelGGL((small_p2_kernel<T, NT_, RW_>), grid, block, lds, p.stream, (const uint16_t *)a.data,     \
+                     (const uint16_t *)y.data, (uint16_t *)c.data, (int)p.B, (int)p.M, (int)p.N, (int)p.w, nblk, \
+                     a.sb, y.sb, y.sr, c.sb, c.sr)
+  switch (NT) {
+    case 1: WM_SP2(1, 64); break;
+    case 2: WM_SP2(2, 64); break;
+    case 3: WM_SP2(3, 32); break;
+    default: WM_SP2(4, 32); break;
+  }
+#undef WM_SP2
+  return hipGetLastError();
+}
+
+bool band_contiguous(const View &v, int64_t W) { return v.sc == 1 && v.sr == W && ((uintptr_t)v.data % 16) == 0; }
+
+}  // namespace
+
+bool small_supports(int op, int64_t M, int64_t N, int64_t w, int dtype) {
+  if (!small_shape_ok(M, N, w, dtype)) return false;
+  if (op == 1) return true;
+  if (op == 2) return w % 4 == 0;
+  return false;
+}
+
+bool try_launch_small_p1(const Problem &p, const View &x, const View &y, const View &c, hipError_t *err) {
+  if (!small_supports(1, p.M, p.N, p.w, p.dtype)) return false;
+  if (!fast_layout(x, p.dtype) || !fast_layout(y, p.dtype) || !band_contiguous(c, 2 * p.w + 1)) return false;
+  *err = p.dtype == WM_DTYPE_BF16 ? launch_small_p1<bf16_t>(p, x, y, c) : launch_small_p1<f16_t>(p, x, y, c);
+  return true;
+}
+
+bool try_launch_small_p2(const Problem &p, const View &a, const View &y, const View &c, hipError_t *err) {
+  if (!small_supports(2, p.M, p.N, p.w, p.dtype)) return false;
+  {  // the two LDS images must fit the default 64 KB dynamic limit; wider cases go to the wide-band family
+    const int64_t NT = (p.N + 31) / 32, rows = NT <= 2 ? 256 : 128, W = 2 * p.w + 1;
+    if ((rows * W + 24 + (rows + 2 * p.w + 32) * (32 * NT + 16)) * 2 > 65536) return false;
+  }
+  if (!band_contiguous(a, 2 * p.w + 1) || !fast_layout(y, p.dtype) || !fast_layout(c, p.dtype)) return false;
+  *err = p.dtype == WM_DTYPE_BF16 ? launch_small_p2<bf16_t>(p, a, y, c) : launch_small_p2<f16_t>(p, a, y, c);
+  return true;
+}
+
+}  // namespace wm

@@ -18,6 +18,7 @@ HEADER = os.path.join(REPO, "include", "window_matmul_hip.h")
 DTYPES = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2, torch.float64: 3}
 FORCE_STRIDED = 0x1
 NO_ALIGNED_BAND = 0x2
+NO_NARROW_BAND = 0x4
 
 
 class Operand(ctypes.Structure):

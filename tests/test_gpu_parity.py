@@ -30,6 +30,7 @@ EDGE = [
     (3, 37, 5, 6), (1, 1, 8, 3), (2, 129, 64, 4), (2, 130, 64, 64), (1, 257, 80, 33), (2, 100, 128, 49),
     (1, 300, 64, 150), (2, 65, 16, 100), (1, 513, 72, 256), (2, 96, 64, 8), (1, 200, 40, 12), (3, 64, 64, 1),
     (1, 1000, 64, 32), (2, 333, 24, 7), (3, 700, 64, 32), (1, 1100, 32, 256), (2, 900, 128, 64), (9, 260, 16, 96),
+    (2, 600, 128, 16), (2, 515, 80, 20), (1, 300, 64, 7), (2, 260, 48, 28), (1, 257, 64, 8), (2, 1030, 64, 12),
 ]
 CASES = REF_GRID + EDGE
 DTYPES = [torch.float32, torch.bfloat16, torch.float16, torch.float64]
@@ -56,7 +57,8 @@ def close(got, want, dtype):
     torch.testing.assert_close(got.cpu().to(want.dtype), want, **TOL[dtype])
 
 
-@pytest.mark.parametrize("flags", [0, abi.FORCE_STRIDED], ids=["auto", "strided"])
+@pytest.mark.parametrize("flags", [0, abi.FORCE_STRIDED, abi.NO_NARROW_BAND | abi.NO_ALIGNED_BAND],
+                         ids=["auto", "strided", "wide-unaligned"])
 @pytest.mark.parametrize("dtype", DTYPES, ids=lambda d: str(d).split(".")[-1])
 @pytest.mark.parametrize("B,M,N,w", CASES)
 def test_all_entry_points_match_oracle(device, B, M, N, w, dtype, flags):
