@@ -371,33 +371,58 @@ __global__ __launch_bounds__(kThreads, 2) void mfma_p1_kernel(const uint16_t *__
     for (int ks = 0; ks < NK; ++ks) xop[ks] = load_row_chunk(xr + 16 * ks, X, i < M);
   }
 
-  int y_r[YS], y_h[YS];
+  // Everything that does not change from chunk to chunk is worked out once per lane here: the
+  // kernel is bound by instruction issue, and per-chunk address and range arithmetic was most of it.
+  // Y loader slots: row y_c0 + 64 k of the sequence, 8 columns from y_h; sink slots never valid.
+  int y_c0[YS], y_lds_off[YS];
+  const uint16_t *y_run[YS];  // address of the slot's chunk in the next chunk to be requested
+  const int y_cmax = min(M - 1, c_hi);
 #pragma unroll
   for (int s = 0; s < YS; ++s) {
     const int q = tid + kThreads * s;
-    y_r[s] = q < KC * N / 8 ? q / (N / 8) : KC;  // KC = no row: loads nothing real, writes to the sink row
-    y_h[s] = q < KC * N / 8 ? (q % (N / 8)) * 8 : 0;
+    const bool real = q < KC * N / 8;
+    const int yr = real ? q / (N / 8) : KC, yh = real ? (q % (N / 8)) * 8 : 0;  // row KC of the LDS tile is a sink
+    y_c0[s] = real ? c_start + yr : -0x40000000;
+    y_lds_off[s] = yr * SY + yh;
+    y_run[s] = Yb + (int64_t)(c_start + yr) * ysr + yh;
   }
+  const int64_t y_step = (int64_t)KC * ysr;
   u32x4 y_reg[PF][YS];
-  auto fetch = [&](int k, u32x4(&yr)[YS]) {  // loads only; chunks past c_hi read the safe address
-    const int cb = c_start + k * KC;
+  auto fetch = [&](int k, u32x4(&yr)[YS]) {  // loads only, called for k = 0, 1, 2, ... in order
 #pragma unroll
     for (int s = 0; s < YS; ++s) {
-      const int c = cb + y_r[s];
-      yr[s] = fetch_row_chunk(Yb + (int64_t)c * ysr + y_h[s], Y, (y_r[s] < KC) & (c >= 0) & (c < M) & (c <= c_hi));
+      const unsigned c = (unsigned)(y_c0[s] + k * KC);  // valid iff 0 <= c <= y_cmax
+      yr[s] = fetch_row_chunk(y_run[s], Y, c <= (unsigned)y_cmax);
+      y_run[s] += y_step;
     }
   };
   auto stash = [&](int k, const u32x4(&yr)[YS]) {
-    const int cb = c_start + k * KC, buf = k & 1;
+    uint16_t *dst = y_lds[k & 1];
 #pragma unroll
     for (int s = 0; s < YS; ++s) {
-      const int c = cb + y_r[s];
-      *reinterpret_cast<u32x4 *>(&y_lds[buf][y_r[s] * SY + y_h[s]]) =
-          mask_row_chunk(pin(yr[s]), (c >= 0) & (c < M) & (c <= c_hi));
+      const unsigned c = (unsigned)(y_c0[s] + k * KC);
+      *reinterpret_cast<u32x4 *>(dst + y_lds_off[s]) = mask_row_chunk(pin(yr[s]), c <= (unsigned)y_cmax);
     }
   };
 
   uint16_t *stage = s_lds[wave];
+  // Store slots: lane -> row r = lane / 8 + 8 s of the wave's 32 rows, column group g = lane % 8.
+  const int iw_first = i0 + wave * 32;
+  int st_lo[4], st_hi[4];   // chunk-relative valid element range is [st_lo - cb, st_hi - cb]
+  uint16_t *st_dst[4];      // address of dense column 8 g of the row (add cb)
+  const uint16_t *st_src[4];
+#pragma unroll
+  for (int s = 0; s < 4; ++s) {
+    const int r = (lane >> 3) + 8 * s, g = lane & 7;
+    const int i = iw_first + r;
+    st_lo[s] = i - w - 8 * g;
+    st_hi[s] = i < M ? i + w - 8 * g : -0x40000000;
+    st_dst[s] = Cb + (int64_t)i * W + (w - i) + 8 * g;
+    st_src[s] = stage + r * SS + 8 * g;
+  }
+  uint16_t *stage_wr = stage + (lane & 31) * SS + 4 * (lane >> 5);
+  const int y_rd_off = (lane & 31) * SY + 8 * (lane >> 5);
+
   // One slot: request Y chunk k+PF, multiply chunk k, stage the 32 x 64 result, store it, then move
   // chunk k+1 into LDS.  The stores are issued before the wait for chunk k+1, which was requested
   // a whole slot earlier, so the wait leaves them (and the newest loads) in flight.
@@ -406,76 +431,80 @@ __global__ __launch_bounds__(kThreads, 2) void mfma_p1_kernel(const uint16_t *__
     const int cb = c_start + k * KC;
     fetch(k + PF, mine);
     __builtin_amdgcn_sched_barrier(0);
+    const bool seq_edge = cb < 0 || cb + KC > M;  // some column of the chunk is outside the sequence
 #pragma unroll
     for (int mt = 0; mt < KC / 32; ++mt) {
       f32x16 acc;
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[v] = 0.f;
-      const uint16_t *yl = &y_lds[buf][(32 * mt + (lane & 31)) * SY + 8 * (lane >> 5)];
+      const uint16_t *yl = y_lds[buf] + y_rd_off + 32 * mt * SY;
 #pragma unroll
       for (int ks = 0; ks < NK; ++ks)
         acc = Mma<T>::run(*reinterpret_cast<const u32x4 *>(yl + 16 * ks), xop[ks], acc);
       // acc[v]: dense column = 32 mt + 8 (v / 4) + 4 (lane / 32) + v % 4, row = lane % 32
 #pragma unroll
       for (int q4 = 0; q4 < 4; ++q4) {
-        const int cl = 32 * mt + 8 * q4 + 4 * (lane >> 5);
-        const int c = cb + cl;
         uint32_t lo = Mma<T>::pack2(acc[4 * q4], acc[4 * q4 + 1]);
         uint32_t hi = Mma<T>::pack2(acc[4 * q4 + 2], acc[4 * q4 + 3]);
-        // columns outside the sequence are +0.0 by definition, whatever X holds
-        if (c < 0 || c >= M) lo &= 0xffff0000u;
-        if (c + 1 < 0 || c + 1 >= M) lo &= 0x0000ffffu;
-        if (c + 2 < 0 || c + 2 >= M) hi &= 0xffff0000u;
-        if (c + 3 < 0 || c + 3 >= M) hi &= 0x0000ffffu;
+        if (seq_edge) {  // columns outside the sequence are +0.0 by definition, whatever X holds
+          const int c = cb + 32 * mt + 8 * q4 + 4 * (lane >> 5);
+          if (c < 0 || c >= M) lo &= 0xffff0000u;
+          if (c + 1 < 0 || c + 1 >= M) lo &= 0x0000ffffu;
+          if (c + 2 < 0 || c + 2 >= M) hi &= 0xffff0000u;
+          if (c + 3 < 0 || c + 3 >= M) hi &= 0x0000ffffu;
+        }
         u32x2 o = {lo, hi};
-        *reinterpret_cast<u32x2 *>(&stage[(lane & 31) * SS + cl]) = o;
+        *reinterpret_cast<u32x2 *>(stage_wr + 32 * mt + 8 * q4) = o;
       }
     }
     wave_sync_lds();
     // Row-contiguous stores: 8 lanes cover the 64 dense columns of one row.
-    // pass A: whole chunks go out; head pieces are parked in the seam buffer.
-    u32x4 v[4];
-    int tail_hi[4];  // >= 0: this slot holds a tail piece with elements 0..tail_hi, handled in pass B
+    if (cb >= iw_first + 31 - w && cb + KC - 1 <= iw_first + w && iw_first + 31 < M) {
+      // every chunk of the wave's tile lies inside the band: nothing to decide
 #pragma unroll
-    for (int s = 0; s < 4; ++s) {
-      const int q = lane + 64 * s, r = q >> 3, g = q & 7;
-      const int rw = wave * 32 + r, i = i0 + rw;
-      const int c8 = cb + 8 * g;
-      const int e_lo = (i - w) - c8, e_hi = (i + w) - c8;
-      tail_hi[s] = -1;
-      if (i < M && e_hi >= 0 && e_lo <= 7) {
-        v[s] = *reinterpret_cast<const u32x4 *>(&stage[r * SS + 8 * g]);
-        uint16_t *dst = Cb + (int64_t)i * W + (c8 - i + w);
-        if (e_lo <= 0 && e_hi >= 7) {
-          store_chunk<ALIGNED>(dst, v[s]);
-        } else if (e_lo > 0) {  // head piece: elements e_lo..7 (W >= 17, so it reaches the chunk's end)
-          if (ALIGNED && rw > 0 && (r > 0 || seam_across_waves))
-            *reinterpret_cast<u32x4 *>(&seam[rw * 8]) = v[s];
-          else
-            store_chunk_elements(dst, v[s], e_lo, 7);
-        } else {
-          tail_hi[s] = e_hi;
+      for (int s = 0; s < 4; ++s) store_chunk<ALIGNED>(st_dst[s] + cb, *reinterpret_cast<const u32x4 *>(st_src[s]));
+      wave_sync_lds();
+    } else {
+      // pass A: whole chunks go out; head pieces are parked in the seam buffer.
+      u32x4 v[4];
+      int tail_hi[4];  // >= 0: this slot holds a tail piece with elements 0..tail_hi, handled in pass B
+#pragma unroll
+      for (int s = 0; s < 4; ++s) {
+        const int rw = wave * 32 + (lane >> 3) + 8 * s, r = rw & 31;
+        const int e_lo = st_lo[s] - cb, e_hi = st_hi[s] - cb;
+        tail_hi[s] = -1;
+        if (e_hi >= 0 && e_lo <= 7) {
+          v[s] = *reinterpret_cast<const u32x4 *>(st_src[s]);
+          uint16_t *dst = st_dst[s] + cb;
+          if (e_lo <= 0 && e_hi >= 7) {
+            store_chunk<ALIGNED>(dst, v[s]);
+          } else if (e_lo > 0) {  // head piece: elements e_lo..7 (W >= 17, so it reaches the chunk's end)
+            if (ALIGNED && rw > 0 && (r > 0 || seam_across_waves))
+              *reinterpret_cast<u32x4 *>(&seam[rw * 8]) = v[s];
+            else
+              store_chunk_elements(dst, v[s], e_lo, 7);
+          } else {
+            tail_hi[s] = e_hi;
+          }
         }
       }
-    }
-    wave_sync_lds();
-    // pass B: tail pieces pick up the head piece of the row below and leave as whole chunks.
+      wave_sync_lds();
+      // pass B: tail pieces pick up the head piece of the row below and leave as whole chunks.
 #pragma unroll
-    for (int s = 0; s < 4; ++s) {
-      if (tail_hi[s] >= 0) {
-        const int q = lane + 64 * s, r = q >> 3, g = q & 7;
-        const int rw = wave * 32 + r, i = i0 + rw;
-        const int c8 = cb + 8 * g;
-        uint16_t *dst = Cb + (int64_t)i * W + (c8 - i + w);
-        if (ALIGNED && rw + 1 < TM && i + 1 < M && (r < 31 || seam_across_waves)) {
-          const u32x4 head = *reinterpret_cast<const u32x4 *>(&seam[(rw + 1) * 8]);
-          const u32x4 mine_part = keep_range(v[s], 0, tail_hi[s]);
-          const u32x4 head_part = keep_range(head, tail_hi[s] + 1, 7);
-          u32x4 merged = {mine_part[0] | head_part[0], mine_part[1] | head_part[1], mine_part[2] | head_part[2],
-                          mine_part[3] | head_part[3]};
-          store_chunk<true>(dst, merged);
-        } else {
-          store_chunk_elements(dst, v[s], 0, tail_hi[s]);
+      for (int s = 0; s < 4; ++s) {
+        if (tail_hi[s] >= 0) {
+          const int rw = wave * 32 + (lane >> 3) + 8 * s, r = rw & 31;
+          uint16_t *dst = st_dst[s] + cb;
+          if (ALIGNED && rw + 1 < TM && i0 + rw + 1 < M && (r < 31 || seam_across_waves)) {
+            const u32x4 head = *reinterpret_cast<const u32x4 *>(&seam[(rw + 1) * 8]);
+            const u32x4 mine_part = keep_range(v[s], 0, tail_hi[s]);
+            const u32x4 head_part = keep_range(head, tail_hi[s] + 1, 7);
+            u32x4 merged = {mine_part[0] | head_part[0], mine_part[1] | head_part[1], mine_part[2] | head_part[2],
+                            mine_part[3] | head_part[3]};
+            store_chunk<true>(dst, merged);
+          } else {
+            store_chunk_elements(dst, v[s], 0, tail_hi[s]);
+          }
         }
       }
     }

@@ -77,6 +77,9 @@ __global__ __launch_bounds__(kThreads) void small_p1_kernel(const uint16_t *__re
     }
 
     uint16_t *img = flat + delta + (64 * wave) * W;  // this wave's 64 rows of the flat band image
+    // image index of entry (r, j) is delta + r W + j = delta + 2w r + c_rel (mod 4 it is delta when w is
+    // even, c_rel being a multiple of 4): then every quad of 4 consecutive entries is 8-byte aligned
+    const bool quad_aligned = (w % 2 == 0) && (delta % 4 == 0);
 #pragma unroll
     for (int nt = 0; nt < 2; ++nt) {
 #pragma unroll
@@ -99,10 +102,18 @@ __global__ __launch_bounds__(kThreads) void small_p1_kernel(const uint16_t *__re
           const uint32_t lo = Mma<T>::pack2(acc[4 * q4], acc[4 * q4 + 1]);
           const uint32_t hi = Mma<T>::pack2(acc[4 * q4 + 2], acc[4 * q4 + 3]);
           // entries outside the sequence are +0.0 by definition, whatever X holds
-          if (j >= 0 && j <= 2 * w) row[j] = (c >= 0 && c < M) ? (uint16_t)lo : (uint16_t)0;
-          if (j + 1 >= 0 && j + 1 <= 2 * w) row[j + 1] = (c + 1 >= 0 && c + 1 < M) ? (uint16_t)(lo >> 16) : (uint16_t)0;
-          if (j + 2 >= 0 && j + 2 <= 2 * w) row[j + 2] = (c + 2 >= 0 && c + 2 < M) ? (uint16_t)hi : (uint16_t)0;
-          if (j + 3 >= 0 && j + 3 <= 2 * w) row[j + 3] = (c + 3 >= 0 && c + 3 < M) ? (uint16_t)(hi >> 16) : (uint16_t)0;
+          const bool seq_all = c >= 0 && c + 3 < M;
+          if (quad_aligned && j >= 0 && j + 3 <= 2 * w && seq_all) {
+            u32x2 o = {lo, hi};  // whole quad inside band and sequence: one 8-byte LDS write
+            *reinterpret_cast<u32x2 *>(row + j) = o;
+          } else if (j + 3 >= 0 && j <= 2 * w) {
+            if (j >= 0 && j <= 2 * w) row[j] = (c >= 0 && c < M) ? (uint16_t)lo : (uint16_t)0;
+            if (j + 1 >= 0 && j + 1 <= 2 * w)
+              row[j + 1] = (c + 1 >= 0 && c + 1 < M) ? (uint16_t)(lo >> 16) : (uint16_t)0;
+            if (j + 2 >= 0 && j + 2 <= 2 * w) row[j + 2] = (c + 2 >= 0 && c + 2 < M) ? (uint16_t)hi : (uint16_t)0;
+            if (j + 3 >= 0 && j + 3 <= 2 * w)
+              row[j + 3] = (c + 3 >= 0 && c + 3 < M) ? (uint16_t)(hi >> 16) : (uint16_t)0;
+          }
         }
       }
     }
