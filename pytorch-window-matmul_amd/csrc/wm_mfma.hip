@@ -28,6 +28,8 @@
 // output band are stored as +0.0 whatever the operands hold.
 #include "wm_mfma_common.hpp"
 
+#include <type_traits>
+
 namespace wm {
 namespace {
 
@@ -431,38 +433,52 @@ __global__ __launch_bounds__(kThreads, 2) void mfma_p1_kernel(const uint16_t *__
     const int cb = c_start + k * KC;
     fetch(k + PF, mine);
     __builtin_amdgcn_sched_barrier(0);
-    const bool seq_edge = cb < 0 || cb + KC > M;  // some column of the chunk is outside the sequence
+    // multiply and stage; the version for chunks with columns outside the sequence forces those
+    // columns to +0.0 (by definition, whatever X holds) and is kept out of the common path
+    auto multiply_and_stage = [&](auto edge) {
 #pragma unroll
-    for (int mt = 0; mt < KC / 32; ++mt) {
-      f32x16 acc;
+      for (int mt = 0; mt < KC / 32; ++mt) {
+        f32x16 acc;
 #pragma unroll
-      for (int v = 0; v < 16; ++v) acc[v] = 0.f;
-      const uint16_t *yl = y_lds[buf] + y_rd_off + 32 * mt * SY;
+        for (int v = 0; v < 16; ++v) acc[v] = 0.f;
+        const uint16_t *yl = y_lds[buf] + y_rd_off + 32 * mt * SY;
 #pragma unroll
-      for (int ks = 0; ks < NK; ++ks)
-        acc = Mma<T>::run(*reinterpret_cast<const u32x4 *>(yl + 16 * ks), xop[ks], acc);
-      // acc[v]: dense column = 32 mt + 8 (v / 4) + 4 (lane / 32) + v % 4, row = lane % 32
+        for (int ks = 0; ks < NK; ++ks)
+          acc = Mma<T>::run(*reinterpret_cast<const u32x4 *>(yl + 16 * ks), xop[ks], acc);
+        // acc[v]: dense column = 32 mt + 8 (v / 4) + 4 (lane / 32) + v % 4, row = lane % 32
 #pragma unroll
-      for (int q4 = 0; q4 < 4; ++q4) {
-        uint32_t lo = Mma<T>::pack2(acc[4 * q4], acc[4 * q4 + 1]);
-        uint32_t hi = Mma<T>::pack2(acc[4 * q4 + 2], acc[4 * q4 + 3]);
-        if (seq_edge) {  // columns outside the sequence are +0.0 by definition, whatever X holds
-          const int c = cb + 32 * mt + 8 * q4 + 4 * (lane >> 5);
-          if (c < 0 || c >= M) lo &= 0xffff0000u;
-          if (c + 1 < 0 || c + 1 >= M) lo &= 0x0000ffffu;
-          if (c + 2 < 0 || c + 2 >= M) hi &= 0xffff0000u;
-          if (c + 3 < 0 || c + 3 >= M) hi &= 0x0000ffffu;
+        for (int q4 = 0; q4 < 4; ++q4) {
+          uint32_t lo = Mma<T>::pack2(acc[4 * q4], acc[4 * q4 + 1]);
+          uint32_t hi = Mma<T>::pack2(acc[4 * q4 + 2], acc[4 * q4 + 3]);
+          if (decltype(edge)::value) {
+            const int c = cb + 32 * mt + 8 * q4 + 4 * (lane >> 5);
+            if (c < 0 || c >= M) lo &= 0xffff0000u;
+            if (c + 1 < 0 || c + 1 >= M) lo &= 0x0000ffffu;
+            if (c + 2 < 0 || c + 2 >= M) hi &= 0xffff0000u;
+            if (c + 3 < 0 || c + 3 >= M) hi &= 0x0000ffffu;
+          }
+          u32x2 o = {lo, hi};
+          *reinterpret_cast<u32x2 *>(stage_wr + 32 * mt + 8 * q4) = o;
         }
-        u32x2 o = {lo, hi};
-        *reinterpret_cast<u32x2 *>(stage_wr + 32 * mt + 8 * q4) = o;
       }
-    }
+    };
+    if (cb < 0 || cb + KC > M)
+      multiply_and_stage(std::true_type{});
+    else
+      multiply_and_stage(std::false_type{});
     wave_sync_lds();
     // Row-contiguous stores: 8 lanes cover the 64 dense columns of one row.
     if (cb >= iw_first + 31 - w && cb + KC - 1 <= iw_first + w && iw_first + 31 < M) {
-      // every chunk of the wave's tile lies inside the band: nothing to decide
+      // every chunk of the wave's tile lies inside the band: nothing to decide, and each group of 8
+      // lanes writes one whole 128-byte line, which is what makes the streaming store pay
 #pragma unroll
-      for (int s = 0; s < 4; ++s) store_chunk<ALIGNED>(st_dst[s] + cb, *reinterpret_cast<const u32x4 *>(st_src[s]));
+      for (int s = 0; s < 4; ++s) {
+        const u32x4 val = *reinterpret_cast<const u32x4 *>(st_src[s]);
+        if (ALIGNED)
+          store_chunk_streaming(st_dst[s] + cb, val);
+        else
+          store_chunk<false>(st_dst[s] + cb, val);
+      }
       wave_sync_lds();
     } else {
       // pass A: whole chunks go out; head pieces are parked in the seam buffer.
@@ -477,7 +493,7 @@ __global__ __launch_bounds__(kThreads, 2) void mfma_p1_kernel(const uint16_t *__
           v[s] = *reinterpret_cast<const u32x4 *>(st_src[s]);
           uint16_t *dst = st_dst[s] + cb;
           if (e_lo <= 0 && e_hi >= 7) {
-            store_chunk<ALIGNED>(dst, v[s]);
+            store_chunk<ALIGNED>(dst, v[s]);  // (plain: lines of edge tiles are completed piecewise)
           } else if (e_lo > 0) {  // head piece: elements e_lo..7 (W >= 17, so it reaches the chunk's end)
             if (ALIGNED && rw > 0 && (r > 0 || seam_across_waves))
               *reinterpret_cast<u32x4 *>(&seam[rw * 8]) = v[s];

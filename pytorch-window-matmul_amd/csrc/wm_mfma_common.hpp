@@ -25,9 +25,11 @@ struct __attribute__((packed, aligned(2))) Chunk2 {
   u32x4 v;
 };
 
+// Band chunks are read exactly once per kernel: the aligned variant loads them non-temporal so
+// that the stream does not evict the operand rows that neighbouring workgroups share in L2.
 template <bool ALIGNED>
 __device__ __forceinline__ u32x4 load_chunk(const uint16_t *p) {
-  if (ALIGNED) return *reinterpret_cast<const u32x4 *>(p);
+  if (ALIGNED) return __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(p));
   return reinterpret_cast<const Chunk2 *>(p)->v;
 }
 template <bool ALIGNED>
@@ -36,6 +38,12 @@ __device__ __forceinline__ void store_chunk(uint16_t *p, u32x4 v) {
     *reinterpret_cast<u32x4 *>(p) = v;
   else
     reinterpret_cast<Chunk2 *>(p)->v = v;
+}
+// Streaming store for data that is written once and not read again by this kernel (the band):
+// marked non-temporal so that it does not push the operand rows other workgroups still need
+// out of the L2.
+__device__ __forceinline__ void store_chunk_streaming(uint16_t *p, u32x4 v) {
+  __builtin_nontemporal_store(v, reinterpret_cast<u32x4 *>(p));
 }
 
 // Keeps elements e_lo..e_hi (inclusive, in 0..7) of a chunk of eight 16-bit values, clears the rest.

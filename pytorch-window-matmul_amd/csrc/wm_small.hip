@@ -128,7 +128,7 @@ __global__ __launch_bounds__(kThreads) void small_p1_kernel(const uint16_t *__re
     const int first = 8 * q - delta;  // band element index of the chunk's element 0
     uint16_t *dst = Cb + first;
     if (first >= 0 && first + 8 <= n_el)
-      *reinterpret_cast<u32x4 *>(dst) = v;
+      store_chunk_streaming(dst, v);
     else
       store_chunk_elements(dst, v, -first, n_el - 1 - first);  // only the workgroup's first and last chunk
   }
@@ -178,7 +178,7 @@ __global__ __launch_bounds__(kThreads) void small_p2_kernel(const uint16_t *__re
       const int qy = q - chunks, yr = qy / ncg, hg = qy - yr * ncg, c = cv0 + yr;
       const uint16_t *src = q < chunks ? Ab - delta + 8 * q : Yb + (int64_t)c * ysr + 8 * hg;
       const bool ok = q < chunks || (q < chunks + ychunks && c >= 0 && c < M);
-      reg[s] = *reinterpret_cast<const u32x4 *>(ok ? src : A);
+      reg[s] = *reinterpret_cast<const u32x4 *>(ok ? src : A);  // (band and Y share the loop: plain loads)
     }
 #pragma unroll
     for (int s = 0; s < BATCH; ++s) {
