@@ -36,12 +36,16 @@ namespace {
 // ------------------------------------------------------------------------------------------
 // P2: C[b,i,h] = sum_c T[i][c] * Y[b,c,h]
 // ------------------------------------------------------------------------------------------
-template <typename T, int NT, bool ALIGNED>
+template <typename T, int NT, bool ALIGNED, int KCH>
 __global__ __launch_bounds__(kThreads, 2) void mfma_p2_kernel(const uint16_t *__restrict__ A,
                                                               const uint16_t *__restrict__ Y,
                                                               uint16_t *__restrict__ C, int B, int M, int N, int w,
                                                               int nblk, int galign, int64_t asb, int64_t ysb,
                                                               int64_t ysr, int64_t csb, int64_t csr) {
+  constexpr int KC = KCH;                 // chunk length of this kernel (shadows the family default)
+  constexpr int TS = TM * KC / 8 / kThreads;  // band chunks per thread per tile
+  constexpr int GPR = KC / 8;              // 8-column groups per tile row
+  constexpr int YS = (KC * NT + 63) / 64;  // Y chunks per thread per tile
   constexpr int NP = 32 * NT;
   constexpr int ST = KC + 8;                         // T tile row stride: 144 B, conflict-free b128 reads
   constexpr int SY = lds_stride_tr(NP);
@@ -61,20 +65,20 @@ __global__ __launch_bounds__(kThreads, 2) void mfma_p2_kernel(const uint16_t *__
   const int nk = (c_hi - c_start + KC) / KC;
 
   // per-thread chunk coordinates (loop invariant)
-  int t_lo[4], t_hi[4];        // valid dense-column range of the chunk's row
-  const uint16_t *t_ptr[4];    // address of dense column 0 of the row (may be virtual)
+  int t_lo[TS], t_hi[TS];        // valid dense-column range of the chunk's row
+  const uint16_t *t_ptr[TS];    // address of dense column 0 of the row (may be virtual)
 #pragma unroll
-  for (int s = 0; s < 4; ++s) {
-    const int q = tid + kThreads * s, r = q >> 3;
+  for (int s = 0; s < TS; ++s) {
+    const int q = tid + kThreads * s, r = q / GPR;
     const int i = i0 + r;
     t_lo[s] = max(i - w, 0);
     t_hi[s] = i < M ? min(i + w, M - 1) : -1;
     t_ptr[s] = Ab + (int64_t)i * W + (w - i);
   }
   const int ychunks = KC * (N >> 3), ncg = N >> 3;
-  int y_r[NT], y_h[NT];
+  int y_r[YS], y_h[YS];
 #pragma unroll
-  for (int s = 0; s < NT; ++s) {
+  for (int s = 0; s < YS; ++s) {
     const int q = tid + kThreads * s;
     y_r[s] = q < ychunks ? q / ncg : KC;  // KC = no row: loads nothing real, writes to the sink row
     y_h[s] = q < ychunks ? (q % ncg) * 8 : 0;
@@ -82,16 +86,16 @@ __global__ __launch_bounds__(kThreads, 2) void mfma_p2_kernel(const uint16_t *__
 
   // Register-staged prefetch PF chunks deep: chunk k+PF is requested before chunk k is
   // multiplied, so PF chunks of band and Y rows are in flight per workgroup at any time.
-  u32x4 t_reg[PF][4], y_reg[PF][NT];
-  auto fetch = [&](int k, u32x4(&tr)[4], u32x4(&yr)[NT]) {  // loads only
+  u32x4 t_reg[PF][TS], y_reg[PF][YS];
+  auto fetch = [&](int k, u32x4(&tr)[TS], u32x4(&yr)[YS]) {  // loads only
     const int cb = c_start + k * KC;
 #pragma unroll
-    for (int s = 0; s < 4; ++s) {
-      const int c8 = cb + 8 * ((tid + kThreads * s) & 7);
+    for (int s = 0; s < TS; ++s) {
+      const int c8 = cb + 8 * ((tid + kThreads * s) & (GPR - 1));
       tr[s] = fetch_band_chunk<ALIGNED>(t_ptr[s] + c8, A, t_lo[s] - c8, t_hi[s] - c8);
     }
 #pragma unroll
-    for (int s = 0; s < NT; ++s) {
+    for (int s = 0; s < YS; ++s) {
       const int c = cb + y_r[s];
       yr[s] = fetch_row_chunk(Yb + (int64_t)c * ysr + y_h[s], Y, (y_r[s] < KC) & (c >= 0) & (c <= c_hi));
     }
@@ -99,32 +103,32 @@ __global__ __launch_bounds__(kThreads, 2) void mfma_p2_kernel(const uint16_t *__
   // A chunk is interior when every element of its T tile and every Y row is valid; its masks
   // are skipped (most chunks of a wide band).
   const int in_lo = rows == TM ? max(i0 + TM - 1 - w, 0) : 0x7fffffff, in_hi = min(i0 + w, c_hi);
-  auto stash = [&](int k, const u32x4(&tr)[4], const u32x4(&yr)[NT]) {  // mask, then to LDS buffer k & 1
+  auto stash = [&](int k, const u32x4(&tr)[TS], const u32x4(&yr)[YS]) {  // mask, then to LDS buffer k & 1
     const int cb = c_start + k * KC, buf = k & 1;
-    u32x4 tv[4], yv[NT];
+    u32x4 tv[TS], yv[YS];
 #pragma unroll
-    for (int s = 0; s < 4; ++s) tv[s] = pin(tr[s]);
+    for (int s = 0; s < TS; ++s) tv[s] = pin(tr[s]);
 #pragma unroll
-    for (int s = 0; s < NT; ++s) yv[s] = pin(yr[s]);
+    for (int s = 0; s < YS; ++s) yv[s] = pin(yr[s]);
     if (!(cb >= in_lo && cb + KC - 1 <= in_hi)) {
 #pragma unroll
-      for (int s = 0; s < 4; ++s) {
-        const int c8 = cb + 8 * ((tid + kThreads * s) & 7);
+      for (int s = 0; s < TS; ++s) {
+        const int c8 = cb + 8 * ((tid + kThreads * s) & (GPR - 1));
         tv[s] = mask_band_chunk(tv[s], t_lo[s] - c8, t_hi[s] - c8);
       }
 #pragma unroll
-      for (int s = 0; s < NT; ++s) {
+      for (int s = 0; s < YS; ++s) {
         const int c = cb + y_r[s];
         yv[s] = mask_row_chunk(yv[s], (c >= 0) & (c <= c_hi));
       }
     }
 #pragma unroll
-    for (int s = 0; s < 4; ++s) {
+    for (int s = 0; s < TS; ++s) {
       const int q = tid + kThreads * s;
-      *reinterpret_cast<u32x4 *>(&t_lds[buf][(q >> 3) * ST + (q & 7) * 8]) = tv[s];
+      *reinterpret_cast<u32x4 *>(&t_lds[buf][(q / GPR) * ST + (q & (GPR - 1)) * 8]) = tv[s];
     }
 #pragma unroll
-    for (int s = 0; s < NT; ++s) *reinterpret_cast<u32x4 *>(&y_lds[buf][y_r[s] * SY + y_h[s]]) = yv[s];
+    for (int s = 0; s < YS; ++s) *reinterpret_cast<u32x4 *>(&y_lds[buf][y_r[s] * SY + y_h[s]]) = yv[s];
   };
 
   f32x16 acc[NT];
@@ -143,7 +147,7 @@ __global__ __launch_bounds__(kThreads, 2) void mfma_p2_kernel(const uint16_t *__
   // The prefetch is unconditional -- chunks past the end are invalid by their coordinates and
   // read the safe address -- and the slots are chained by explicit loop exits, so that the
   // compiler can count outstanding loads exactly and waits only for the set it stores.
-  auto slot = [&](int k, u32x4(&mine_t)[4], u32x4(&mine_y)[NT], u32x4(&next_t)[4], u32x4(&next_y)[NT]) {
+  auto slot = [&](int k, u32x4(&mine_t)[TS], u32x4(&mine_y)[YS], u32x4(&next_t)[TS], u32x4(&next_y)[YS]) {
     const int buf = k & 1;
     fetch(k + PF, mine_t, mine_y);
     __builtin_amdgcn_sched_barrier(0);
@@ -564,13 +568,16 @@ int band_group(const View &v, int64_t w) { return (w % 32 == 0 && ((uintptr_t)v.
 
 unsigned grid_size(int64_t B, int64_t nblk) { return (unsigned)(((B + 7) / 8) * 8 * nblk); }
 
+#ifndef WM_P2_KC
+#define WM_P2_KC 64
+#endif
 template <typename T, bool ALIGNED>
 hipError_t launch_p2(const Problem &p, const View &a, const View &y, const View &c) {
   const int nblk = (int)((p.M + TM - 1) / TM);
   const int galign = band_group(a, p.w);
   const dim3 grid(grid_size(p.B, nblk)), block(kThreads);
 #define WM_P2(NT)                                                                                              \
-  hipLaunchKernelGGL((mfma_p2_kernel<T, NT, ALIGNED>), grid, block, 0, p.stream, (const uint16_t *)a.data,     \
+  hipLaunchKernelGGL((mfma_p2_kernel<T, NT, ALIGNED, WM_P2_KC>), grid, block, 0, p.stream, (const uint16_t *)a.data,     \
                      (const uint16_t *)y.data, (uint16_t *)c.data, (int)p.B, (int)p.M, (int)p.N, (int)p.w, nblk, \
                      galign, a.sb, y.sb, y.sr, c.sb, c.sr)
   switch ((p.N + 31) / 32) {
