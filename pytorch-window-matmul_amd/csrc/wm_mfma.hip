@@ -37,7 +37,7 @@ namespace {
 // P2: C[b,i,h] = sum_c T[i][c] * Y[b,c,h]
 // ------------------------------------------------------------------------------------------
 template <typename T, int NT, bool ALIGNED, int KCH>
-__global__ __launch_bounds__(kThreads, 2) void mfma_p2_kernel(const uint16_t *__restrict__ A,
+__global__ __launch_bounds__(kThreads, NT <= 2 ? 3 : 2) void mfma_p2_kernel(const uint16_t *__restrict__ A,
                                                               const uint16_t *__restrict__ Y,
                                                               uint16_t *__restrict__ C, int B, int M, int N, int w,
                                                               int nblk, int galign, int64_t asb, int64_t ysb,
@@ -47,10 +47,13 @@ __global__ __launch_bounds__(kThreads, 2) void mfma_p2_kernel(const uint16_t *__
   constexpr int GPR = KC / 8;              // 8-column groups per tile row
   constexpr int YS = (KC * NT + 63) / 64;  // Y chunks per thread per tile
   constexpr int NP = 32 * NT;
-  constexpr int ST = KC + 8;                         // T tile row stride: 144 B, conflict-free b128 reads
+  // T tile rows are not padded (LDS is what limits the workgroups per CU); the 16-byte chunk g of
+  // row r lives at chunk position g ^ (r mod GPR), which keeps the b128 operand reads of 8
+  // consecutive rows in different banks
+  constexpr int ST = KC;
   constexpr int SY = lds_stride_tr(NP);
   __shared__ __attribute__((aligned(16))) uint16_t t_lds[2][TM * ST];
-  __shared__ __attribute__((aligned(16))) uint16_t y_lds[2][(KC + 1) * SY];  // row KC: sink for idle loader slots
+  __shared__ __attribute__((aligned(16))) uint16_t y_lds[2][KC * SY];  // columns NP.. of a row are padding
 
   int b, blk;
   if (!decode_block(nblk, B, &b, &blk)) return;
@@ -76,12 +79,13 @@ __global__ __launch_bounds__(kThreads, 2) void mfma_p2_kernel(const uint16_t *__
     t_ptr[s] = Ab + (int64_t)i * W + (w - i);
   }
   const int ychunks = KC * (N >> 3), ncg = N >> 3;
-  int y_r[YS], y_h[YS];
+  int y_r[YS], y_h[YS], y_off[YS];
 #pragma unroll
   for (int s = 0; s < YS; ++s) {
     const int q = tid + kThreads * s;
-    y_r[s] = q < ychunks ? q / ncg : KC;  // KC = no row: loads nothing real, writes to the sink row
+    y_r[s] = q < ychunks ? q / ncg : KC;  // KC = no row: loads nothing real ...
     y_h[s] = q < ychunks ? (q % ncg) * 8 : 0;
+    y_off[s] = q < ychunks ? y_r[s] * SY + y_h[s] : NP;  // ... and writes into the padding of row 0
   }
 
   // Register-staged prefetch PF chunks deep: chunk k+PF is requested before chunk k is
@@ -125,10 +129,10 @@ __global__ __launch_bounds__(kThreads, 2) void mfma_p2_kernel(const uint16_t *__
 #pragma unroll
     for (int s = 0; s < TS; ++s) {
       const int q = tid + kThreads * s;
-      *reinterpret_cast<u32x4 *>(&t_lds[buf][(q / GPR) * ST + (q & (GPR - 1)) * 8]) = tv[s];
+      *reinterpret_cast<u32x4 *>(&t_lds[buf][(q / GPR) * ST + (((q ^ (q / GPR)) & (GPR - 1)) << 3)]) = tv[s];
     }
 #pragma unroll
-    for (int s = 0; s < YS; ++s) *reinterpret_cast<u32x4 *>(&y_lds[buf][y_r[s] * SY + y_h[s]]) = yv[s];
+    for (int s = 0; s < YS; ++s) *reinterpret_cast<u32x4 *>(&y_lds[buf][y_off[s]]) = yv[s];
   };
 
   f32x16 acc[NT];
@@ -151,10 +155,11 @@ __global__ __launch_bounds__(kThreads, 2) void mfma_p2_kernel(const uint16_t *__
     const int buf = k & 1;
     fetch(k + PF, mine_t, mine_y);
     __builtin_amdgcn_sched_barrier(0);
-    const uint16_t *tl = &t_lds[buf][(wave * 32 + (lane & 31)) * ST + 8 * (lane >> 5)];
+    const int trow = wave * 32 + (lane & 31);
+    const uint16_t *tl = &t_lds[buf][trow * ST];
 #pragma unroll
     for (int ks = 0; ks < KC / 16; ++ks) {
-      const u32x4 bop = *reinterpret_cast<const u32x4 *>(tl + ks * 16);
+      const u32x4 bop = *reinterpret_cast<const u32x4 *>(tl + (((2 * ks + (lane >> 5)) ^ trow) & (GPR - 1)) * 8);
 #pragma unroll
       for (int nt = 0; nt < NT; ++nt) {
         const u32x4 aop = lds_read_transposed(y_lds[buf], SY, ks * 16, 32 * nt, lane);
@@ -197,16 +202,16 @@ __global__ __launch_bounds__(kThreads, 2) void mfma_p2_kernel(const uint16_t *__
 // P3: C[b,c,h] = sum_r T[r][c] * Y[b,r,h]
 // ------------------------------------------------------------------------------------------
 template <typename T, int NT, bool ALIGNED>
-__global__ __launch_bounds__(kThreads, 2) void mfma_p3_kernel(const uint16_t *__restrict__ A,
+__global__ __launch_bounds__(kThreads, NT <= 2 ? 3 : 2) void mfma_p3_kernel(const uint16_t *__restrict__ A,
                                                               const uint16_t *__restrict__ Y,
                                                               uint16_t *__restrict__ C, int B, int M, int N, int w,
                                                               int nblk, int galign, int64_t asb, int64_t ysb,
                                                               int64_t ysr, int64_t csb, int64_t csr) {
   constexpr int NP = 32 * NT;
-  constexpr int ST = lds_stride_tr(TM);  // T tile [KC rows r][TM cols c]
+  constexpr int ST = TM;  // T tile [KC rows r][TM cols c], unpadded and swizzled (see lds_read_transposed_swz)
   constexpr int SY = lds_stride_tr(NP);
   __shared__ __attribute__((aligned(16))) uint16_t t_lds[2][KC * ST];
-  __shared__ __attribute__((aligned(16))) uint16_t y_lds[2][(KC + 1) * SY];  // row KC: sink for idle loader slots
+  __shared__ __attribute__((aligned(16))) uint16_t y_lds[2][KC * SY];  // columns NP.. of a row are padding
 
   int b, blk;
   if (!decode_block(nblk, B, &b, &blk)) return;
@@ -222,12 +227,13 @@ __global__ __launch_bounds__(kThreads, 2) void mfma_p3_kernel(const uint16_t *__
   const uint16_t *Yb = Y + (int64_t)b * ysb;
 
   const int ychunks = KC * (N >> 3), ncg = N >> 3;
-  int y_r[NT], y_h[NT];
+  int y_r[NT], y_h[NT], y_off[NT];
 #pragma unroll
   for (int s = 0; s < NT; ++s) {
     const int q = tid + kThreads * s;
-    y_r[s] = q < ychunks ? q / ncg : KC;  // KC = no row: loads nothing real, writes to the sink row
+    y_r[s] = q < ychunks ? q / ncg : KC;  // KC = no row: loads nothing real ...
     y_h[s] = q < ychunks ? (q % ncg) * 8 : 0;
+    y_off[s] = q < ychunks ? y_r[s] * SY + y_h[s] : NP;  // ... and writes into the padding of row 0
   }
 
   u32x4 t_reg[PF][4], y_reg[PF][NT];
@@ -269,10 +275,10 @@ __global__ __launch_bounds__(kThreads, 2) void mfma_p3_kernel(const uint16_t *__
 #pragma unroll
     for (int s = 0; s < 4; ++s) {
       const int q = tid + kThreads * s;
-      *reinterpret_cast<u32x4 *>(&t_lds[buf][(q >> 4) * ST + (q & 15) * 8]) = tv[s];
+      *reinterpret_cast<u32x4 *>(&t_lds[buf][(q >> 4) * ST + swz32((q & 15) * 8, q >> 4)]) = tv[s];
     }
 #pragma unroll
-    for (int s = 0; s < NT; ++s) *reinterpret_cast<u32x4 *>(&y_lds[buf][y_r[s] * SY + y_h[s]]) = yv[s];
+    for (int s = 0; s < NT; ++s) *reinterpret_cast<u32x4 *>(&y_lds[buf][y_off[s]]) = yv[s];
   };
 
   f32x16 acc[NT];
@@ -293,7 +299,7 @@ __global__ __launch_bounds__(kThreads, 2) void mfma_p3_kernel(const uint16_t *__
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int ks = 0; ks < KC / 16; ++ks) {
-      const u32x4 bop = lds_read_transposed(t_lds[buf], ST, ks * 16, wave * 32, lane);
+      const u32x4 bop = lds_read_transposed_swz(t_lds[buf], ST, ks * 16, wave * 32, lane);
 #pragma unroll
       for (int nt = 0; nt < NT; ++nt) {
         const u32x4 aop = lds_read_transposed(y_lds[buf], SY, ks * 16, 32 * nt, lane);

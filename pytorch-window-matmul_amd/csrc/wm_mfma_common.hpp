@@ -134,6 +134,24 @@ __device__ __forceinline__ u32x4 lds_read_transposed(const uint16_t *mat, int st
   return r;
 }
 
+// Same fetch from a matrix stored WITHOUT row padding (row length a multiple of 128 elements) and
+// swizzled instead: the 32-byte block b of row k lives at block position b ^ ((k & 3) << 1).  The
+// four rows a 16-lane group touches (k = 4n .. 4n+3) then fall into four different bank groups.
+__device__ __forceinline__ int swz32(int x, int k) { return (((x >> 4) ^ ((k & 3) << 1)) << 4) | (x & 15); }
+__device__ __forceinline__ u32x4 lds_read_transposed_swz(const uint16_t *mat, int stride, int k0, int x0, int lane) {
+  const int s = lane & 15, grp = lane >> 4;
+  const int xb = x0 + 16 * (grp & 1) + 4 * (s & 3);
+  const int kb = k0 + 8 * (grp >> 1) + (s >> 2);  // k0 is a multiple of 8: kb & 3 == s >> 2, same for kb + 4
+  typedef s16x4 __attribute__((address_space(3))) * lds_ptr;
+  const uint16_t *p0 = mat + kb * stride + swz32(xb, kb);
+  const uint16_t *p1 = p0 + 4 * stride;
+  const s16x4 a = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(p0));
+  const s16x4 b = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(p1));
+  const u32x2 ua = __builtin_bit_cast(u32x2, a), ub = __builtin_bit_cast(u32x2, b);
+  u32x4 r = {ua[0], ua[1], ub[0], ub[1]};
+  return r;
+}
+
 // Pins a prefetched register at this point of the program: the compiler may not use the value
 // (and therefore may not wait for its load) any earlier than here.
 __device__ __forceinline__ u32x4 pin(u32x4 v) {
@@ -159,7 +177,10 @@ __device__ __forceinline__ bool decode_block(int nblk, int B, int *b, int *blk) 
 
 // Row stride (elements) of matrices read with lds_read_transposed: the byte stride must be
 // 32 or 96 (mod 128) so that the 4 rows touched by a 16-lane group fall into distinct banks.
-constexpr int lds_stride_tr(int n_padded) { return n_padded + 16; }
+#ifndef WM_PAD_TR
+#define WM_PAD_TR 16
+#endif
+constexpr int lds_stride_tr(int n_padded) { return n_padded + WM_PAD_TR; }
 
 // Element-wise store of elements [e_lo, e_hi] of a chunk (the slow path for chunk pieces that
 // cannot be completed with their neighbour row's piece).

@@ -12,7 +12,7 @@ import torch
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 REPO = os.path.dirname(HERE)
-LIB_PATH = os.path.join(HERE, "libwindow_matmul_hip.so")
+LIB_PATH = os.environ.get("WM_LIBRARY_PATH", os.path.join(HERE, "libwindow_matmul_hip.so"))
 HEADER = os.path.join(REPO, "include", "window_matmul_hip.h")
 
 DTYPES = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2, torch.float64: 3}
