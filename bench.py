@@ -57,6 +57,21 @@ def kernel_bytes(B, M, N, w, es):
     return band + 2 * mat  # P1: X, Y in, band out;  P2 / P3: band, Y in, C out
 
 
+def profiled_traffic(kernel_label):
+    """HBM bytes per launch of the dominant kernel as measured with rocprofv3 counters (FETCH_SIZE and
+    WRITE_SIZE runs, scaled by a copy of known size); read from the committed summary, None if absent."""
+    path = os.path.join(REPO, "profiles", "config3_bf16_hbm_traffic.md")
+    prim = {"P1": "p1", "P2": "p2", "P3": "p3"}.get(kernel_label[-3:-1])
+    try:
+        for line in open(path):
+            parts = line.split()
+            if len(parts) == 3 and parts[0] == "traffic_bytes_per_launch" and parts[1] == prim:
+                return int(parts[2])
+    except OSError:
+        pass
+    return None
+
+
 def time_gpu(fn, iters, warmup):
     """Mean duration of one launch, each launch bracketed by its own pair of HIP events on the
     current stream (so that the gap between dependent launches is not counted as kernel time)."""
@@ -224,7 +239,8 @@ def main():
         "config": {"workload": cfg["label"], "B": B, "M": M, "N": N, "w": w,
                    "band_gflop_per_step": round(flops / 1e9, 2)},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None, "kernel": dom,
+                     "frac": round(achieved / HBM_PEAK_GBS, 4),
+                     "traffic": profiled_traffic(dom) if args.workload == "c3" else None, "kernel": dom,
                      "algorithmic_bytes_per_launch": kb, "avg_launch_ms": per_kernel[dom]["ms"]},
         "kernels": per_kernel,
         "softmax_fwd_ms": round(softmax_ms, 4),
