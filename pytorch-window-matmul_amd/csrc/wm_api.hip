@@ -26,25 +26,27 @@ int to_status(hipError_t err) {
 typedef bool (*mfma_fn)(const Problem &, const View &, const View &, const View &, hipError_t *);
 typedef hipError_t (*strided_fn)(const Problem &, const View &, const View &, const View &);
 
-// Kernel choice per primitive: narrow-band family, else wide-band MFMA family, else strided.
-int run_primitive(mfma_fn narrow, mfma_fn fast, strided_fn slow, const Problem &p, const View &a, const View &y,
-                  const View &c) {
+// Kernel choice per primitive: narrow-band family, else wide-band MFMA family (both 16-bit
+// storage), else the float32 MFMA family, else strided.
+int run_primitive(mfma_fn narrow, mfma_fn fast, mfma_fn f32, strided_fn slow, const Problem &p, const View &a,
+                  const View &y, const View &c) {
   hipError_t err = hipSuccess;
   if (!(p.flags & WM_FLAG_FORCE_STRIDED)) {
     if (narrow && !(p.flags & WM_FLAG_NO_NARROW_BAND) && narrow(p, a, y, c, &err)) return to_status(err);
     if (fast(p, a, y, c, &err)) return to_status(err);
+    if (f32(p, a, y, c, &err)) return to_status(err);
   }
   return to_status(slow(p, a, y, c));
 }
 
 int p1(const Problem &p, const View &x, const View &y, const View &c) {
-  return run_primitive(try_launch_small_p1, try_launch_mfma_p1, launch_strided_p1, p, x, y, c);
+  return run_primitive(try_launch_small_p1, try_launch_mfma_p1, try_launch_f32_p1, launch_strided_p1, p, x, y, c);
 }
 int p2(const Problem &p, const View &a, const View &y, const View &c) {
-  return run_primitive(try_launch_small_p2, try_launch_mfma_p2, launch_strided_p2, p, a, y, c);
+  return run_primitive(try_launch_small_p2, try_launch_mfma_p2, try_launch_f32_p2, launch_strided_p2, p, a, y, c);
 }
 int p3(const Problem &p, const View &a, const View &y, const View &c) {
-  return run_primitive(nullptr, try_launch_mfma_p3, launch_strided_p3, p, a, y, c);
+  return run_primitive(nullptr, try_launch_mfma_p3, try_launch_f32_p3, launch_strided_p3, p, a, y, c);
 }
 
 }  // namespace
@@ -117,6 +119,10 @@ const char *wm_kernel_choice(int op, int64_t B, int64_t M, int64_t N, int64_t w,
     }
     if (mfma_supports(op, B, M, N, w, dtype)) {
       static const char *names[] = {"mfma_p1", "mfma_p2", "mfma_p3"};
+      return names[op - 1];
+    }
+    if (f32_supports(op, M, N, w, dtype)) {
+      static const char *names[] = {"f32_mfma_p1", "f32_mfma_p2", "f32_mfma_p3"};
       return names[op - 1];
     }
   }

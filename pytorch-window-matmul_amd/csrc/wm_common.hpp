@@ -48,6 +48,11 @@ bool try_launch_mfma_p3(const Problem &p, const View &a, const View &y, const Vi
 bool try_launch_small_p1(const Problem &p, const View &x, const View &y, const View &c, hipError_t *err);
 bool try_launch_small_p2(const Problem &p, const View &a, const View &y, const View &c, hipError_t *err);
 bool small_supports(int op, int64_t M, int64_t N, int64_t w, int dtype);
+// float32 MFMA family (N multiple of 8 up to 128, w >= 4).
+bool try_launch_f32_p1(const Problem &p, const View &x, const View &y, const View &c, hipError_t *err);
+bool try_launch_f32_p2(const Problem &p, const View &a, const View &y, const View &c, hipError_t *err);
+bool try_launch_f32_p3(const Problem &p, const View &a, const View &y, const View &c, hipError_t *err);
+bool f32_supports(int op, int64_t M, int64_t N, int64_t w, int dtype);
 // Pure predicate behind the three functions above (shape/dtype only).
 bool mfma_supports(int op, int64_t B, int64_t M, int64_t N, int64_t w, int dtype);
 

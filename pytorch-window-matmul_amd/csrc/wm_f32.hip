@@ -1,0 +1,346 @@
+// float32 MFMA kernel family (v_mfma_f32_32x32x2_f32) for gfx950.
+//
+// Same tiling idea as the 16-bit wide-band family -- a workgroup of four waves owns 128 rows
+// and walks the contraction in chunks, the skewed tile T[r][c] = band[r, c-r+w] and the dense
+// operand chunk go through LDS -- but with 4-byte elements and a matrix instruction whose
+// operands are one float per lane (row = lane % 32, k = lane / 32).  float32 at these shapes is
+// bound by the matrix pipe (157 TFLOP/s), not by HBM, so the memory side is kept simple:
+// 16-byte band accesses at 4-byte alignment (no aligned column grid, no seam handling),
+// one chunk of register prefetch, double-buffered LDS, one barrier per chunk.
+//
+// Contraction order.  An MFMA step contracts two k values, one per half-wave.  The kernels walk
+// k in groups of 8: step (u, j), half-wave s, uses k = 8u + 4s + j.  Both operands use the same
+// map, so the sum is unchanged, and an operand whose k runs along memory is fetched as one
+// 16-byte LDS read per group (4 steps) instead of one 4-byte read per step.
+#include "wm_common.hpp"
+
+namespace wm {
+namespace {
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+constexpr int kThreads = 256;
+constexpr int TM = 128;  // rows per workgroup, 32 per wave
+constexpr int KC = 32;   // chunk length
+
+struct __attribute__((packed, aligned(4))) Chunk4 {
+  f32x4 v;
+};
+__device__ __forceinline__ f32x4 load4(const float *p) { return reinterpret_cast<const Chunk4 *>(p)->v; }
+__device__ __forceinline__ void store4(float *p, f32x4 v) { reinterpret_cast<Chunk4 *>(p)->v = v; }
+
+// Elements [e_lo, e_hi] of a 4-element band chunk, the rest cleared (on bits: NaN-safe).
+__device__ __forceinline__ f32x4 keep4(f32x4 v, int e_lo, int e_hi) {
+  f32x4 r;
+#pragma unroll
+  for (int e = 0; e < 4; ++e) r[e] = (e >= e_lo && e <= e_hi) ? v[e] : 0.f;
+  return r;
+}
+// Band chunk with valid elements [e_lo, e_hi]: read whole when any element is valid (the up-to-3
+// elements beside a row's valid range are band entries of the same or the neighbouring row for
+// w >= 3; the kernels are used for w >= 4), from `safe` otherwise; invalid elements cleared.
+__device__ __forceinline__ f32x4 load_band4(const float *p, const float *safe, int e_lo, int e_hi) {
+  const bool any = (e_hi >= 0) & (e_lo <= 3) & (e_lo <= e_hi);
+  return keep4(load4(any ? p : safe), any ? e_lo : 4, e_hi);
+}
+__device__ __forceinline__ f32x4 load_row4(const float *p, const float *safe, bool valid) {
+  const f32x4 v = *reinterpret_cast<const f32x4 *>(valid ? p : safe);
+  f32x4 z = {0.f, 0.f, 0.f, 0.f};
+  return valid ? v : z;
+}
+__device__ __forceinline__ f32x16 mma(float a, float b, f32x16 c) {
+  return __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, 0, 0, 0);
+}
+__device__ __forceinline__ bool decode_block(int nblk, int B, int *b, int *blk) {
+  const int id = blockIdx.x, xcd = id & 7, slot = id >> 3;  // all blocks of a batch element on one XCD
+  *b = (slot / nblk) * 8 + xcd;
+  *blk = slot % nblk;
+  return *b < B;
+}
+
+// ------------------------------------------------------------------------------------------
+// P2: C[b,i,h] = sum_c T[i][c] Y[b,c,h]          P3: C[b,c,h] = sum_r T[r][c] Y[b,r,h]
+// acc(m = h, n = output row): A operand Y[k][h] (4-byte LDS reads along h), B operand T.
+// ------------------------------------------------------------------------------------------
+template <int NT, bool TRANSPOSED>
+__global__ __launch_bounds__(kThreads, 2) void f32_band_in_kernel(const float *__restrict__ A,
+                                                                  const float *__restrict__ Y,
+                                                                  float *__restrict__ C, int B, int M, int N, int w,
+                                                                  int nblk, int64_t asb, int64_t ysb, int64_t ysr,
+                                                                  int64_t csb, int64_t csr) {
+  constexpr int NP = 32 * NT;
+  constexpr int ST = TRANSPOSED ? TM + 4 : KC + 4;  // T tile: [KC][TM] (P3) or [TM][KC] (P2), floats
+  constexpr int TROWS = TRANSPOSED ? KC : TM;
+  constexpr int SY = NP + 4;
+  __shared__ __attribute__((aligned(16))) float t_lds[2][TROWS * ST];
+  __shared__ __attribute__((aligned(16))) float y_lds[2][KC * SY];
+
+  int b, blk;
+  if (!decode_block(nblk, B, &b, &blk)) return;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int W = 2 * w + 1;
+  const int o0 = blk * TM;                 // first output row of the block (i for P2, c for P3)
+  const int o1 = min(o0 + TM, M) - 1;      // last one
+  const int k_lo = max(o0 - w, 0), k_hi = min(o1 + w, M - 1);  // contraction range (c for P2, r for P3)
+  const int nk = (k_hi - k_lo + KC) / KC;
+  const float *Ab = A + (int64_t)b * asb;
+  const float *Yb = Y + (int64_t)b * ysb;
+  const int ncg = N >> 2, ychunks = KC * ncg;
+
+  f32x4 t_reg[4], y_reg[NT];
+  auto fetch = [&](int k) {
+    const int kb = k_lo + k * KC;
+#pragma unroll
+    for (int s = 0; s < 4; ++s) {
+      const int q = tid + kThreads * s;
+      if (!TRANSPOSED) {  // tile row = band row i, 4 consecutive dense columns c
+        const int i = o0 + (q >> 3), c4 = kb + 4 * (q & 7);
+        const int lo = max(i - w, 0), hi = i <= o1 ? min(i + w, k_hi) : -1;
+        t_reg[s] = load_band4(Ab + (int64_t)i * W + (w - i) + c4, A, lo - c4, hi - c4);
+      } else {  // tile row = band row r (the contraction index), 4 consecutive output columns c
+        const int r = kb + (q >> 5), c4 = o0 + 4 * (q & 31);
+        const int lo = max(r - w, o0), hi = r <= k_hi ? min(r + w, o1) : -1;
+        t_reg[s] = load_band4(Ab + (int64_t)r * W + (w - r) + c4, A, lo - c4, hi - c4);
+      }
+    }
+#pragma unroll
+    for (int s = 0; s < NT; ++s) {
+      const int q = tid + kThreads * s;
+      const int kr = kb + q / ncg;
+      y_reg[s] = load_row4(Yb + (int64_t)kr * ysr + (q % ncg) * 4, Y, (q < ychunks) & (kr <= k_hi));
+    }
+  };
+  auto stash = [&](int buf) {
+#pragma unroll
+    for (int s = 0; s < 4; ++s) {
+      const int q = tid + kThreads * s;
+      float *dst = TRANSPOSED ? &t_lds[buf][(q >> 5) * ST + 4 * (q & 31)] : &t_lds[buf][(q >> 3) * ST + 4 * (q & 7)];
+      *reinterpret_cast<f32x4 *>(dst) = t_reg[s];
+    }
+#pragma unroll
+    for (int s = 0; s < NT; ++s) {
+      const int q = tid + kThreads * s;
+      if (q < ychunks) *reinterpret_cast<f32x4 *>(&y_lds[buf][(q / ncg) * SY + (q % ncg) * 4]) = y_reg[s];
+    }
+  };
+
+  f32x16 acc[NT];
+#pragma unroll
+  for (int t = 0; t < NT; ++t)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) acc[t][v] = 0.f;
+
+  fetch(0);
+  stash(0);
+  __syncthreads();
+  const int half = lane >> 5, col = lane & 31;
+  for (int k = 0; k < nk; ++k) {
+    const int buf = k & 1;
+    if (k + 1 < nk) fetch(k + 1);
+    const float *tl = t_lds[buf];
+    const float *yl = y_lds[buf];
+#pragma unroll
+    for (int u = 0; u < KC / 8; ++u) {
+      const int kk = 8 * u + 4 * half;  // this half-wave's 4 k values of the group
+      f32x4 bop;
+      if (!TRANSPOSED) {
+        bop = *reinterpret_cast<const f32x4 *>(tl + (wave * 32 + col) * ST + kk);
+      } else {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) bop[j] = tl[(kk + j) * ST + wave * 32 + col];
+      }
+#pragma unroll
+      for (int t = 0; t < NT; ++t)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[t] = mma(yl[(kk + j) * SY + 32 * t + col], bop[j], acc[t]);
+    }
+    if (k + 1 < nk) stash(buf ^ 1);
+    __syncthreads();
+  }
+
+  // acc[t][v]: h = 32 t + 8 (v / 4) + 4 (lane / 32) + v % 4, output row = wave * 32 + lane % 32
+  const int o = o0 + wave * 32 + col;
+  if (o <= o1) {
+    float *crow = C + (int64_t)b * csb + (int64_t)o * csr;
+#pragma unroll
+    for (int t = 0; t < NT; ++t)
+#pragma unroll
+      for (int q4 = 0; q4 < 4; ++q4) {
+        const int h = 32 * t + 8 * q4 + 4 * half;
+        if (h < N) {
+          f32x4 out = {acc[t][4 * q4], acc[t][4 * q4 + 1], acc[t][4 * q4 + 2], acc[t][4 * q4 + 3]};
+          *reinterpret_cast<f32x4 *>(crow + h) = out;
+        }
+      }
+  }
+}
+
+// ------------------------------------------------------------------------------------------
+// P1: band[b,i,c-i+w] = sum_h X[b,i,h] Y[b,c,h]   (+0.0 where c is outside the sequence)
+// acc(m = c, n = i): A operand Y chunk (LDS, k = h along memory), B operand X rows (registers).
+// ------------------------------------------------------------------------------------------
+template <int NK8>  // N = 8 NK8
+__global__ __launch_bounds__(kThreads, 2) void f32_band_out_kernel(const float *__restrict__ X,
+                                                                   const float *__restrict__ Y,
+                                                                   float *__restrict__ C, int B, int M, int w,
+                                                                   int nblk, int64_t xsb, int64_t xsr, int64_t ysb,
+                                                                   int64_t ysr, int64_t csb) {
+  constexpr int N = 8 * NK8;
+  constexpr int SY = N + 4;
+  constexpr int YS = (KC * N / 4 + kThreads - 1) / kThreads;
+  __shared__ __attribute__((aligned(16))) float y_lds[2][KC * SY];
+
+  int b, blk;
+  if (!decode_block(nblk, B, &b, &blk)) return;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int half = lane >> 5, col = lane & 31;
+  const int W = 2 * w + 1;
+  const int i0 = blk * TM;
+  const int rows = min(TM, M - i0);
+  const int c_lo = i0 - w, c_hi = i0 + rows - 1 + w;  // not clipped: entries outside the sequence are zeros
+  const int nk = (c_hi - c_lo + KC) / KC;
+  const float *Yb = Y + (int64_t)b * ysb;
+  float *Cb = C + (int64_t)b * csb;
+
+  // this lane's row of X, the k values of its half-wave: xop[u][j] = X[i][8u + 4 half + j]
+  const int i = i0 + wave * 32 + col;
+  f32x4 xop[NK8];
+#pragma unroll
+  for (int u = 0; u < NK8; ++u)
+    xop[u] = load_row4(X + (int64_t)b * xsb + (int64_t)i * xsr + 8 * u + 4 * half, X, i < M);
+
+  f32x4 y_reg[YS];
+  auto fetch = [&](int k) {
+    const int cb = c_lo + k * KC;
+#pragma unroll
+    for (int s = 0; s < YS; ++s) {
+      const int q = tid + kThreads * s;
+      const int c = cb + q / (N / 4);
+      y_reg[s] = load_row4(Yb + (int64_t)c * ysr + (q % (N / 4)) * 4, Y, (q < KC * N / 4) & (c >= 0) & (c < M));
+    }
+  };
+  auto stash = [&](int buf) {
+#pragma unroll
+    for (int s = 0; s < YS; ++s) {
+      const int q = tid + kThreads * s;
+      if (q < KC * N / 4) *reinterpret_cast<f32x4 *>(&y_lds[buf][(q / (N / 4)) * SY + (q % (N / 4)) * 4]) = y_reg[s];
+    }
+  };
+
+  fetch(0);
+  stash(0);
+  __syncthreads();
+  for (int k = 0; k < nk; ++k) {
+    const int buf = k & 1;
+    const int cb = c_lo + k * KC;
+    if (k + 1 < nk) fetch(k + 1);
+    f32x16 acc;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) acc[v] = 0.f;
+    const float *yl = y_lds[buf] + col * SY + 4 * half;
+#pragma unroll
+    for (int u = 0; u < NK8; ++u) {
+      const f32x4 aop = *reinterpret_cast<const f32x4 *>(yl + 8 * u);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) acc = mma(aop[j], xop[u][j], acc);
+    }
+    // acc[v]: dense column c = cb + 8 (v / 4) + 4 half + v % 4, row i; band column j = c - i + w
+    if (i < M) {
+      float *brow = Cb + (int64_t)i * W + (w - i);  // address of dense column 0 of row i
+#pragma unroll
+      for (int q4 = 0; q4 < 4; ++q4) {
+        const int c = cb + 8 * q4 + 4 * half;
+        f32x4 out;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) out[e] = (c + e >= 0 && c + e < M) ? acc[4 * q4 + e] : 0.f;  // +0.0 outside
+        const int e_lo = (i - w) - c, e_hi = (i + w) - c;
+        if (e_lo <= 0 && e_hi >= 3) {
+          store4(brow + c, out);
+        } else {
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            if (e >= e_lo && e <= e_hi) brow[c + e] = out[e];
+        }
+      }
+    }
+    if (k + 1 < nk) stash(buf ^ 1);
+    __syncthreads();
+  }
+}
+
+// ------------------------------------------------------------------------------------------
+// host side
+// ------------------------------------------------------------------------------------------
+bool f32_shape_ok(int64_t M, int64_t N, int64_t w, int dtype) {
+  if (dtype != WM_DTYPE_F32) return false;
+  if (N < 8 || N > 128 || N % 8 != 0) return false;
+  return M >= 1 && M <= (1 << 30) && w >= 4 && w <= (1 << 28);
+}
+bool f32_band_ok(const View &v, int64_t W) { return v.sc == 1 && v.sr == W && ((uintptr_t)v.data % 4) == 0; }
+unsigned f32_grid(int64_t B, int64_t nblk) { return (unsigned)(((B + 7) / 8) * 8 * nblk); }
+
+template <bool TRANSPOSED>
+hipError_t launch_band_in(const Problem &p, const View &a, const View &y, const View &c) {
+  const int nblk = (int)((p.M + TM - 1) / TM);
+  const dim3 grid(f32_grid(p.B, nblk)), block(kThreads);
+#define WM_F32_IN(NT)                                                                                        \
+  hipLaunchKernelGGL((f32_band_in_kernel<NT, TRANSPOSED>), grid, block, 0, p.stream, (const float *)a.data,  \
+                     (const float *)y.data, (float *)c.data, (int)p.B, (int)p.M, (int)p.N, (int)p.w, nblk,   \
+                     a.sb, y.sb, y.sr, c.sb, c.sr)
+  switch ((p.N + 31) / 32) {
+    case 1: WM_F32_IN(1); break;
+    case 2: WM_F32_IN(2); break;
+    case 3: WM_F32_IN(3); break;
+    default: WM_F32_IN(4); break;
+  }
+#undef WM_F32_IN
+  return hipGetLastError();
+}
+
+hipError_t launch_band_out(const Problem &p, const View &x, const View &y, const View &c) {
+  const int nblk = (int)((p.M + TM - 1) / TM);
+  const dim3 grid(f32_grid(p.B, nblk)), block(kThreads);
+#define WM_F32_OUT(NK8)                                                                                     \
+  case NK8:                                                                                                 \
+    hipLaunchKernelGGL((f32_band_out_kernel<NK8>), grid, block, 0, p.stream, (const float *)x.data,         \
+                       (const float *)y.data, (float *)c.data, (int)p.B, (int)p.M, (int)p.w, nblk, x.sb,    \
+                       x.sr, y.sb, y.sr, c.sb);                                                             \
+    break;
+  switch (p.N / 8) {
+    WM_F32_OUT(1) WM_F32_OUT(2) WM_F32_OUT(3) WM_F32_OUT(4) WM_F32_OUT(5) WM_F32_OUT(6) WM_F32_OUT(7) WM_F32_OUT(8)
+    WM_F32_OUT(9) WM_F32_OUT(10) WM_F32_OUT(11) WM_F32_OUT(12) WM_F32_OUT(13) WM_F32_OUT(14) WM_F32_OUT(15)
+    WM_F32_OUT(16)
+    default: return hipErrorInvalidValue;
+  }
+#undef WM_F32_OUT
+  return hipGetLastError();
+}
+
+}  // namespace
+
+bool f32_supports(int op, int64_t M, int64_t N, int64_t w, int dtype) {
+  (void)op;
+  return f32_shape_ok(M, N, w, dtype);
+}
+
+bool try_launch_f32_p1(const Problem &p, const View &x, const View &y, const View &c, hipError_t *err) {
+  if (!f32_shape_ok(p.M, p.N, p.w, p.dtype)) return false;
+  if (!fast_layout(x, p.dtype) || !fast_layout(y, p.dtype) || !f32_band_ok(c, 2 * p.w + 1)) return false;
+  *err = launch_band_out(p, x, y, c);
+  return true;
+}
+bool try_launch_f32_p2(const Problem &p, const View &a, const View &y, const View &c, hipError_t *err) {
+  if (!f32_shape_ok(p.M, p.N, p.w, p.dtype)) return false;
+  if (!f32_band_ok(a, 2 * p.w + 1) || !fast_layout(y, p.dtype) || !fast_layout(c, p.dtype)) return false;
+  *err = launch_band_in<false>(p, a, y, c);
+  return true;
+}
+bool try_launch_f32_p3(const Problem &p, const View &a, const View &y, const View &c, hipError_t *err) {
+  if (!f32_shape_ok(p.M, p.N, p.w, p.dtype)) return false;
+  if (!f32_band_ok(a, 2 * p.w + 1) || !fast_layout(y, p.dtype) || !fast_layout(c, p.dtype)) return false;
+  *err = launch_band_in<true>(p, a, y, c);
+  return true;
+}
+
+}  // namespace wm
