@@ -113,8 +113,11 @@ torch::Tensor window_matmul_forward(torch::Tensor src, torch::Tensor other, int6
 }
 
 // reference: window_matmul_backward -> window_matmul_bw_cuda (window_matmul.cpp:80-85, cuda:272-319)
-std::tuple<torch::Tensor, torch::Tensor> window_matmul_backward(torch::Tensor src, torch::Tensor other,
-                                                                 int64_t window_size, torch::Tensor grad_output) {
+// need_src / need_other (extensions of the reference signature, both true by default) let the
+// autograd Function skip the kernel of a gradient nobody asked for; a skipped one comes back as None.
+std::tuple<c10::optional<torch::Tensor>, c10::optional<torch::Tensor>> window_matmul_backward(
+    torch::Tensor src, torch::Tensor other, int64_t window_size, torch::Tensor grad_output, bool need_src,
+    bool need_other) {
   TORCH_CHECK(window_size >= 0, "Input mismatch");
   check_window_inputs(src, other);
   const int64_t B = src.size(0), M = src.size(1), N = src.size(2);
@@ -124,13 +127,16 @@ std::tuple<torch::Tensor, torch::Tensor> window_matmul_backward(torch::Tensor sr
   auto q = vector_friendly(src);
   auto kt = key_rows(other).transpose(1, 2);
   auto ga = band_friendly(grad_output);
-  auto grad_q = torch::empty({B, M, N}, src.options());
+  c10::optional<torch::Tensor> grad_q, grad_k;
+  if (need_src) grad_q = torch::empty({B, M, N}, src.options());
   // grad_k is produced row-major per key row and handed back in the (B,N,M)
   // orientation of `other` as a transposed view, like the reference (cuda:318).
-  auto grad_k = torch::empty({B, M, N}, src.options()).transpose(1, 2);
-  wm_operand oq = operand(q), ok = operand(kt), oga = operand(ga), ogq = operand(grad_q), ogk = operand(grad_k);
-  raise_on_error(wm_window_matmul_backward(&oq, &ok, &oga, &ogq, &ogk, B, M, N, window_size, dtype, 0,
-                                           current_stream(src)),
+  if (need_other) grad_k = torch::empty({B, M, N}, src.options()).transpose(1, 2);
+  wm_operand oq = operand(q), ok = operand(kt), oga = operand(ga), ogq{}, ogk{};
+  if (need_src) ogq = operand(*grad_q);
+  if (need_other) ogk = operand(*grad_k);
+  raise_on_error(wm_window_matmul_backward(&oq, &ok, &oga, need_src ? &ogq : nullptr, need_other ? &ogk : nullptr, B,
+                                           M, N, window_size, dtype, 0, current_stream(src)),
                  "window_matmul_backward");
   return std::make_tuple(grad_q, grad_k);
 }
@@ -152,9 +158,9 @@ torch::Tensor unwindow_matmul_forward(torch::Tensor src, torch::Tensor other, in
 }
 
 // reference: unwindow_matmul_backward -> unwindow_matmul_bw_cuda (window_matmul.cpp:93-98, cuda:360-416)
-std::tuple<torch::Tensor, torch::Tensor> unwindow_matmul_backward(torch::Tensor src, torch::Tensor other,
-                                                                   int64_t window_size,
-                                                                   torch::Tensor grad_output) {
+std::tuple<c10::optional<torch::Tensor>, c10::optional<torch::Tensor>> unwindow_matmul_backward(
+    torch::Tensor src, torch::Tensor other, int64_t window_size, torch::Tensor grad_output, bool need_src,
+    bool need_other) {
   TORCH_CHECK(window_size >= 0, "Input mismatch");
   check_unwindow_inputs(src, other, window_size);
   const int64_t B = other.size(0), M = other.size(1), N = other.size(2);
@@ -164,11 +170,14 @@ std::tuple<torch::Tensor, torch::Tensor> unwindow_matmul_backward(torch::Tensor 
   auto a = band_friendly(src);
   auto v = vector_friendly(other);
   auto go = vector_friendly(grad_output);
-  auto grad_a = torch::empty({B, M, 2 * window_size + 1}, src.options());
-  auto grad_v = torch::empty({B, M, N}, src.options());
-  wm_operand oa = operand(a), ov = operand(v), ogo = operand(go), oga = operand(grad_a), ogv = operand(grad_v);
-  raise_on_error(wm_unwindow_matmul_backward(&oa, &ov, &ogo, &oga, &ogv, B, M, N, window_size, dtype, 0,
-                                             current_stream(src)),
+  c10::optional<torch::Tensor> grad_a, grad_v;
+  if (need_src) grad_a = torch::empty({B, M, 2 * window_size + 1}, src.options());
+  if (need_other) grad_v = torch::empty({B, M, N}, src.options());
+  wm_operand oa = operand(a), ov = operand(v), ogo = operand(go), oga{}, ogv{};
+  if (need_src) oga = operand(*grad_a);
+  if (need_other) ogv = operand(*grad_v);
+  raise_on_error(wm_unwindow_matmul_backward(&oa, &ov, &ogo, need_src ? &oga : nullptr, need_other ? &ogv : nullptr, B,
+                                             M, N, window_size, dtype, 0, current_stream(src)),
                  "unwindow_matmul_backward");
   return std::make_tuple(grad_a, grad_v);
 }
@@ -178,8 +187,11 @@ std::tuple<torch::Tensor, torch::Tensor> unwindow_matmul_backward(torch::Tensor 
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.doc() = "MI355X banded matmul kernels behind the window_matmul package";
   m.def("window_matmul_forward", &window_matmul_forward, "WindowMatmul forward");
-  m.def("window_matmul_backward", &window_matmul_backward, "WindowMatmul backward");
+  m.def("window_matmul_backward", &window_matmul_backward, "WindowMatmul backward", py::arg("src"), py::arg("other"),
+        py::arg("window_size"), py::arg("grad_output"), py::arg("need_src") = true, py::arg("need_other") = true);
   m.def("unwindow_matmul_forward", &unwindow_matmul_forward, "UnwindowMatmul forward");
-  m.def("unwindow_matmul_backward", &unwindow_matmul_backward, "UnwindowMatmul backward");
+  m.def("unwindow_matmul_backward", &unwindow_matmul_backward, "UnwindowMatmul backward", py::arg("src"),
+        py::arg("other"), py::arg("window_size"), py::arg("grad_output"), py::arg("need_src") = true,
+        py::arg("need_other") = true);
   m.def("abi_version", []() { return wm_abi_version(); }, "ABI version of libwindow_matmul_hip.so");
 }

@@ -42,7 +42,10 @@ class WindowMatmulFunc(torch.autograd.Function):
         inp, other = ctx.saved_tensors
         # the band width fixes the window: W = 2w + 1  (reference window_matmul.py:22)
         half_width = grad_output.shape[-1] // 2
-        grad_inp, grad_other = _native.window_matmul_backward(inp, other, half_width, grad_output)
+        # a gradient nobody asked for is not computed (the reference always computes both)
+        grad_inp, grad_other = _native.window_matmul_backward(
+            inp, other, half_width, grad_output, ctx.needs_input_grad[0], ctx.needs_input_grad[1]
+        )
         return grad_inp, grad_other, None
 
 
@@ -64,7 +67,9 @@ class UnwindowMatmulFunc(torch.autograd.Function):
     def backward(ctx, grad_output: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor, None]:
         inp, other = ctx.saved_tensors
         half_width = inp.shape[-1] // 2  # reference window_matmul.py:59
-        grad_inp, grad_other = _native.unwindow_matmul_backward(inp, other, half_width, grad_output)
+        grad_inp, grad_other = _native.unwindow_matmul_backward(
+            inp, other, half_width, grad_output, ctx.needs_input_grad[0], ctx.needs_input_grad[1]
+        )
         return grad_inp, grad_other, None
 
 

@@ -169,3 +169,35 @@ def test_error_behaviour(device):
         native.window_matmul_forward(q, torch.zeros(2, 4, 8), 1)
     with pytest.raises(RuntimeError, match="not implemented for"):
         native.window_matmul_forward(q.int(), torch.zeros(2, 4, 8, device=device).int(), 1)
+
+
+@pytest.mark.parametrize("which", ["first", "second"])
+def test_gradient_of_one_input_only(device, which):
+    """Only the requested gradient is produced, and it equals the one of the two-sided backward."""
+    import window_matmul_kernel as native
+    from window_matmul import unwindow_matmul, window_matmul
+
+    B, M, N, w = 3, 96, 32, 12
+    q0, k0, v0 = (seeded((B, M, N), s, torch.float32).to(device) for s in (31, 32, 33))
+    a0 = seeded((B, M, 2 * w + 1), 34, torch.float32).to(device)
+    first = which == "first"
+
+    q = q0.clone().requires_grad_(first)
+    k = k0.clone().requires_grad_(not first)
+    window_matmul(q, k.transpose(-1, -2), w).square().sum().backward()
+    att = native.window_matmul_forward(q0, k0.transpose(-1, -2), w)
+    gq, gk = native.window_matmul_backward(q0, k0.transpose(-1, -2), w, 2 * att)
+    torch.testing.assert_close(q.grad if first else k.grad, gq if first else gk.transpose(-1, -2), rtol=1e-5, atol=1e-5)
+    assert (k.grad if first else q.grad) is None
+    one = native.window_matmul_backward(q0, k0.transpose(-1, -2), w, 2 * att, first, not first)
+    assert one[1 if first else 0] is None and one[0 if first else 1] is not None
+
+    a = a0.clone().requires_grad_(first)
+    v = v0.clone().requires_grad_(not first)
+    unwindow_matmul(a, v, w).square().sum().backward()
+    out = native.unwindow_matmul_forward(a0, v0, w)
+    ga, gv = native.unwindow_matmul_backward(a0, v0, w, 2 * out)
+    torch.testing.assert_close(a.grad if first else v.grad, ga if first else gv, rtol=1e-5, atol=1e-5)
+    assert (v.grad if first else a.grad) is None
+    one = native.unwindow_matmul_backward(a0, v0, w, 2 * out, need_src=first, need_other=not first)
+    assert one[1 if first else 0] is None and one[0 if first else 1] is not None
