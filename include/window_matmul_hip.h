@@ -33,7 +33,7 @@
 extern "C" {
 #endif
 
-#define WM_ABI_VERSION 1
+#define WM_ABI_VERSION 2
 
 typedef enum wm_dtype {
   WM_DTYPE_F32 = 0,
@@ -108,6 +108,29 @@ int wm_unwindow_matmul_backward(const wm_operand *a, const wm_operand *v, const 
  * aligned rows.  Returns a static string.  No counterpart in the reference. */
 const char *wm_kernel_choice(int op, int64_t B, int64_t M, int64_t N, int64_t w, int dtype,
                              int fast_layout, unsigned flags);
+
+/* Softmax along the band dimension: p[b,i,:] = softmax(scale * a[b,i,:]) over the 2w+1
+ * entries of each row of a (B, M, 2w+1) tensor.  No counterpart in the reference's native
+ * module: it replaces the torch call its callers put between the two ops
+ * (reference tests/test_attention.py:60-61, `att_scores / sqrt(N)` then `softmax(dim=-1)`).
+ * With mask_out_of_range == 0 every entry takes part with the value it holds, as in that
+ * caller (window_matmul leaves +0.0 in entries outside the sequence).  With
+ * mask_out_of_range != 0 entries whose key position i+j-w is outside [0, M) count as
+ * -infinity: their probability and their gradient are +0.0 whatever they hold.
+ * a and p may be the same buffer.  Contiguous, 16-byte aligned tensors of float32 / float16 /
+ * bfloat16 with rows up to ~64 KB get the LDS-staged kernel; anything else a strided one. */
+int wm_band_softmax_forward(const wm_operand *a, const wm_operand *p, int64_t B, int64_t M, int64_t w,
+                            double scale, int mask_out_of_range, int dtype, unsigned flags, void *stream);
+
+/* Backward of the above from the saved probabilities:
+ * grad_a[b,i,j] = scale * p[b,i,j] * (grad_p[b,i,j] - sum_j' p[b,i,j'] * grad_p[b,i,j']).
+ * grad_a may alias grad_p or p.  Same masking rule (masked entries of grad_p are not read). */
+int wm_band_softmax_backward(const wm_operand *p, const wm_operand *grad_p, const wm_operand *grad_a,
+                             int64_t B, int64_t M, int64_t w, double scale, int mask_out_of_range,
+                             int dtype, unsigned flags, void *stream);
+
+/* Name of the kernel the two functions above would use ("staged_softmax" / "strided_softmax"). */
+const char *wm_band_softmax_kernel_choice(int64_t w, int dtype, int contiguous, int backward, unsigned flags);
 
 /* Human-readable name of a wm_status code (static string). */
 const char *wm_status_string(int status);

@@ -11,6 +11,8 @@ Three independent statements of the same mathematics live here:
   129-141, 177-191).
 * ``dense_oracle`` -- dense masked matmul in float64 (``bmm`` then gather /
   scatter then ``bmm``), a different formulation used to pin the restatement.
+* ``softmax_oracle`` -- float64 numpy softmax over the band dimension (the torch step
+  the reference's callers put between the two ops), for the band softmax kernels.
 * ``reference_module`` -- the reference's own CPU path compiled from its
   sources into ``oracle/_ref`` (only where that build exists).
 """
@@ -31,3 +33,4 @@ from .dense_oracle import (  # noqa: F401
     dense_to_band,
 )
 from .reference_module import reference_module  # noqa: F401
+from . import softmax_oracle  # noqa: F401

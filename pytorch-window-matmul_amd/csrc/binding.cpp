@@ -182,6 +182,42 @@ std::tuple<c10::optional<torch::Tensor>, c10::optional<torch::Tensor>> unwindow_
   return std::make_tuple(grad_a, grad_v);
 }
 
+// Softmax over the band dimension, the step callers put between the two ops
+// (reference tests/test_attention.py:60-61); not part of the reference's native module.
+torch::Tensor band_softmax_forward(torch::Tensor src, double scale, bool mask_out_of_range) {
+  check_gpu(src, "A");
+  TORCH_CHECK(src.dim() == 3 && src.size(2) % 2 == 1, "Input mismatch");
+  const int dtype = abi_dtype(src, "band_softmax_forward");
+  at::hip::HIPGuardMasqueradingAsCUDA guard(src.device());
+  auto a = band_friendly(src);
+  auto out = torch::empty_like(a);
+  wm_operand oa = operand(a), oo = operand(out);
+  raise_on_error(wm_band_softmax_forward(&oa, &oo, a.size(0), a.size(1), a.size(2) / 2, scale, mask_out_of_range,
+                                         dtype, 0, current_stream(src)),
+                 "band_softmax_forward");
+  return out;
+}
+
+torch::Tensor band_softmax_backward(torch::Tensor probs, torch::Tensor grad_output, double scale,
+                                    bool mask_out_of_range) {
+  check_gpu(probs, "P");
+  check_gpu(grad_output, "grad_P");
+  TORCH_CHECK(probs.dim() == 3 && probs.size(2) % 2 == 1, "Input mismatch");
+  TORCH_CHECK(grad_output.sizes() == probs.sizes() && grad_output.scalar_type() == probs.scalar_type() &&
+                  grad_output.device() == probs.device(),
+              "Input mismatch");
+  const int dtype = abi_dtype(probs, "band_softmax_backward");
+  at::hip::HIPGuardMasqueradingAsCUDA guard(probs.device());
+  auto p = band_friendly(probs);
+  auto g = band_friendly(grad_output);
+  auto out = torch::empty_like(p);
+  wm_operand op = operand(p), og = operand(g), oo = operand(out);
+  raise_on_error(wm_band_softmax_backward(&op, &og, &oo, p.size(0), p.size(1), p.size(2) / 2, scale,
+                                          mask_out_of_range, dtype, 0, current_stream(probs)),
+                 "band_softmax_backward");
+  return out;
+}
+
 }  // namespace
 
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
@@ -193,5 +229,9 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("unwindow_matmul_backward", &unwindow_matmul_backward, "UnwindowMatmul backward", py::arg("src"),
         py::arg("other"), py::arg("window_size"), py::arg("grad_output"), py::arg("need_src") = true,
         py::arg("need_other") = true);
+  m.def("band_softmax_forward", &band_softmax_forward, "softmax over the band dimension", py::arg("src"),
+        py::arg("scale") = 1.0, py::arg("mask_out_of_range") = false);
+  m.def("band_softmax_backward", &band_softmax_backward, "backward of band_softmax_forward", py::arg("probs"),
+        py::arg("grad_output"), py::arg("scale") = 1.0, py::arg("mask_out_of_range") = false);
   m.def("abi_version", []() { return wm_abi_version(); }, "ABI version of libwindow_matmul_hip.so");
 }

@@ -109,6 +109,35 @@ int wm_unwindow_matmul_backward(const wm_operand *a, const wm_operand *v, const 
   return WM_OK;
 }
 
+int wm_band_softmax_forward(const wm_operand *a, const wm_operand *p, int64_t B, int64_t M, int64_t w, double scale,
+                            int mask_out_of_range, int dtype, unsigned flags, void *stream) {
+  if (int st = check_common(B, M, 0, w, dtype, flags)) return st;
+  if (!(scale == scale)) return WM_ERR_BAD_SHAPE;
+  if (B == 0 || M == 0) return WM_OK;
+  if (missing(a) || missing(p)) return WM_ERR_NULL_POINTER;
+  const Problem prob{B, M, 0, w, dtype, flags, static_cast<hipStream_t>(stream)};
+  return to_status(launch_band_softmax_forward(prob, make_view(a), make_view(p), scale, mask_out_of_range));
+}
+
+int wm_band_softmax_backward(const wm_operand *p, const wm_operand *grad_p, const wm_operand *grad_a, int64_t B,
+                             int64_t M, int64_t w, double scale, int mask_out_of_range, int dtype, unsigned flags,
+                             void *stream) {
+  if (int st = check_common(B, M, 0, w, dtype, flags)) return st;
+  if (!(scale == scale)) return WM_ERR_BAD_SHAPE;
+  if (B == 0 || M == 0) return WM_OK;
+  if (missing(p) || missing(grad_p) || missing(grad_a)) return WM_ERR_NULL_POINTER;
+  const Problem prob{B, M, 0, w, dtype, flags, static_cast<hipStream_t>(stream)};
+  return to_status(launch_band_softmax_backward(prob, make_view(p), make_view(grad_p), make_view(grad_a), scale,
+                                                mask_out_of_range));
+}
+
+const char *wm_band_softmax_kernel_choice(int64_t w, int dtype, int contiguous, int backward, unsigned flags) {
+  if (w < 0 || dtype < WM_DTYPE_F32 || dtype > WM_DTYPE_F64) return "invalid";
+  if (contiguous && !(flags & WM_FLAG_FORCE_STRIDED) && band_softmax_staged(2 * w + 1, dtype, backward != 0))
+    return "staged_softmax";
+  return "strided_softmax";
+}
+
 const char *wm_kernel_choice(int op, int64_t B, int64_t M, int64_t N, int64_t w, int dtype, int fast,
                              unsigned flags) {
   if (op < 1 || op > 3) return "invalid";

@@ -56,6 +56,14 @@ bool f32_supports(int op, int64_t M, int64_t N, int64_t w, int dtype);
 // Pure predicate behind the three functions above (shape/dtype only).
 bool mfma_supports(int op, int64_t B, int64_t M, int64_t N, int64_t w, int dtype);
 
+// Softmax along the band dimension (wm_softmax.hip).  `mask` non-zero treats entries outside
+// the sequence as -infinity.  In-place use (out aliasing an input) is allowed.
+hipError_t launch_band_softmax_forward(const Problem &p, const View &a, const View &out, double scale, int mask);
+hipError_t launch_band_softmax_backward(const Problem &p, const View &probs, const View &grad_probs,
+                                        const View &grad_a, double scale, int mask);
+// Whether rows of length W get the LDS-staged kernel (given contiguous, 16-byte aligned tensors).
+bool band_softmax_staged(int64_t W, int dtype, bool backward);
+
 inline size_t dtype_size(int dtype) {
   switch (dtype) {
     case WM_DTYPE_F32: return 4;

@@ -55,6 +55,11 @@ def lib():
         L.wm_status_string.argtypes = [ctypes.c_int]
         L.wm_kernel_choice.restype = ctypes.c_char_p
         L.wm_kernel_choice.argtypes = [ctypes.c_int, i64, i64, i64, i64, ctypes.c_int, ctypes.c_int, u32]
+        sm_tail = [i64, i64, i64, ctypes.c_double, ctypes.c_int, ctypes.c_int, u32, vp]
+        L.wm_band_softmax_forward.argtypes = [P, P] + sm_tail
+        L.wm_band_softmax_backward.argtypes = [P, P, P] + sm_tail
+        L.wm_band_softmax_kernel_choice.restype = ctypes.c_char_p
+        L.wm_band_softmax_kernel_choice.argtypes = [i64, ctypes.c_int, ctypes.c_int, ctypes.c_int, u32]
         _LIB = L
     return _LIB
 
@@ -109,3 +114,20 @@ def unwindow_backward(a, v, w, go, flags=0, want_a=True, want_v=True):
     _check(lib().wm_unwindow_matmul_backward(op(a), op(v), op(go), op(ga), op(gv), B, M, N, w, DTYPES[v.dtype], flags,
                                             _stream()), "wm_unwindow_matmul_backward")
     return ga, gv
+
+
+def band_softmax_forward(a, scale=1.0, mask=False, flags=0, out=None):
+    """a (B,M,2w+1) -> softmax(scale * a) along the band; out may be a itself."""
+    B, M, W = a.shape
+    p = torch.empty_like(a) if out is None else out
+    _check(lib().wm_band_softmax_forward(op(a), op(p), B, M, W // 2, float(scale), int(mask), DTYPES[a.dtype], flags,
+                                        _stream()), "wm_band_softmax_forward")
+    return p
+
+
+def band_softmax_backward(p, gp, scale=1.0, mask=False, flags=0, out=None):
+    B, M, W = p.shape
+    ga = torch.empty_like(p) if out is None else out
+    _check(lib().wm_band_softmax_backward(op(p), op(gp), op(ga), B, M, W // 2, float(scale), int(mask),
+                                         DTYPES[p.dtype], flags, _stream()), "wm_band_softmax_backward")
+    return ga

@@ -14,10 +14,11 @@ def test_library_exports_every_declared_symbol():
     L = abi.lib()
     names = abi.declared_symbols()
     assert {"wm_window_matmul_forward", "wm_window_matmul_backward", "wm_unwindow_matmul_forward",
-            "wm_unwindow_matmul_backward", "wm_kernel_choice", "wm_status_string", "wm_abi_version"} <= set(names)
+            "wm_unwindow_matmul_backward", "wm_band_softmax_forward", "wm_band_softmax_backward",
+            "wm_band_softmax_kernel_choice", "wm_kernel_choice", "wm_status_string", "wm_abi_version"} <= set(names)
     for name in names:
         assert hasattr(L, name), name
-    assert L.wm_abi_version() == 1
+    assert L.wm_abi_version() == 2
 
 
 def test_argument_validation_happens_on_the_host():
