@@ -154,7 +154,7 @@ def main():
     if not torch.cuda.is_available():
         sys.exit("bench.py: no GPU visible")
     import wm_ctypes as abi
-    from window_matmul import unwindow_matmul, window_matmul
+    from window_matmul import band_softmax, unwindow_matmul, window_matmul
 
     cfg = WORKLOADS[args.workload]
     B, M, N, w = cfg["B"], cfg["M"], cfg["N"], cfg["w"]
@@ -169,9 +169,9 @@ def main():
     q, k, v, go = synth(cfg["qk_scale"]), synth(cfg["qk_scale"]), synth(), synth()
     q.requires_grad_(True), k.requires_grad_(True), v.requires_grad_(True)
 
-    def step():
+    def step(softmax=lambda att: torch.softmax(att, dim=-1)):
         att = window_matmul(q, k.transpose(1, 2), w)
-        probs = torch.softmax(att, dim=-1)
+        probs = softmax(att)
         out = unwindow_matmul(probs, v, w)
         if cfg["backward"]:
             q.grad = k.grad = v.grad = None
@@ -190,6 +190,16 @@ def main():
             step()
         torch.cuda.synchronize()
         ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+        # the same chain with this library's band softmax in place of torch's (one changed line
+        # in caller code; reported beside the drop-in figure, never as `value`)
+        for _ in range(args.warmup):
+            step(band_softmax)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            step(band_softmax)
+        torch.cuda.synchronize()
+        band_ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
 
     # per-kernel timing through the C ABI (one launch per call), same tensors, same stream
     with torch.no_grad():
@@ -216,6 +226,12 @@ def main():
             per_kernel[name] = {"ms": round(ms, 4), "GBps": round(kb / ms / 1e6, 1),
                                 "TFLOPs": round(band_unit_flops(B, M, N, w) / ms / 1e9, 1)}
         softmax_ms = time_gpu(lambda: torch.softmax(att, dim=-1), max(args.steps, 10), 3)
+        band_bytes = att.numel() * es
+        sm_out = torch.empty_like(att)
+        bs_fwd_ms = time_gpu(lambda: abi.band_softmax_forward(att, 1.0, out=sm_out), max(args.steps, 10), 3)
+        bs_bwd_ms = time_gpu(lambda: abi.band_softmax_backward(probs, ga if ga is not None else att, 1.0, out=sm_out),
+                             max(args.steps, 10), 3)
+        del sm_out
         # device-to-device copy of the band as the achievable-bandwidth yardstick
         scratch = torch.empty_like(att)
         copy_ms = time_gpu(lambda: scratch.copy_(att), 20, 3)
@@ -244,6 +260,11 @@ def main():
                      "algorithmic_bytes_per_launch": kb, "avg_launch_ms": per_kernel[dom]["ms"]},
         "kernels": per_kernel,
         "softmax_fwd_ms": round(softmax_ms, 4),
+        "band_softmax": None if args.kernels_only else {
+            "ms_per_step": round(band_ms_per_step, 4), "TFLOPs": round(flops / band_ms_per_step / 1e9, 2),
+            "fwd_ms": round(bs_fwd_ms, 4), "fwd_GBps": round(2 * band_bytes / bs_fwd_ms / 1e6, 1),
+            "bwd_ms": round(bs_bwd_ms, 4), "bwd_GBps": round(3 * band_bytes / bs_bwd_ms / 1e6, 1),
+            "note": "same chain with window_matmul.band_softmax replacing torch.softmax"},
         "copy_yardstick_GBps": round(copy_gbs, 1),
         "kernel_sum_GBps": round(len(per_kernel) * kb / sum(v["ms"] for v in per_kernel.values()) / 1e6, 1),
     }
