@@ -49,7 +49,9 @@ typedef enum wm_status {
   WM_ERR_BAD_DTYPE = 3,        /* dtype is not a wm_dtype value                     */
   WM_ERR_BAD_FLAGS = 4,        /* unknown bit set in flags                          */
   WM_ERR_LAUNCH_FAILED = 5,    /* the HIP runtime rejected a kernel launch          */
-  WM_ERR_NO_DEVICE_CODE = 6    /* the library holds no code object for this GPU     */
+  WM_ERR_NO_DEVICE_CODE = 6,   /* the library holds no code object for this GPU     */
+  WM_ERR_UNSUPPORTED = 7       /* a fused entry point has no kernel for this shape, dtype or layout;
+                                  nothing was launched: run the chain of the separate ops instead */
 } wm_status;
 
 /* Kernel selection.  0 lets the library choose per (shape, dtype, layout). */
@@ -131,6 +133,28 @@ int wm_band_softmax_backward(const wm_operand *p, const wm_operand *grad_p, cons
 
 /* Name of the kernel the two functions above would use ("staged_softmax" / "strided_softmax"). */
 const char *wm_band_softmax_kernel_choice(int64_t w, int dtype, int contiguous, int backward, unsigned flags);
+
+/* Fused window attention, forward:
+ *   o = unwindow_matmul(softmax(scale * window_matmul(q, k^T, w), -1), v, w)
+ * in one kernel; the (B, M, 2w+1) band never reaches memory.  No counterpart in the
+ * reference's native module: it fuses the chain its callers write
+ * (reference tests/test_attention.py:57-63) and keeps that chain's semantics.  With
+ * mask_out_of_range == 0 the band entries outside the sequence take part in the softmax
+ * with score 0, as they do when window_matmul's +0.0 entries go through torch.softmax, and
+ * contribute no value row; with mask_out_of_range != 0 they are left out.
+ * q, k, v, o are (B, M, N) operands (k holds key ROWS here, unlike the (B, N, M) view the
+ * window op takes).  lse, if not NULL, receives the natural-log sum of exponentials of every
+ * row as float32 (B * M values, contiguous) for use by a backward pass.
+ * Returns WM_ERR_UNSUPPORTED, having launched nothing, unless dtype is float16 / bfloat16,
+ * N is a multiple of 32 up to 128, w >= 1, scale > 0 and all four operands have unit column
+ * stride and 16-byte aligned rows (see wm_window_attention_supported). */
+int wm_window_attention_forward(const wm_operand *q, const wm_operand *k, const wm_operand *v,
+                                const wm_operand *o, float *lse, int64_t B, int64_t M, int64_t N,
+                                int64_t w, double scale, int mask_out_of_range, int dtype,
+                                unsigned flags, void *stream);
+
+/* 1 if the fused kernel exists for this shape, dtype and scale (layout aside), else 0. */
+int wm_window_attention_supported(int64_t M, int64_t N, int64_t w, int dtype, double scale);
 
 /* Human-readable name of a wm_status code (static string). */
 const char *wm_status_string(int status);

@@ -13,6 +13,8 @@ Three independent statements of the same mathematics live here:
   scatter then ``bmm``), a different formulation used to pin the restatement.
 * ``softmax_oracle`` -- float64 numpy softmax over the band dimension (the torch step
   the reference's callers put between the two ops), for the band softmax kernels.
+* ``attention_oracle`` -- the callers' chain window_matmul -> softmax -> unwindow_matmul
+  composed from the two above, for the fused attention kernels.
 * ``reference_module`` -- the reference's own CPU path compiled from its
   sources into ``oracle/_ref`` (only where that build exists).
 """
@@ -34,3 +36,4 @@ from .dense_oracle import (  # noqa: F401
 )
 from .reference_module import reference_module  # noqa: F401
 from . import softmax_oracle  # noqa: F401
+from . import attention_oracle  # noqa: F401

@@ -131,6 +131,25 @@ int wm_band_softmax_backward(const wm_operand *p, const wm_operand *grad_p, cons
                                                 mask_out_of_range));
 }
 
+int wm_window_attention_forward(const wm_operand *q, const wm_operand *k, const wm_operand *v, const wm_operand *o,
+                                float *lse, int64_t B, int64_t M, int64_t N, int64_t w, double scale,
+                                int mask_out_of_range, int dtype, unsigned flags, void *stream) {
+  if (int st = check_common(B, M, N, w, dtype, flags)) return st;
+  if (!(scale == scale)) return WM_ERR_BAD_SHAPE;
+  if (B == 0 || M == 0) return WM_OK;
+  if (missing(q) || missing(k) || missing(v) || missing(o)) return WM_ERR_NULL_POINTER;
+  const Problem prob{B, M, N, w, dtype, flags, static_cast<hipStream_t>(stream)};
+  hipError_t err = hipSuccess;
+  if (!try_launch_attention_forward(prob, make_view(q), make_view(k), make_view(v), make_view(o), lse, scale,
+                                    mask_out_of_range, &err))
+    return WM_ERR_UNSUPPORTED;
+  return to_status(err);
+}
+
+int wm_window_attention_supported(int64_t M, int64_t N, int64_t w, int dtype, double scale) {
+  return attention_supports(M, N, w, dtype, scale) ? 1 : 0;
+}
+
 const char *wm_band_softmax_kernel_choice(int64_t w, int dtype, int contiguous, int backward, unsigned flags) {
   if (w < 0 || dtype < WM_DTYPE_F32 || dtype > WM_DTYPE_F64) return "invalid";
   if (contiguous && !(flags & WM_FLAG_FORCE_STRIDED) && band_softmax_staged(2 * w + 1, dtype, backward != 0))
@@ -167,6 +186,7 @@ const char *wm_status_string(int status) {
     case WM_ERR_BAD_DTYPE: return "unknown dtype";
     case WM_ERR_BAD_FLAGS: return "unknown flag bit";
     case WM_ERR_LAUNCH_FAILED: return "kernel launch failed";
+    case WM_ERR_UNSUPPORTED: return "this entry point has no kernel for the given shape, dtype or layout";
     case WM_ERR_NO_DEVICE_CODE: return "no device code for this GPU (library is built for gfx950)";
     default: return "unknown status";
   }

@@ -1,0 +1,289 @@
+// Fused window attention, forward:  O = unwindow_matmul(softmax(scale * window_matmul(Q, K^T)), V)
+// in one kernel, without the (B, M, 2w+1) band ever reaching memory.  It reproduces the chain the
+// reference's callers write (reference tests/test_attention.py:57-63), including its treatment of
+// band entries outside the sequence: window_matmul leaves +0.0 there, so without masking they take
+// part in the softmax with score 0 (and contribute nothing to the output); with masking they are
+// left out.  Besides O the kernel stores the log-sum-exp of every row, which is all a recomputing
+// backward needs.
+//
+// One workgroup owns 128 queries (32 per wavefront) and walks over the keys its band can reach in
+// chunks of 64, staged in LDS (K and V, double buffered) and shared by its four wavefronts.
+// Per wavefront and block of 32 keys:
+//   S^T = K_blk . Q^T         v_mfma_f32_32x32x16, A = key rows from LDS, B = the wavefront's
+//                             queries, held in registers for the whole kernel.  In the result a
+//                             lane owns ONE query (lane % 32) and 16 of the 32 keys, so the row
+//                             maximum and sum of the softmax are in-lane loops plus one exchange
+//                             with lane ^ 32.
+//   P^T = exp2(c S^T - m)     online softmax; the running maximum m is only raised when a block
+//                             exceeds it by more than 8 (in log2 units), so most blocks skip the
+//                             rescaling of O.  Rounded to 16 bits, P^T is already laid out as the
+//                             B operand of the next product.
+//   O^T += V_blk^T . P^T      A = V columns, fetched from the row-major LDS tile with
+//                             ds_read_b64_tr_b16.
+// Blocks that lie entirely outside a wavefront's band are skipped, blocks entirely inside it run
+// without any masking arithmetic.
+#include "wm_mfma_common.hpp"
+
+#include <type_traits>
+
+namespace wm {
+namespace {
+
+constexpr int AT_TM = 128;  // queries per workgroup
+constexpr int AT_KC = 64;   // keys per chunk
+constexpr float kRaiseStep = 8.0f;
+constexpr float kLog2eF = 1.4426950408889634f;
+constexpr float kLn2F = 0.6931471805599453f;
+
+// Transposed operand fetch like lds_read_transposed, but for the k order that the accumulator
+// layout of the first product dictates: the lane with half = lane / 32 gets rows
+// k0 + 4 half + {0..3} and k0 + 8 + 4 half + {0..3}.
+__device__ __forceinline__ u32x4 lds_read_transposed_split(const uint16_t *mat, int stride, int k0, int x0, int lane) {
+  const int s = lane & 15, grp = lane >> 4;
+  const int xb = x0 + 16 * (grp & 1) + 4 * (s & 3);
+  const int kb = k0 + 4 * (grp >> 1) + (s >> 2);
+  typedef s16x4 __attribute__((address_space(3))) * lds_ptr;
+  const uint16_t *p0 = mat + kb * stride + xb;
+  const uint16_t *p1 = p0 + 8 * stride;
+  const s16x4 a = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(p0));
+  const s16x4 b = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(p1));
+  const u32x2 ua = __builtin_bit_cast(u32x2, a), ub = __builtin_bit_cast(u32x2, b);
+  u32x4 r = {ua[0], ua[1], ub[0], ub[1]};
+  return r;
+}
+
+// Value of the same register in lane ^ 32 combined with the own one.
+__device__ __forceinline__ float across_halves_max(float v) {
+  const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+__device__ __forceinline__ float across_halves_sum(float v) {
+  const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+
+template <typename T, int NB, bool MASK>
+__global__ __launch_bounds__(kThreads, 2) void attention_forward_kernel(
+    const uint16_t *__restrict__ Q, const uint16_t *__restrict__ K, const uint16_t *__restrict__ V,
+    uint16_t *__restrict__ O, float *__restrict__ L, int B, int M, int w, int nblk, float c, int64_t qsb, int64_t qsr,
+    int64_t ksb, int64_t ksr, int64_t vsb, int64_t vsr, int64_t osb, int64_t osr) {
+  constexpr int N = 32 * NB, NK = N / 16;
+  constexpr int KS = N + 8;   // key rows 16 (mod 128) bytes apart in banks: conflict-free b128 reads
+  constexpr int VS = N + 16;  // value rows 32 (mod 128) bytes apart: what the transposed reads want
+  constexpr int SLOTS = AT_KC * N / 8 / kThreads;  // 16-byte pieces per thread, chunk and tensor
+  __shared__ __attribute__((aligned(16))) uint16_t k_lds[2][AT_KC * KS];
+  __shared__ __attribute__((aligned(16))) uint16_t v_lds[2][AT_KC * VS];
+
+  int b, blk;
+  if (!decode_block(nblk, B, &b, &blk)) return;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, half = lane >> 5;
+  const int i0 = blk * AT_TM;
+  const int qw0 = i0 + 32 * wave;     // first query of this wavefront
+  const int qi = qw0 + (lane & 31);   // this lane's query
+  const uint16_t *Kb = K + (int64_t)b * ksb;
+  const uint16_t *Vb = V + (int64_t)b * vsb;
+
+  // B operand of the first product: the wavefront's 32 queries, all of N, in registers
+  u32x4 qf[NK];
+  {
+    const uint16_t *qr = Q + (int64_t)b * qsb + (int64_t)qi * qsr + 8 * half;
+#pragma unroll
+    for (int ks = 0; ks < NK; ++ks) qf[ks] = load_row_chunk(qr + 16 * ks, Q, qi < M);
+  }
+
+  const int kc_lo = max(i0 - w, 0) / AT_KC;
+  const int kc_hi = min(i0 + AT_TM - 1 + w, M - 1) / AT_KC;
+
+  // loader slots: row and column of the 16-byte piece this thread moves, per chunk
+  int l_row[SLOTS], l_col[SLOTS];
+#pragma unroll
+  for (int u = 0; u < SLOTS; ++u) {
+    const int p = tid + kThreads * u;
+    l_row[u] = p / (N / 8);
+    l_col[u] = (p % (N / 8)) * 8;
+  }
+  u32x4 kreg[SLOTS], vreg[SLOTS];
+  auto fetch = [&](int kc) {  // loads only; rows past the sequence or the last chunk come from a safe address
+#pragma unroll
+    for (int u = 0; u < SLOTS; ++u) {
+      const int key = kc * AT_KC + l_row[u];
+      const bool ok = key < M && kc <= kc_hi;
+      kreg[u] = fetch_row_chunk(Kb + (int64_t)key * ksr + l_col[u], K, ok);
+      vreg[u] = fetch_row_chunk(Vb + (int64_t)key * vsr + l_col[u], V, ok);
+    }
+  };
+  auto stash = [&](int kc, int buf) {
+#pragma unroll
+    for (int u = 0; u < SLOTS; ++u) {
+      const int key = kc * AT_KC + l_row[u];
+      const bool ok = key < M && kc <= kc_hi;
+      *reinterpret_cast<u32x4 *>(&k_lds[buf][l_row[u] * KS + l_col[u]]) = mask_row_chunk(kreg[u], ok);
+      *reinterpret_cast<u32x4 *>(&v_lds[buf][l_row[u] * VS + l_col[u]]) = mask_row_chunk(vreg[u], ok);
+    }
+  };
+
+  f32x16 o[NB];
+#pragma unroll
+  for (int hb = 0; hb < NB; ++hb)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) o[hb][v] = 0.0f;
+  float m_used = -1.0e30f;  // running maximum in log2 units (finite, so that -inf scores give exp2(-inf) = 0)
+  float l_part = 0.0f;      // this lane's share of the running sum
+  const float ninf = -__builtin_huge_valf();
+
+  auto block = [&](int buf, int kb, int c0, auto edge) {
+    constexpr bool EDGE = decltype(edge)::value;
+    f32x16 s;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) s[v] = 0.0f;
+    const uint16_t *krow = &k_lds[buf][(32 * kb + (lane & 31)) * KS + 8 * half];
+#pragma unroll
+    for (int ks = 0; ks < NK; ++ks) s = Mma<T>::run(*reinterpret_cast<const u32x4 *>(krow + 16 * ks), qf[ks], s);
+    // accumulator v of this lane: key c0 + 8 (v / 4) + 4 half + v % 4, query qi
+    if (EDGE) {
+      const int d0 = c0 + 4 * half - qi;   // key - query for v = 0
+      const int klim = M - c0 - 4 * half;  // keys of this lane with offset below klim exist
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int ofs = 8 * (v / 4) + v % 4;
+        const bool valid = (unsigned)(d0 + ofs + w) <= (unsigned)(2 * w) && ofs < klim;
+        s[v] = valid ? s[v] : ninf;
+      }
+    }
+    float bm = s[0];
+#pragma unroll
+    for (int v = 1; v < 16; ++v) bm = fmaxf(bm, s[v]);
+    bm = across_halves_max(bm) * c;
+    const bool raise = bm > m_used + kRaiseStep;
+    if (__builtin_amdgcn_ballot_w64(raise) != 0) {
+      const float m_new = raise ? bm : m_used;
+      const float alpha = __builtin_amdgcn_exp2f(m_used - m_new);
+      m_used = m_new;
+      l_part *= alpha;
+#pragma unroll
+      for (int hb = 0; hb < NB; ++hb)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) o[hb][v] *= alpha;
+    }
+    float p[16];
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+      p[v] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[v], c, -m_used));
+      l_part += p[v];
+    }
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      const u32x4 pf = {Mma<T>::pack2(p[8 * t + 0], p[8 * t + 1]), Mma<T>::pack2(p[8 * t + 2], p[8 * t + 3]),
+                        Mma<T>::pack2(p[8 * t + 4], p[8 * t + 5]), Mma<T>::pack2(p[8 * t + 6], p[8 * t + 7])};
+#pragma unroll
+      for (int hb = 0; hb < NB; ++hb) {
+        const u32x4 vf = lds_read_transposed_split(v_lds[buf], VS, 32 * kb + 16 * t, 32 * hb, lane);
+        o[hb] = Mma<T>::run(vf, pf, o[hb]);
+      }
+    }
+  };
+
+  fetch(kc_lo);
+  stash(kc_lo, 0);
+  __syncthreads();
+  for (int kc = kc_lo; kc <= kc_hi; ++kc) {
+    const int buf = (kc - kc_lo) & 1;
+    fetch(kc + 1);
+#pragma unroll
+    for (int kb = 0; kb < 2; ++kb) {
+      const int c0 = kc * AT_KC + 32 * kb;
+      // wave-uniform: skip blocks outside this wavefront's band or the sequence
+      if (c0 + 31 < qw0 - w || c0 > qw0 + 31 + w || c0 >= M) continue;
+      const bool interior = c0 >= qw0 + 31 - w && c0 + 31 <= qw0 + w && c0 + 31 < M;
+      if (interior)
+        block(buf, kb, c0, std::false_type());
+      else
+        block(buf, kb, c0, std::true_type());
+    }
+    stash(kc + 1, buf ^ 1);
+    __syncthreads();
+  }
+
+  float l = across_halves_sum(l_part);
+  if (!MASK) {
+    // Band entries outside the sequence: score 0 each, no value row (wave-uniform test first).
+    if (qw0 < w || qw0 + 31 + w > M - 1) {
+      const int n_out = max(0, w - qi) + max(0, qi + w - (M - 1));
+      if (n_out > 0) {
+        const float m_new = fmaxf(m_used, 0.0f);
+        const float alpha = __builtin_amdgcn_exp2f(m_used - m_new);
+        l = l * alpha + (float)n_out * __builtin_amdgcn_exp2f(-m_new);
+        m_used = m_new;
+#pragma unroll
+        for (int hb = 0; hb < NB; ++hb)
+#pragma unroll
+          for (int v = 0; v < 16; ++v) o[hb][v] *= alpha;
+      }
+    }
+  }
+  if (qi >= M) return;
+  const float inv = 1.0f / l;
+  uint16_t *orow = O + (int64_t)b * osb + (int64_t)qi * osr + 4 * half;
+#pragma unroll
+  for (int hb = 0; hb < NB; ++hb)
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      const u32x2 out = {Mma<T>::pack2(o[hb][4 * g] * inv, o[hb][4 * g + 1] * inv),
+                         Mma<T>::pack2(o[hb][4 * g + 2] * inv, o[hb][4 * g + 3] * inv)};
+      *reinterpret_cast<u32x2 *>(orow + 32 * hb + 8 * g) = out;
+    }
+  if (L != nullptr && half == 0) L[(int64_t)b * M + qi] = (m_used + __builtin_amdgcn_logf(l)) * kLn2F;
+}
+
+template <typename T, int NB>
+hipError_t launch_forward(const Problem &p, const View &q, const View &k, const View &v, const View &o, float *lse,
+                          double scale, int mask) {
+  const int nblk = (int)((p.M + AT_TM - 1) / AT_TM);
+  const int64_t groups = (p.B + 7) / 8;
+  if (groups * 8 * nblk > 0x7fffffff) return hipErrorInvalidValue;
+  const dim3 grid((unsigned)(groups * 8 * nblk)), block(kThreads);
+  const float c = (float)(scale * 1.4426950408889634);
+#define WM_AT(MASKED)                                                                                                 \
+  hipLaunchKernelGGL((attention_forward_kernel<T, NB, MASKED>), grid, block, 0, p.stream, (const uint16_t *)q.data,   \
+                     (const uint16_t *)k.data, (const uint16_t *)v.data, (uint16_t *)o.data, lse, (int)p.B, (int)p.M, \
+                     (int)p.w, nblk, c, q.sb, q.sr, k.sb, k.sr, v.sb, v.sr, o.sb, o.sr)
+  if (mask)
+    WM_AT(true);
+  else
+    WM_AT(false);
+#undef WM_AT
+  return hipGetLastError();
+}
+
+template <typename T>
+hipError_t forward_by_width(const Problem &p, const View &q, const View &k, const View &v, const View &o, float *lse,
+                            double scale, int mask) {
+  switch (p.N / 32) {
+    case 1: return launch_forward<T, 1>(p, q, k, v, o, lse, scale, mask);
+    case 2: return launch_forward<T, 2>(p, q, k, v, o, lse, scale, mask);
+    case 3: return launch_forward<T, 3>(p, q, k, v, o, lse, scale, mask);
+    default: return launch_forward<T, 4>(p, q, k, v, o, lse, scale, mask);
+  }
+}
+
+}  // namespace
+
+bool attention_supports(int64_t M, int64_t N, int64_t w, int dtype, double scale) {
+  if (dtype != WM_DTYPE_BF16 && dtype != WM_DTYPE_F16) return false;
+  if (N % 32 != 0 || N < 32 || N > 128) return false;
+  if (M < 1 || w < 1 || w > 0x3fffffff) return false;
+  return scale > 0.0 && scale < 1.0e30;
+}
+
+bool try_launch_attention_forward(const Problem &p, const View &q, const View &k, const View &v, const View &o,
+                                  float *lse, double scale, int mask, hipError_t *err) {
+  if (p.flags & WM_FLAG_FORCE_STRIDED) return false;
+  if (!attention_supports(p.M, p.N, p.w, p.dtype, scale)) return false;
+  if (!fast_layout(q, p.dtype) || !fast_layout(k, p.dtype) || !fast_layout(v, p.dtype) || !fast_layout(o, p.dtype))
+    return false;
+  *err = p.dtype == WM_DTYPE_BF16 ? forward_by_width<bf16_t>(p, q, k, v, o, lse, scale, mask)
+                                  : forward_by_width<f16_t>(p, q, k, v, o, lse, scale, mask);
+  return true;
+}
+
+}  // namespace wm

@@ -64,6 +64,12 @@ hipError_t launch_band_softmax_backward(const Problem &p, const View &probs, con
 // Whether rows of length W get the LDS-staged kernel (given contiguous, 16-byte aligned tensors).
 bool band_softmax_staged(int64_t W, int dtype, bool backward);
 
+// Fused window attention forward (wm_attention.hip): q, k, v, o row-major (B,M,N) views, lse an
+// optional float32 (B,M) buffer.  Returns false when the kernel does not take the problem.
+bool attention_supports(int64_t M, int64_t N, int64_t w, int dtype, double scale);
+bool try_launch_attention_forward(const Problem &p, const View &q, const View &k, const View &v, const View &o,
+                                  float *lse, double scale, int mask, hipError_t *err);
+
 inline size_t dtype_size(int dtype) {
   switch (dtype) {
     case WM_DTYPE_F32: return 4;

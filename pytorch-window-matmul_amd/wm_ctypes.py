@@ -60,6 +60,9 @@ def lib():
         L.wm_band_softmax_backward.argtypes = [P, P, P] + sm_tail
         L.wm_band_softmax_kernel_choice.restype = ctypes.c_char_p
         L.wm_band_softmax_kernel_choice.argtypes = [i64, ctypes.c_int, ctypes.c_int, ctypes.c_int, u32]
+        L.wm_window_attention_forward.argtypes = [P, P, P, P, vp, i64, i64, i64, i64, ctypes.c_double, ctypes.c_int,
+                                                  ctypes.c_int, u32, vp]
+        L.wm_window_attention_supported.argtypes = [i64, i64, i64, ctypes.c_int, ctypes.c_double]
         _LIB = L
     return _LIB
 
@@ -131,3 +134,18 @@ def band_softmax_backward(p, gp, scale=1.0, mask=False, flags=0, out=None):
     _check(lib().wm_band_softmax_backward(op(p), op(gp), op(ga), B, M, W // 2, float(scale), int(mask),
                                          DTYPES[p.dtype], flags, _stream()), "wm_band_softmax_backward")
     return ga
+
+
+UNSUPPORTED = 7
+
+
+def attention_forward(q, k, v, w, scale=1.0, mask=False, flags=0, want_lse=True):
+    """q, k, v (B,M,N) row-major (k holds key rows) -> (o (B,M,N), lse (B,M) float32 or None)."""
+    B, M, N = q.shape
+    o = torch.empty(B, M, N, dtype=q.dtype, device=q.device)
+    lse = torch.empty(B, M, dtype=torch.float32, device=q.device) if want_lse else None
+    _check(lib().wm_window_attention_forward(op(q), op(k), op(v), op(o),
+                                            ctypes.c_void_p(lse.data_ptr()) if want_lse else None, B, M, N, w,
+                                            float(scale), int(mask), DTYPES[q.dtype], flags, _stream()),
+           "wm_window_attention_forward")
+    return o, lse

@@ -1,0 +1,90 @@
+"""GPU parity of the fused window attention against the float64 oracle of the callers' chain
+(reference tests/test_attention.py:57-63) on the same seeded, rounded inputs, and against the
+chain of this library's separate ops at the benchmark shape.
+
+Tolerance: float16 / bfloat16 2e-2 (relative and absolute) on outputs and gradients; the
+log-sum-exp is float32 and checked to 2e-3."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+import wm_ctypes as abi
+from oracle import attention_oracle as ao
+from conftest import seeded
+
+pytestmark = pytest.mark.gpu
+
+TOL = dict(rtol=2e-2, atol=2e-2)
+# (B, M, N, w): one short tile, ragged tiles, w larger than the sequence, bands that cross several
+# 64-key chunks, every supported head width
+CASES = [
+    (2, 1, 32, 1), (3, 37, 64, 6), (2, 128, 64, 4), (2, 129, 64, 64), (1, 257, 96, 33), (2, 100, 128, 49),
+    (1, 300, 64, 150), (2, 65, 32, 100), (1, 513, 64, 256), (9, 260, 64, 96), (2, 600, 128, 16), (2, 1030, 64, 12),
+    (1, 1000, 64, 300), (3, 200, 64, 1),
+]
+DTYPES = [torch.bfloat16, torch.float16]
+
+
+def close(got, want):
+    torch.testing.assert_close(got.detach().cpu().to(torch.float64), torch.from_numpy(np.asarray(want)), **TOL)
+
+
+@pytest.mark.parametrize("mask", [False, True], ids=["zero_filled", "masked"])
+@pytest.mark.parametrize("dtype", DTYPES, ids=lambda d: str(d).split(".")[-1])
+@pytest.mark.parametrize("case", CASES, ids=lambda c: "B%d_M%d_N%d_w%d" % c)
+def test_forward_matches_oracle(device, case, dtype, mask):
+    B, M, N, w = case
+    scale = 1.0 / math.sqrt(N)
+    q, k, v = (seeded((B, M, N), s, dtype) for s in (51, 52, 53))
+    want_o, want_lse = ao.window_attention_forward(q, k, v, w, scale, mask)
+    o, lse = abi.attention_forward(q.to(device), k.to(device), v.to(device), w, scale, mask)
+    close(o, want_o)
+    torch.testing.assert_close(lse.cpu().to(torch.float64), torch.from_numpy(want_lse), rtol=2e-3, atol=2e-3)
+
+
+def test_large_scores_and_strided_views(device):
+    """Scores far from zero (running maximum raised many times, both signs) and head-major views."""
+    B, H, M, N, w = 2, 3, 300, 64, 40
+    big = seeded((B, M, H * N), 54, torch.bfloat16, 3.0).to(device)
+    q = big.view(B, M, H, N).transpose(1, 2).reshape(B * H, M, N)  # copies; the next two stay views
+    kv = seeded((B * H, M, 2 * N), 55, torch.bfloat16, 3.0).to(device)
+    k, v = kv[:, :, :N], kv[:, :, N:]
+    assert not k.is_contiguous()
+    for mask in (False, True):
+        want_o, want_lse = ao.window_attention_forward(q.cpu(), k.cpu(), v.cpu(), w, 1.0, mask)
+        o, lse = abi.attention_forward(q, k, v, w, 1.0, mask)
+        close(o, want_o)
+        torch.testing.assert_close(lse.cpu().to(torch.float64), torch.from_numpy(want_lse), rtol=2e-3, atol=2e-3)
+
+
+def test_unsupported_shapes_are_refused(device):
+    q = seeded((2, 64, 48), 56, torch.bfloat16).to(device)
+    with pytest.raises(RuntimeError, match="no kernel"):
+        abi.attention_forward(q, q, q, 4)
+    q = seeded((2, 64, 64), 56, torch.float32).to(device)
+    with pytest.raises(RuntimeError, match="no kernel"):
+        abi.attention_forward(q, q, q, 4)
+    L = abi.lib()
+    assert L.wm_window_attention_supported(4096, 64, 256, abi.DTYPES[torch.bfloat16], 0.125) == 1
+    assert L.wm_window_attention_supported(4096, 64, 256, abi.DTYPES[torch.bfloat16], -0.125) == 0
+    assert L.wm_window_attention_supported(4096, 80, 256, abi.DTYPES[torch.bfloat16], 0.125) == 0
+    assert L.wm_window_attention_supported(4096, 64, 0, abi.DTYPES[torch.bfloat16], 0.125) == 0
+
+
+def test_benchmark_shape_against_separate_ops(device):
+    """B=96 M=4096 N=64 w=256 bfloat16: the fused forward against window_matmul -> softmax ->
+    unwindow_matmul of this library (themselves checked against the oracle elsewhere)."""
+    from window_matmul import unwindow_matmul, window_matmul
+
+    B, M, N, w = 96, 4096, 64, 256
+    g = torch.Generator().manual_seed(7)
+    q, k, v = ((torch.randn(B, M, N, generator=g) * s).to(torch.bfloat16).to(device) for s in (1.0, 1.0, 1.0))
+    scale = 1.0 / math.sqrt(N)
+    o, lse = abi.attention_forward(q, k, v, w, scale)
+    att = window_matmul(q, k.transpose(1, 2), w).float() * scale
+    want = unwindow_matmul(torch.softmax(att, -1).to(torch.bfloat16), v, w)
+    torch.testing.assert_close(o.float(), want.float(), **TOL)
+    torch.testing.assert_close(lse, torch.logsumexp(att, -1), rtol=2e-3, atol=2e-3)
+    assert torch.isfinite(o).all()
