@@ -153,7 +153,21 @@ int wm_window_attention_forward(const wm_operand *q, const wm_operand *k, const 
                                 int64_t w, double scale, int mask_out_of_range, int dtype,
                                 unsigned flags, void *stream);
 
-/* 1 if the fused kernel exists for this shape, dtype and scale (layout aside), else 0. */
+/* Backward of wm_window_attention_forward by recomputation: from q, k, v, the forward's o and
+ * lse, and the upstream gradient grad_o, writes grad_q, grad_k, grad_v (all (B, M, N) operands,
+ * k and grad_k as key rows).  delta is a caller-owned float32 workspace of B * M values (it
+ * receives sum_h grad_o * o per row).  The masking choice of the forward is carried by lse and
+ * needs no argument here.  Two kernels are enqueued on the stream; no atomics, so results are
+ * reproducible run to run.  Same support rule and WM_ERR_UNSUPPORTED behaviour as the forward.
+ * No counterpart in the reference's native module (see the forward). */
+int wm_window_attention_backward(const wm_operand *q, const wm_operand *k, const wm_operand *v,
+                                 const wm_operand *o, const float *lse, const wm_operand *grad_o,
+                                 const wm_operand *grad_q, const wm_operand *grad_k,
+                                 const wm_operand *grad_v, float *delta, int64_t B, int64_t M,
+                                 int64_t N, int64_t w, double scale, int dtype, unsigned flags,
+                                 void *stream);
+
+/* 1 if the fused kernels exist for this shape, dtype and scale (layout aside), else 0. */
 int wm_window_attention_supported(int64_t M, int64_t N, int64_t w, int dtype, double scale);
 
 /* Human-readable name of a wm_status code (static string). */

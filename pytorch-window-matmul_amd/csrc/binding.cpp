@@ -218,6 +218,72 @@ torch::Tensor band_softmax_backward(torch::Tensor probs, torch::Tensor grad_outp
   return out;
 }
 
+// Fused window attention (no counterpart in the reference's native module): forward returns
+// (o, lse); q, k, v are (B, M, N) with k holding key rows.  Raises when the fused kernels do not
+// cover the problem; window_attention_supported() lets the caller choose the separate ops first.
+bool window_attention_supported(torch::Tensor q, int64_t window_size, double scale) {
+  if (q.dim() != 3 || !q.device().is_cuda()) return false;
+  int dtype;
+  switch (q.scalar_type()) {
+    case at::kHalf: dtype = WM_DTYPE_F16; break;
+    case at::kBFloat16: dtype = WM_DTYPE_BF16; break;
+    default: return false;
+  }
+  return wm_window_attention_supported(q.size(1), q.size(2), window_size, dtype, scale) != 0;
+}
+
+void check_attention_inputs(const torch::Tensor &q, const torch::Tensor &k, const torch::Tensor &v) {
+  check_gpu(q, "Q");
+  check_gpu(k, "K");
+  check_gpu(v, "V");
+  TORCH_CHECK(q.dim() == 3 && k.sizes() == q.sizes() && v.sizes() == q.sizes(), "Input mismatch");
+  TORCH_CHECK(k.scalar_type() == q.scalar_type() && v.scalar_type() == q.scalar_type(), "Input mismatch");
+  TORCH_CHECK(k.device() == q.device() && v.device() == q.device(), "Input mismatch");
+}
+
+std::tuple<torch::Tensor, torch::Tensor> window_attention_forward(torch::Tensor q, torch::Tensor k, torch::Tensor v,
+                                                                  int64_t window_size, double scale,
+                                                                  bool mask_out_of_range) {
+  check_attention_inputs(q, k, v);
+  const int dtype = abi_dtype(q, "window_attention_forward");
+  at::hip::HIPGuardMasqueradingAsCUDA guard(q.device());
+  const int64_t B = q.size(0), M = q.size(1), N = q.size(2);
+  auto qq = vector_friendly(q), kk = vector_friendly(k), vv = vector_friendly(v);
+  auto o = torch::empty({B, M, N}, q.options());
+  auto lse = torch::empty({B, M}, q.options().dtype(at::kFloat));
+  wm_operand oq = operand(qq), ok = operand(kk), ov = operand(vv), oo = operand(o);
+  raise_on_error(wm_window_attention_forward(&oq, &ok, &ov, &oo, lse.data_ptr<float>(), B, M, N, window_size, scale,
+                                             mask_out_of_range, dtype, 0, current_stream(q)),
+                 "window_attention_forward");
+  return std::make_tuple(o, lse);
+}
+
+std::tuple<torch::Tensor, torch::Tensor, torch::Tensor> window_attention_backward(
+    torch::Tensor q, torch::Tensor k, torch::Tensor v, torch::Tensor o, torch::Tensor lse, torch::Tensor grad_output,
+    int64_t window_size, double scale) {
+  check_attention_inputs(q, k, v);
+  check_grad(grad_output, q, q.sizes().vec());
+  check_grad(o, q, q.sizes().vec());
+  TORCH_CHECK(lse.device() == q.device() && lse.scalar_type() == at::kFloat && lse.dim() == 2 &&
+                  lse.size(0) == q.size(0) && lse.size(1) == q.size(1) && lse.is_contiguous(),
+              "Input mismatch");
+  const int dtype = abi_dtype(q, "window_attention_backward");
+  at::hip::HIPGuardMasqueradingAsCUDA guard(q.device());
+  const int64_t B = q.size(0), M = q.size(1), N = q.size(2);
+  auto qq = vector_friendly(q), kk = vector_friendly(k), vv = vector_friendly(v), oo = vector_friendly(o),
+       go = vector_friendly(grad_output);
+  auto gq = torch::empty({B, M, N}, q.options()), gk = torch::empty({B, M, N}, q.options()),
+       gv = torch::empty({B, M, N}, q.options());
+  auto delta = torch::empty({B, M}, lse.options());
+  wm_operand a = operand(qq), b = operand(kk), c = operand(vv), d = operand(oo), e = operand(go), f = operand(gq),
+             g = operand(gk), h = operand(gv);
+  raise_on_error(wm_window_attention_backward(&a, &b, &c, &d, lse.data_ptr<float>(), &e, &f, &g, &h,
+                                              delta.data_ptr<float>(), B, M, N, window_size, scale, dtype, 0,
+                                              current_stream(q)),
+                 "window_attention_backward");
+  return std::make_tuple(gq, gk, gv);
+}
+
 }  // namespace
 
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
@@ -233,5 +299,13 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
         py::arg("scale") = 1.0, py::arg("mask_out_of_range") = false);
   m.def("band_softmax_backward", &band_softmax_backward, "backward of band_softmax_forward", py::arg("probs"),
         py::arg("grad_output"), py::arg("scale") = 1.0, py::arg("mask_out_of_range") = false);
+  m.def("window_attention_supported", &window_attention_supported, "whether the fused attention kernels cover q",
+        py::arg("q"), py::arg("window_size"), py::arg("scale"));
+  m.def("window_attention_forward", &window_attention_forward, "fused window attention forward -> (o, lse)",
+        py::arg("q"), py::arg("k"), py::arg("v"), py::arg("window_size"), py::arg("scale"),
+        py::arg("mask_out_of_range") = false);
+  m.def("window_attention_backward", &window_attention_backward, "fused window attention backward -> (gq, gk, gv)",
+        py::arg("q"), py::arg("k"), py::arg("v"), py::arg("o"), py::arg("lse"), py::arg("grad_output"),
+        py::arg("window_size"), py::arg("scale"));
   m.def("abi_version", []() { return wm_abi_version(); }, "ABI version of libwindow_matmul_hip.so");
 }

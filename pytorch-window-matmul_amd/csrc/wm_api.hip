@@ -146,6 +146,25 @@ int wm_window_attention_forward(const wm_operand *q, const wm_operand *k, const 
   return to_status(err);
 }
 
+int wm_window_attention_backward(const wm_operand *q, const wm_operand *k, const wm_operand *v, const wm_operand *o,
+                                 const float *lse, const wm_operand *grad_o, const wm_operand *grad_q,
+                                 const wm_operand *grad_k, const wm_operand *grad_v, float *delta, int64_t B,
+                                 int64_t M, int64_t N, int64_t w, double scale, int dtype, unsigned flags,
+                                 void *stream) {
+  if (int st = check_common(B, M, N, w, dtype, flags)) return st;
+  if (!(scale == scale)) return WM_ERR_BAD_SHAPE;
+  if (B == 0 || M == 0) return WM_OK;
+  if (missing(q) || missing(k) || missing(v) || missing(o) || missing(grad_o) || missing(grad_q) || missing(grad_k) ||
+      missing(grad_v) || lse == nullptr || delta == nullptr)
+    return WM_ERR_NULL_POINTER;
+  const Problem prob{B, M, N, w, dtype, flags, static_cast<hipStream_t>(stream)};
+  hipError_t err = hipSuccess;
+  if (!try_launch_attention_backward(prob, make_view(q), make_view(k), make_view(v), make_view(o), make_view(grad_o),
+                                     lse, delta, make_view(grad_q), make_view(grad_k), make_view(grad_v), scale, &err))
+    return WM_ERR_UNSUPPORTED;
+  return to_status(err);
+}
+
 int wm_window_attention_supported(int64_t M, int64_t N, int64_t w, int dtype, double scale) {
   return attention_supports(M, N, w, dtype, scale) ? 1 : 0;
 }

@@ -32,7 +32,6 @@ namespace {
 constexpr int AT_TM = 128;  // queries per workgroup
 constexpr int AT_KC = 64;   // keys per chunk
 constexpr float kRaiseStep = 8.0f;
-constexpr float kLog2eF = 1.4426950408889634f;
 constexpr float kLn2F = 0.6931471805599453f;
 
 // Transposed operand fetch like lds_read_transposed, but for the k order that the accumulator

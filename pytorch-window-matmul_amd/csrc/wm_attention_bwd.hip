@@ -1,0 +1,435 @@
+// Fused window attention, backward, by recomputation from the saved log-sum-exp L of every row:
+//   P[i,c]  = exp(scale * q_i . k_c - L_i)            for |i - c| <= w, 0 <= c < M
+//   D_i     = sum_h dO[i,h] * O[i,h]                   (= sum_c P[i,c] * dP[i,c])
+//   dP[i,c] = dO_i . v_c
+//   dS[i,c] = scale * P[i,c] * (dP[i,c] - D_i)
+//   dQ_i = sum_c dS[i,c] k_c      dK_c = sum_i dS[i,c] q_i      dV_c = sum_i P[i,c] dO_i
+// Band entries outside the sequence need no special case here: they only enter through L (the
+// forward counted them there when asked to) and their own gradients are dropped by the chain of
+// separate ops as well.
+//
+// Two output-stationary kernels, no atomics:
+//   query kernel  a workgroup owns 128 queries and walks over the key chunks of its band
+//                 (K and V staged in LDS): S^T, dP^T, then dQ^T += K^T dS^T.  It also writes D.
+//   key kernel    a workgroup owns 128 keys and walks over the query chunks of their band
+//                 (Q, dO, L, D staged in LDS): S, dP, then dV^T += dO^T P and dK^T += Q^T dS.
+// Both use the layout of the forward kernel: in every 32x32 score tile a lane owns one row of the
+// stationary side (lane % 32) and 16 rows of the streamed side, so P and dS come out of the
+// arithmetic already arranged as B operands of the products that consume them, and the streamed
+// tiles are read from LDS both by rows (first products) and transposed (second products).
+#include "wm_mfma_common.hpp"
+
+#include <type_traits>
+
+namespace wm {
+namespace {
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+constexpr int AB_TM = 128;  // stationary rows per workgroup (32 per wavefront)
+constexpr int AB_KC = 64;   // streamed rows per chunk
+
+// See wm_attention.hip: rows k0 + 4 half + {0..3} and k0 + 8 + 4 half + {0..3}.
+__device__ __forceinline__ u32x4 lds_tr_split(const uint16_t *mat, int stride, int k0, int x0, int lane) {
+  const int s = lane & 15, grp = lane >> 4;
+  const int xb = x0 + 16 * (grp & 1) + 4 * (s & 3);
+  const int kb = k0 + 4 * (grp >> 1) + (s >> 2);
+  typedef s16x4 __attribute__((address_space(3))) * lds_ptr;
+  const uint16_t *p0 = mat + kb * stride + xb;
+  const uint16_t *p1 = p0 + 8 * stride;
+  const s16x4 a = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(p0));
+  const s16x4 b = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(p1));
+  const u32x2 ua = __builtin_bit_cast(u32x2, a), ub = __builtin_bit_cast(u32x2, b);
+  u32x4 r = {ua[0], ua[1], ub[0], ub[1]};
+  return r;
+}
+
+__device__ __forceinline__ float halves_sum(float v) {
+  const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+
+template <typename T>
+__device__ __forceinline__ float dot8(u32x4 a, u32x4 b) {
+  float acc = 0.0f;
+#pragma unroll
+  for (int d = 0; d < 4; ++d) {
+    T a0, a1, b0, b1;
+    const uint16_t al = (uint16_t)a[d], ah = (uint16_t)(a[d] >> 16), bl = (uint16_t)b[d], bh = (uint16_t)(b[d] >> 16);
+    __builtin_memcpy(&a0, &al, 2), __builtin_memcpy(&a1, &ah, 2);
+    __builtin_memcpy(&b0, &bl, 2), __builtin_memcpy(&b1, &bh, 2);
+    acc += to_acc<T>(a0) * to_acc<T>(b0) + to_acc<T>(a1) * to_acc<T>(b1);
+  }
+  return acc;
+}
+
+template <typename T>
+__device__ __forceinline__ u32x4 pack8(const float *x) {
+  const u32x4 r = {Mma<T>::pack2(x[0], x[1]), Mma<T>::pack2(x[2], x[3]), Mma<T>::pack2(x[4], x[5]),
+                   Mma<T>::pack2(x[6], x[7])};
+  return r;
+}
+
+// Stores a 32-row accumulator block set, transposed layout (lane = row lane % 32, accumulator v =
+// column 32 hb + 8 (v / 4) + 4 half + v % 4), as 16-bit rows.
+template <typename T, int NB>
+__device__ __forceinline__ void store_rows(uint16_t *row, const f32x16 (&acc)[NB], int half) {
+#pragma unroll
+  for (int hb = 0; hb < NB; ++hb)
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      const u32x2 out = {Mma<T>::pack2(acc[hb][4 * g], acc[hb][4 * g + 1]),
+                         Mma<T>::pack2(acc[hb][4 * g + 2], acc[hb][4 * g + 3])};
+      *reinterpret_cast<u32x2 *>(row + 32 * hb + 8 * g + 4 * half) = out;
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// query kernel: dQ and D
+// ---------------------------------------------------------------------------------------------
+template <typename T, int NB>
+__global__ __launch_bounds__(kThreads, NB <= 2 ? 2 : 1) void attention_backward_query_kernel(
+    const uint16_t *__restrict__ Q, const uint16_t *__restrict__ K, const uint16_t *__restrict__ V,
+    const uint16_t *__restrict__ O, const uint16_t *__restrict__ dO, const float *__restrict__ L,
+    uint16_t *__restrict__ dQ, float *__restrict__ D, int B, int M, int w, int nblk, float scale, int64_t qsb,
+    int64_t qsr, int64_t ksb, int64_t ksr, int64_t vsb, int64_t vsr, int64_t osb, int64_t osr, int64_t gsb, int64_t gsr,
+    int64_t dqsb, int64_t dqsr) {
+  constexpr int N = 32 * NB, NK = N / 16;
+  constexpr int TS = N + 16;  // tile rows 32 (mod 128) bytes apart: good for row reads and transposed reads
+  constexpr int SLOTS = AB_KC * N / 8 / kThreads;
+  __shared__ __attribute__((aligned(16))) uint16_t k_lds[2][AB_KC * TS];
+  __shared__ __attribute__((aligned(16))) uint16_t v_lds[2][AB_KC * TS];
+
+  int b, blk;
+  if (!decode_block(nblk, B, &b, &blk)) return;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, half = lane >> 5;
+  const int i0 = blk * AB_TM;
+  const int qw0 = i0 + 32 * wave;
+  const int qi = qw0 + (lane & 31);
+  const bool q_ok = qi < M;
+  const uint16_t *Kb = K + (int64_t)b * ksb;
+  const uint16_t *Vb = V + (int64_t)b * vsb;
+  const float c = scale * 1.4426950408889634f;
+
+  // stationary side in registers: the query rows and their upstream gradient rows (B operands)
+  u32x4 qf[NK], gf[NK];
+  float delta = 0.0f;
+  {
+    const uint16_t *qr = Q + (int64_t)b * qsb + (int64_t)qi * qsr + 8 * half;
+    const uint16_t *gr = dO + (int64_t)b * gsb + (int64_t)qi * gsr + 8 * half;
+    const uint16_t *orow = O + (int64_t)b * osb + (int64_t)qi * osr + 8 * half;
+#pragma unroll
+    for (int ks = 0; ks < NK; ++ks) {
+      qf[ks] = load_row_chunk(qr + 16 * ks, Q, q_ok);
+      gf[ks] = load_row_chunk(gr + 16 * ks, dO, q_ok);
+      delta += dot8<T>(gf[ks], load_row_chunk(orow + 16 * ks, O, q_ok));
+    }
+  }
+  delta = halves_sum(delta);
+  if (q_ok && half == 0) D[(int64_t)b * M + qi] = delta;
+  const float l2 = (q_ok ? L[(int64_t)b * M + qi] : 0.0f) * 1.4426950408889634f;
+  const float delta_s = delta * scale;
+
+  const int kc_lo = max(i0 - w, 0) / AB_KC;
+  const int kc_hi = min(i0 + AB_TM - 1 + w, M - 1) / AB_KC;
+  int l_row[SLOTS], l_col[SLOTS];
+#pragma unroll
+  for (int u = 0; u < SLOTS; ++u) {
+    const int p = tid + kThreads * u;
+    l_row[u] = p / (N / 8);
+    l_col[u] = (p % (N / 8)) * 8;
+  }
+  u32x4 kreg[SLOTS], vreg[SLOTS];
+  auto fetch = [&](int kc) {
+#pragma unroll
+    for (int u = 0; u < SLOTS; ++u) {
+      const int key = kc * AB_KC + l_row[u];
+      const bool ok = key < M && kc <= kc_hi;
+      kreg[u] = fetch_row_chunk(Kb + (int64_t)key * ksr + l_col[u], K, ok);
+      vreg[u] = fetch_row_chunk(Vb + (int64_t)key * vsr + l_col[u], V, ok);
+    }
+  };
+  auto stash = [&](int kc, int buf) {
+#pragma unroll
+    for (int u = 0; u < SLOTS; ++u) {
+      const int key = kc * AB_KC + l_row[u];
+      const bool ok = key < M && kc <= kc_hi;
+      *reinterpret_cast<u32x4 *>(&k_lds[buf][l_row[u] * TS + l_col[u]]) = mask_row_chunk(kreg[u], ok);
+      *reinterpret_cast<u32x4 *>(&v_lds[buf][l_row[u] * TS + l_col[u]]) = mask_row_chunk(vreg[u], ok);
+    }
+  };
+
+  f32x16 dq[NB];
+#pragma unroll
+  for (int hb = 0; hb < NB; ++hb)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) dq[hb][v] = 0.0f;
+  const float ninf = -__builtin_huge_valf();
+
+  auto block = [&](int buf, int kb, int c0, auto edge) {
+    constexpr bool EDGE = decltype(edge)::value;
+    f32x16 s, dp;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) s[v] = 0.0f, dp[v] = 0.0f;
+    const int at = (32 * kb + (lane & 31)) * TS + 8 * half;
+#pragma unroll
+    for (int ks = 0; ks < NK; ++ks) {
+      s = Mma<T>::run(*reinterpret_cast<const u32x4 *>(&k_lds[buf][at + 16 * ks]), qf[ks], s);
+      dp = Mma<T>::run(*reinterpret_cast<const u32x4 *>(&v_lds[buf][at + 16 * ks]), gf[ks], dp);
+    }
+    // accumulator v of this lane: key c0 + 8 (v / 4) + 4 half + v % 4, query qi
+    if (EDGE) {
+      const int d0 = c0 + 4 * half - qi;
+      const int klim = M - c0 - 4 * half;
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int ofs = 8 * (v / 4) + v % 4;
+        const bool valid = (unsigned)(d0 + ofs + w) <= (unsigned)(2 * w) && ofs < klim;
+        s[v] = valid ? s[v] : ninf;
+      }
+    }
+    float ds[16];
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+      const float p = __builtin_amdgcn_exp2f(__builtin_fmaf(s[v], c, -l2));
+      ds[v] = p * __builtin_fmaf(dp[v], scale, -delta_s);
+    }
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      const u32x4 dsf = pack8<T>(ds + 8 * t);
+#pragma unroll
+      for (int hb = 0; hb < NB; ++hb)
+        dq[hb] = Mma<T>::run(lds_tr_split(k_lds[buf], TS, 32 * kb + 16 * t, 32 * hb, lane), dsf, dq[hb]);
+    }
+  };
+
+  fetch(kc_lo);
+  stash(kc_lo, 0);
+  __syncthreads();
+  for (int kc = kc_lo; kc <= kc_hi; ++kc) {
+    const int buf = (kc - kc_lo) & 1;
+    fetch(kc + 1);
+#pragma unroll
+    for (int kb = 0; kb < 2; ++kb) {
+      const int c0 = kc * AB_KC + 32 * kb;
+      if (c0 + 31 < qw0 - w || c0 > qw0 + 31 + w || c0 >= M) continue;  // wave-uniform
+      const bool interior = c0 >= qw0 + 31 - w && c0 + 31 <= qw0 + w && c0 + 31 < M;
+      if (interior)
+        block(buf, kb, c0, std::false_type());
+      else
+        block(buf, kb, c0, std::true_type());
+    }
+    stash(kc + 1, buf ^ 1);
+    __syncthreads();
+  }
+  if (q_ok) store_rows<T, NB>(dQ + (int64_t)b * dqsb + (int64_t)qi * dqsr, dq, half);
+}
+
+// ---------------------------------------------------------------------------------------------
+// key kernel: dK and dV
+// ---------------------------------------------------------------------------------------------
+template <typename T, int NB>
+__global__ __launch_bounds__(kThreads, NB <= 2 ? 2 : 1) void attention_backward_key_kernel(
+    const uint16_t *__restrict__ Q, const uint16_t *__restrict__ K, const uint16_t *__restrict__ V,
+    const uint16_t *__restrict__ dO, const float *__restrict__ L, const float *__restrict__ D,
+    uint16_t *__restrict__ dK, uint16_t *__restrict__ dV, int B, int M, int w, int nblk, float scale, int64_t qsb,
+    int64_t qsr, int64_t ksb, int64_t ksr, int64_t vsb, int64_t vsr, int64_t gsb, int64_t gsr, int64_t dksb,
+    int64_t dksr, int64_t dvsb, int64_t dvsr) {
+  constexpr int N = 32 * NB, NK = N / 16;
+  constexpr int TS = N + 16;
+  constexpr int SLOTS = AB_KC * N / 8 / kThreads;
+  __shared__ __attribute__((aligned(16))) uint16_t q_lds[2][AB_KC * TS];
+  __shared__ __attribute__((aligned(16))) uint16_t g_lds[2][AB_KC * TS];
+  __shared__ __attribute__((aligned(16))) float l_lds[2][AB_KC];  // L * log2(e) of the chunk's queries
+  __shared__ __attribute__((aligned(16))) float d_lds[2][AB_KC];  // D * scale
+
+  int b, blk;
+  if (!decode_block(nblk, B, &b, &blk)) return;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, half = lane >> 5;
+  const int c0 = blk * AB_TM;
+  const int kw0 = c0 + 32 * wave;     // first key of this wavefront
+  const int kj = kw0 + (lane & 31);   // this lane's key
+  const bool k_ok = kj < M;
+  const uint16_t *Qb = Q + (int64_t)b * qsb;
+  const uint16_t *Gb = dO + (int64_t)b * gsb;
+  const float *Lb = L + (int64_t)b * M;
+  const float *Db = D + (int64_t)b * M;
+  const float c = scale * 1.4426950408889634f;
+
+  u32x4 kf[NK], vf[NK];
+  {
+    const uint16_t *kr = K + (int64_t)b * ksb + (int64_t)kj * ksr + 8 * half;
+    const uint16_t *vr = V + (int64_t)b * vsb + (int64_t)kj * vsr + 8 * half;
+#pragma unroll
+    for (int ks = 0; ks < NK; ++ks) {
+      kf[ks] = load_row_chunk(kr + 16 * ks, K, k_ok);
+      vf[ks] = load_row_chunk(vr + 16 * ks, V, k_ok);
+    }
+  }
+
+  const int qc_lo = max(c0 - w, 0) / AB_KC;
+  const int qc_hi = min(c0 + AB_TM - 1 + w, M - 1) / AB_KC;
+  int l_row[SLOTS], l_col[SLOTS];
+#pragma unroll
+  for (int u = 0; u < SLOTS; ++u) {
+    const int p = tid + kThreads * u;
+    l_row[u] = p / (N / 8);
+    l_col[u] = (p % (N / 8)) * 8;
+  }
+  u32x4 qreg[SLOTS], greg[SLOTS];
+  float stat = 0.0f;  // threads 0..63 carry L of one query of the chunk, threads 64..127 carry D
+  auto fetch = [&](int qc) {
+#pragma unroll
+    for (int u = 0; u < SLOTS; ++u) {
+      const int r = qc * AB_KC + l_row[u];
+      const bool ok = r < M && qc <= qc_hi;
+      qreg[u] = fetch_row_chunk(Qb + (int64_t)r * qsr + l_col[u], Q, ok);
+      greg[u] = fetch_row_chunk(Gb + (int64_t)r * gsr + l_col[u], dO, ok);
+    }
+    const int r = qc * AB_KC + (tid & 63);
+    const bool ok = r < M && qc <= qc_hi && tid < 128;
+    const float *src = tid < 64 ? Lb : Db;
+    stat = *(ok ? src + r : L);
+  };
+  auto stash = [&](int qc, int buf) {
+#pragma unroll
+    for (int u = 0; u < SLOTS; ++u) {
+      const int r = qc * AB_KC + l_row[u];
+      const bool ok = r < M && qc <= qc_hi;
+      *reinterpret_cast<u32x4 *>(&q_lds[buf][l_row[u] * TS + l_col[u]]) = mask_row_chunk(qreg[u], ok);
+      *reinterpret_cast<u32x4 *>(&g_lds[buf][l_row[u] * TS + l_col[u]]) = mask_row_chunk(greg[u], ok);
+    }
+    const int r = qc * AB_KC + (tid & 63);
+    const bool ok = r < M && qc <= qc_hi;
+    if (tid < 64) l_lds[buf][tid] = ok ? stat * 1.4426950408889634f : 0.0f;
+    else if (tid < 128) d_lds[buf][tid - 64] = ok ? stat * scale : 0.0f;
+  };
+
+  f32x16 dk[NB], dv[NB];
+#pragma unroll
+  for (int hb = 0; hb < NB; ++hb)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) dk[hb][v] = 0.0f, dv[hb][v] = 0.0f;
+  const float ninf = -__builtin_huge_valf();
+
+  auto block = [&](int buf, int qb, int r0, auto edge) {
+    constexpr bool EDGE = decltype(edge)::value;
+    f32x16 s, dp;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) s[v] = 0.0f, dp[v] = 0.0f;
+    const int at = (32 * qb + (lane & 31)) * TS + 8 * half;
+#pragma unroll
+    for (int ks = 0; ks < NK; ++ks) {
+      s = Mma<T>::run(*reinterpret_cast<const u32x4 *>(&q_lds[buf][at + 16 * ks]), kf[ks], s);
+      dp = Mma<T>::run(*reinterpret_cast<const u32x4 *>(&g_lds[buf][at + 16 * ks]), vf[ks], dp);
+    }
+    // accumulator v of this lane: query r0 + 8 (v / 4) + 4 half + v % 4, key kj
+    if (EDGE) {
+      const int d0 = r0 + 4 * half - kj;
+      const int rlim = M - r0 - 4 * half;
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int ofs = 8 * (v / 4) + v % 4;
+        const bool valid = (unsigned)(d0 + ofs + w) <= (unsigned)(2 * w) && ofs < rlim;
+        s[v] = valid ? s[v] : ninf;
+      }
+    }
+    float p[16], ds[16];
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      const f32x4 l2 = *reinterpret_cast<const f32x4 *>(&l_lds[buf][32 * qb + 8 * g + 4 * half]);
+      const f32x4 dl = *reinterpret_cast<const f32x4 *>(&d_lds[buf][32 * qb + 8 * g + 4 * half]);
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int v = 4 * g + r;
+        p[v] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[v], c, -l2[r]));
+        ds[v] = p[v] * __builtin_fmaf(dp[v], scale, -dl[r]);
+      }
+    }
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      const u32x4 pf = pack8<T>(p + 8 * t), dsf = pack8<T>(ds + 8 * t);
+#pragma unroll
+      for (int hb = 0; hb < NB; ++hb) {
+        dv[hb] = Mma<T>::run(lds_tr_split(g_lds[buf], TS, 32 * qb + 16 * t, 32 * hb, lane), pf, dv[hb]);
+        dk[hb] = Mma<T>::run(lds_tr_split(q_lds[buf], TS, 32 * qb + 16 * t, 32 * hb, lane), dsf, dk[hb]);
+      }
+    }
+  };
+
+  fetch(qc_lo);
+  stash(qc_lo, 0);
+  __syncthreads();
+  for (int qc = qc_lo; qc <= qc_hi; ++qc) {
+    const int buf = (qc - qc_lo) & 1;
+    fetch(qc + 1);
+#pragma unroll
+    for (int qb = 0; qb < 2; ++qb) {
+      const int r0 = qc * AB_KC + 32 * qb;
+      if (r0 + 31 < kw0 - w || r0 > kw0 + 31 + w || r0 >= M) continue;  // wave-uniform
+      const bool interior = r0 >= kw0 + 31 - w && r0 + 31 <= kw0 + w && r0 + 31 < M;
+      if (interior)
+        block(buf, qb, r0, std::false_type());
+      else
+        block(buf, qb, r0, std::true_type());
+    }
+    stash(qc + 1, buf ^ 1);
+    __syncthreads();
+  }
+  if (k_ok) {
+    store_rows<T, NB>(dK + (int64_t)b * dksb + (int64_t)kj * dksr, dk, half);
+    store_rows<T, NB>(dV + (int64_t)b * dvsb + (int64_t)kj * dvsr, dv, half);
+  }
+}
+
+template <typename T, int NB>
+hipError_t launch_backward(const Problem &p, const View &q, const View &k, const View &v, const View &o,
+                           const View &go, const float *lse, float *delta, const View &gq, const View &gk,
+                           const View &gv, double scale) {
+  const int nblk = (int)((p.M + AB_TM - 1) / AB_TM);
+  const int64_t groups = (p.B + 7) / 8;
+  if (groups * 8 * nblk > 0x7fffffff) return hipErrorInvalidValue;
+  const dim3 grid((unsigned)(groups * 8 * nblk)), block(kThreads);
+  typedef const uint16_t *in_t;
+  typedef uint16_t *out_t;
+  hipLaunchKernelGGL((attention_backward_query_kernel<T, NB>), grid, block, 0, p.stream, (in_t)q.data, (in_t)k.data,
+                     (in_t)v.data, (in_t)o.data, (in_t)go.data, lse, (out_t)gq.data, delta, (int)p.B, (int)p.M,
+                     (int)p.w, nblk, (float)scale, q.sb, q.sr, k.sb, k.sr, v.sb, v.sr, o.sb, o.sr, go.sb, go.sr, gq.sb,
+                     gq.sr);
+  hipError_t err = hipGetLastError();
+  if (err != hipSuccess) return err;
+  hipLaunchKernelGGL((attention_backward_key_kernel<T, NB>), grid, block, 0, p.stream, (in_t)q.data, (in_t)k.data,
+                     (in_t)v.data, (in_t)go.data, lse, (const float *)delta, (out_t)gk.data, (out_t)gv.data, (int)p.B,
+                     (int)p.M, (int)p.w, nblk, (float)scale, q.sb, q.sr, k.sb, k.sr, v.sb, v.sr, go.sb, go.sr, gk.sb,
+                     gk.sr, gv.sb, gv.sr);
+  return hipGetLastError();
+}
+
+template <typename T>
+hipError_t backward_by_width(const Problem &p, const View &q, const View &k, const View &v, const View &o,
+                             const View &go, const float *lse, float *delta, const View &gq, const View &gk,
+                             const View &gv, double scale) {
+  switch (p.N / 32) {
+    case 1: return launch_backward<T, 1>(p, q, k, v, o, go, lse, delta, gq, gk, gv, scale);
+    case 2: return launch_backward<T, 2>(p, q, k, v, o, go, lse, delta, gq, gk, gv, scale);
+    case 3: return launch_backward<T, 3>(p, q, k, v, o, go, lse, delta, gq, gk, gv, scale);
+    default: return launch_backward<T, 4>(p, q, k, v, o, go, lse, delta, gq, gk, gv, scale);
+  }
+}
+
+}  // namespace
+
+bool try_launch_attention_backward(const Problem &p, const View &q, const View &k, const View &v, const View &o,
+                                   const View &go, const float *lse, float *delta, const View &gq, const View &gk,
+                                   const View &gv, double scale, hipError_t *err) {
+  if (p.flags & WM_FLAG_FORCE_STRIDED) return false;
+  if (!attention_supports(p.M, p.N, p.w, p.dtype, scale)) return false;
+  const View *all[] = {&q, &k, &v, &o, &go, &gq, &gk, &gv};
+  for (const View *t : all)
+    if (!fast_layout(*t, p.dtype)) return false;
+  *err = p.dtype == WM_DTYPE_BF16 ? backward_by_width<bf16_t>(p, q, k, v, o, go, lse, delta, gq, gk, gv, scale)
+                                  : backward_by_width<f16_t>(p, q, k, v, o, go, lse, delta, gq, gk, gv, scale);
+  return true;
+}
+
+}  // namespace wm

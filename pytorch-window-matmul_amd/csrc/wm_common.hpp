@@ -70,6 +70,12 @@ bool attention_supports(int64_t M, int64_t N, int64_t w, int dtype, double scale
 bool try_launch_attention_forward(const Problem &p, const View &q, const View &k, const View &v, const View &o,
                                   float *lse, double scale, int mask, hipError_t *err);
 
+// Backward of the fused attention (wm_attention_bwd.hip): two kernels on p.stream; `delta` is a
+// float32 (B,M) workspace the first one fills and the second one reads.
+bool try_launch_attention_backward(const Problem &p, const View &q, const View &k, const View &v, const View &o,
+                                   const View &go, const float *lse, float *delta, const View &gq, const View &gk,
+                                   const View &gv, double scale, hipError_t *err);
+
 inline size_t dtype_size(int dtype) {
   switch (dtype) {
     case WM_DTYPE_F32: return 4;

@@ -5,6 +5,7 @@ Drop-in for the ``window_matmul`` package of webis-de/pytorch-window-matmul
 autograd behaviour, with gfx950 HIP kernels underneath.
 """
 from .band_softmax import BandSoftmaxFunc, band_softmax  # addition; deliberately not in __all__
+from .window_attention import WindowAttentionFunc, window_attention  # addition; not in __all__
 from .window_matmul import (
     UnwindowMatmulFunc,
     WindowMatmulFunc,

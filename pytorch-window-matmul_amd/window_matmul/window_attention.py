@@ -1,0 +1,65 @@
+"""Window attention in one call: ``unwindow_matmul(softmax(scale * window_matmul(q, k^T, w)), v, w)``.
+
+The reference package stops at the two banded matmuls; its callers write the chain above
+themselves (reference tests/test_attention.py:57-63).  This function is that chain with the
+same semantics, as an addition next to the unchanged two-function API.  For float16 /
+bfloat16 inputs whose last dimension is a multiple of 32 up to 128 it runs fused kernels that
+never write the ``(…, M, 2w+1)`` band to memory (forward keeps only the log-sum-exp of every
+row, backward recomputes the probabilities); everything else runs the chain of the separate
+ops of this package, on the GPU as well.
+"""
+import math
+from typing import Optional
+
+import torch
+
+import window_matmul_kernel as _native
+
+from .band_softmax import band_softmax
+from .window_matmul import unwindow_matmul, window_matmul
+
+
+class WindowAttentionFunc(torch.autograd.Function):
+    """Fused kernels on 3-D ``(B, M, N)`` operands; ``k`` holds key rows (not transposed)."""
+
+    @staticmethod
+    def forward(ctx, q, k, v, window_size: int, scale: float, mask_out_of_range: bool):
+        out, lse = _native.window_attention_forward(q, k, v, window_size, scale, mask_out_of_range)
+        ctx.save_for_backward(q, k, v, out, lse)
+        ctx.window_size = window_size
+        ctx.scale = scale
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        q, k, v, out, lse = ctx.saved_tensors
+        gq, gk, gv = _native.window_attention_backward(q, k, v, out, lse, grad_output, ctx.window_size, ctx.scale)
+        return gq, gk, gv, None, None, None
+
+
+def window_attention(query: torch.Tensor, key: torch.Tensor, value: torch.Tensor, window_size: int,
+                     scale: Optional[float] = None, mask_out_of_range: bool = False) -> torch.Tensor:
+    """Local attention of every position over its ``2 * window_size + 1`` neighbours.
+
+    ``query``, ``key``, ``value`` are ``(..., M, N)`` (``key`` NOT transposed, unlike the second
+    argument of ``window_matmul``); the result is ``(..., M, N)``.  ``scale`` defaults to
+    ``1 / sqrt(N)``.  With ``mask_out_of_range=False`` (default) the result equals the reference
+    callers' chain exactly as they write it: neighbours that fall outside the sequence take part
+    in the softmax with score 0 and add nothing to the output.  With ``True`` they are left out
+    of the softmax, which is the usual definition of sliding-window attention.
+    """
+    if query.shape != key.shape or query.shape != value.shape or query.dim() < 2:
+        raise RuntimeError("Input mismatch")
+    scale = 1.0 / math.sqrt(query.shape[-1]) if scale is None else float(scale)
+    if not window_size:
+        # a single neighbour: the softmax is 1 and the output is the value itself, as in the
+        # chain (reference tests/test_attention.py:75-87); kept differentiable through torch ops
+        score = (query * key).sum(-1, keepdim=True) * scale
+        return torch.softmax(score, -1) * value
+    q, k, v = (t.reshape(-1, t.shape[-2], t.shape[-1]) for t in (query, key, value))
+    if _native.window_attention_supported(q, window_size, scale):
+        out = WindowAttentionFunc.apply(q, k, v, window_size, scale, bool(mask_out_of_range))
+    else:
+        att = window_matmul(q, k.transpose(-1, -2), window_size)
+        out = unwindow_matmul(band_softmax(att, scale, mask_out_of_range), v, window_size)
+    return out.reshape(query.shape)

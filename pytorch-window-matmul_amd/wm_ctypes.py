@@ -62,6 +62,8 @@ def lib():
         L.wm_band_softmax_kernel_choice.argtypes = [i64, ctypes.c_int, ctypes.c_int, ctypes.c_int, u32]
         L.wm_window_attention_forward.argtypes = [P, P, P, P, vp, i64, i64, i64, i64, ctypes.c_double, ctypes.c_int,
                                                   ctypes.c_int, u32, vp]
+        L.wm_window_attention_backward.argtypes = [P, P, P, P, vp, P, P, P, P, vp, i64, i64, i64, i64, ctypes.c_double,
+                                                   ctypes.c_int, u32, vp]
         L.wm_window_attention_supported.argtypes = [i64, i64, i64, ctypes.c_int, ctypes.c_double]
         _LIB = L
     return _LIB
@@ -149,3 +151,15 @@ def attention_forward(q, k, v, w, scale=1.0, mask=False, flags=0, want_lse=True)
                                             float(scale), int(mask), DTYPES[q.dtype], flags, _stream()),
            "wm_window_attention_forward")
     return o, lse
+
+
+def attention_backward(q, k, v, o, lse, go, w, scale=1.0, flags=0):
+    """Gradients (gq, gk, gv), all (B,M,N) row-major, from the forward's o and lse."""
+    B, M, N = q.shape
+    gq, gk, gv = (torch.empty(B, M, N, dtype=q.dtype, device=q.device) for _ in range(3))
+    delta = torch.empty(B, M, dtype=torch.float32, device=q.device)
+    _check(lib().wm_window_attention_backward(op(q), op(k), op(v), op(o), ctypes.c_void_p(lse.data_ptr()), op(go),
+                                             op(gq), op(gk), op(gv), ctypes.c_void_p(delta.data_ptr()), B, M, N, w,
+                                             float(scale), DTYPES[q.dtype], flags, _stream()),
+           "wm_window_attention_backward")
+    return gq, gk, gv

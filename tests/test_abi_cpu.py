@@ -15,7 +15,8 @@ def test_library_exports_every_declared_symbol():
     names = abi.declared_symbols()
     assert {"wm_window_matmul_forward", "wm_window_matmul_backward", "wm_unwindow_matmul_forward",
             "wm_unwindow_matmul_backward", "wm_band_softmax_forward", "wm_band_softmax_backward",
-            "wm_band_softmax_kernel_choice", "wm_window_attention_forward", "wm_window_attention_supported",
+            "wm_band_softmax_kernel_choice", "wm_window_attention_forward", "wm_window_attention_backward",
+            "wm_window_attention_supported",
             "wm_kernel_choice", "wm_status_string", "wm_abi_version"} <= set(names)
     for name in names:
         assert hasattr(L, name), name

@@ -88,3 +88,75 @@ def test_benchmark_shape_against_separate_ops(device):
     torch.testing.assert_close(o.float(), want.float(), **TOL)
     torch.testing.assert_close(lse, torch.logsumexp(att, -1), rtol=2e-3, atol=2e-3)
     assert torch.isfinite(o).all()
+
+
+@pytest.mark.parametrize("mask", [False, True], ids=["zero_filled", "masked"])
+@pytest.mark.parametrize("dtype", DTYPES, ids=lambda d: str(d).split(".")[-1])
+@pytest.mark.parametrize("case", CASES, ids=lambda c: "B%d_M%d_N%d_w%d" % c)
+def test_backward_matches_oracle(device, case, dtype, mask):
+    B, M, N, w = case
+    scale = 1.0 / math.sqrt(N)
+    q, k, v, go = (seeded((B, M, N), s, dtype) for s in (61, 62, 63, 64))
+    want = ao.window_attention_backward(q, k, v, w, go, scale, mask)
+    qd, kd, vd, gd = (t.to(device) for t in (q, k, v, go))
+    o, lse = abi.attention_forward(qd, kd, vd, w, scale, mask)
+    got = abi.attention_backward(qd, kd, vd, o, lse, gd, w, scale)
+    for name, x, y in zip(("grad_q", "grad_k", "grad_v"), got, want):
+        close(x, y)
+    # two kernels, no atomics: a second run gives the same bits
+    again = abi.attention_backward(qd, kd, vd, o, lse, gd, w, scale)
+    for x, y in zip(got, again):
+        assert torch.equal(x, y)
+
+
+@pytest.mark.parametrize("mask", [False, True], ids=["zero_filled", "masked"])
+def test_python_function_matches_the_chain(device, mask):
+    """window_attention against window_matmul -> torch.softmax -> unwindow_matmul written out as the
+    reference's callers do (reference tests/test_attention.py:57-63): output and input gradients,
+    head-major non-contiguous inputs with leading batch and head dimensions."""
+    from window_matmul import unwindow_matmul, window_attention, window_matmul
+    from oracle import softmax_oracle as so
+
+    batch, heads, M, N, w = 2, 3, 200, 64, 24
+    dtype = torch.bfloat16
+
+    def head_major(seed):
+        t = seeded((batch, M, heads * N), seed, dtype).to(device)
+        return t.view(batch, M, heads, N).transpose(1, 2)
+
+    q0, k0, v0, go = head_major(71), head_major(72), head_major(73), head_major(74)
+    keep = torch.from_numpy(so.valid_mask(M, w)).to(device)
+    res = {}
+    for name in ("chain", "fused"):
+        q, k, v = (t.detach().clone().requires_grad_(True) for t in (q0, k0, v0))
+        if name == "chain":
+            att = window_matmul(q, k.transpose(-1, -2), w).float() / math.sqrt(N)
+            if mask:
+                att = att.masked_fill(~keep, float("-inf"))
+            out = unwindow_matmul(torch.softmax(att, -1).to(dtype), v, w)
+        else:
+            out = window_attention(q, k, v, w, mask_out_of_range=mask)
+        out.backward(go)
+        res[name] = (out.detach(), q.grad, k.grad, v.grad)
+    assert res["fused"][0].shape == q0.shape
+    for x, y in zip(res["fused"], res["chain"]):
+        torch.testing.assert_close(x.float(), y.float(), **TOL)
+
+
+def test_python_function_falls_back_to_the_separate_ops(device):
+    """float32, or a width the fused kernels do not cover: same function, separate ops underneath."""
+    from window_matmul import window_attention
+
+    for dtype, N, tol in ((torch.float32, 64, dict(rtol=1e-4, atol=1e-5)), (torch.bfloat16, 48, TOL)):
+        B, M, w = 2, 90, 10
+        q0, k0, v0, go = (seeded((B, M, N), s, dtype) for s in (81, 82, 83, 84))
+        want_o, _ = ao.window_attention_forward(q0, k0, v0, w, 1.0 / math.sqrt(N))
+        want_g = ao.window_attention_backward(q0, k0, v0, w, go, 1.0 / math.sqrt(N))
+        q, k, v = (t.to(device).requires_grad_(True) for t in (q0, k0, v0))
+        out = window_attention(q, k, v, w)
+        out.backward(go.to(device))
+        for x, y in zip((out, q.grad, k.grad, v.grad), (want_o,) + want_g):
+            torch.testing.assert_close(x.detach().cpu().to(torch.float64), torch.from_numpy(y), **tol)
+    # window_size 0: the value itself
+    q = seeded((2, 5, 64), 85, torch.bfloat16).to(device)
+    torch.testing.assert_close(window_attention(q, q, q, 0), q)
