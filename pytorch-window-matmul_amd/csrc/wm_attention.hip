@@ -62,7 +62,7 @@ __device__ __forceinline__ float across_halves_sum(float v) {
 }
 
 template <typename T, int NB, bool MASK>
-__global__ __launch_bounds__(kThreads, 2) void attention_forward_kernel(
+__global__ __launch_bounds__(kThreads, NB <= 2 ? 4 : 2) void attention_forward_kernel(
     const uint16_t *__restrict__ Q, const uint16_t *__restrict__ K, const uint16_t *__restrict__ V,
     uint16_t *__restrict__ O, float *__restrict__ L, int B, int M, int w, int nblk, float c, int64_t qsb, int64_t qsr,
     int64_t ksb, int64_t ksr, int64_t vsb, int64_t vsr, int64_t osb, int64_t osr) {
@@ -102,22 +102,23 @@ __global__ __launch_bounds__(kThreads, 2) void attention_forward_kernel(
     l_col[u] = (p % (N / 8)) * 8;
   }
   u32x4 kreg[SLOTS], vreg[SLOTS];
-  auto fetch = [&](int kc) {  // loads only; rows past the sequence or the last chunk come from a safe address
+  // Loads only.  Rows past the end of the sequence (and the chunk after the last one) are clamped
+  // to the last row instead of being zero-filled: every key they stand for is masked out by the
+  // edge logic below, so only finite stand-in data is needed.
+  auto fetch = [&](int kc) {
+    const int base = min(kc, kc_hi) * AT_KC;
 #pragma unroll
     for (int u = 0; u < SLOTS; ++u) {
-      const int key = kc * AT_KC + l_row[u];
-      const bool ok = key < M && kc <= kc_hi;
-      kreg[u] = fetch_row_chunk(Kb + (int64_t)key * ksr + l_col[u], K, ok);
-      vreg[u] = fetch_row_chunk(Vb + (int64_t)key * vsr + l_col[u], V, ok);
+      const int key = min(base + l_row[u], M - 1);
+      kreg[u] = *reinterpret_cast<const u32x4 *>(Kb + (int64_t)key * ksr + l_col[u]);
+      vreg[u] = *reinterpret_cast<const u32x4 *>(Vb + (int64_t)key * vsr + l_col[u]);
     }
   };
-  auto stash = [&](int kc, int buf) {
+  auto stash = [&](int buf) {
 #pragma unroll
     for (int u = 0; u < SLOTS; ++u) {
-      const int key = kc * AT_KC + l_row[u];
-      const bool ok = key < M && kc <= kc_hi;
-      *reinterpret_cast<u32x4 *>(&k_lds[buf][l_row[u] * KS + l_col[u]]) = mask_row_chunk(kreg[u], ok);
-      *reinterpret_cast<u32x4 *>(&v_lds[buf][l_row[u] * VS + l_col[u]]) = mask_row_chunk(vreg[u], ok);
+      *reinterpret_cast<u32x4 *>(&k_lds[buf][l_row[u] * KS + l_col[u]]) = kreg[u];
+      *reinterpret_cast<u32x4 *>(&v_lds[buf][l_row[u] * VS + l_col[u]]) = vreg[u];
     }
   };
 
@@ -140,13 +141,16 @@ __global__ __launch_bounds__(kThreads, 2) void attention_forward_kernel(
     for (int ks = 0; ks < NK; ++ks) s = Mma<T>::run(*reinterpret_cast<const u32x4 *>(krow + 16 * ks), qf[ks], s);
     // accumulator v of this lane: key c0 + 8 (v / 4) + 4 half + v % 4, query qi
     if (EDGE) {
-      const int d0 = c0 + 4 * half - qi;   // key - query for v = 0
-      const int klim = M - c0 - 4 * half;  // keys of this lane with offset below klim exist
+      // key offset ofs = 8 (v / 4) + v % 4 of this lane is inside the band and the sequence iff
+      // first <= ofs <= last; one unsigned comparison per element after this per-lane setup
+      const int d0 = c0 + 4 * half - qi;  // key - query at ofs = 0
+      const int first = -w - d0, last = min(w - d0, M - 1 - c0 - 4 * half);
+      const int origin = last < first ? 0x100000 : first;
+      const unsigned span = last < first ? 0u : (unsigned)(last - first);
 #pragma unroll
       for (int v = 0; v < 16; ++v) {
         const int ofs = 8 * (v / 4) + v % 4;
-        const bool valid = (unsigned)(d0 + ofs + w) <= (unsigned)(2 * w) && ofs < klim;
-        s[v] = valid ? s[v] : ninf;
+        s[v] = (unsigned)(ofs - origin) <= span ? s[v] : ninf;
       }
     }
     float bm = s[0];
@@ -166,14 +170,14 @@ __global__ __launch_bounds__(kThreads, 2) void attention_forward_kernel(
     }
     float p[16];
 #pragma unroll
-    for (int v = 0; v < 16; ++v) {
-      p[v] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[v], c, -m_used));
-      l_part += p[v];
-    }
+    for (int v = 0; v < 16; ++v) p[v] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[v], c, -m_used));
 #pragma unroll
     for (int t = 0; t < 2; ++t) {
       const u32x4 pf = {Mma<T>::pack2(p[8 * t + 0], p[8 * t + 1]), Mma<T>::pack2(p[8 * t + 2], p[8 * t + 3]),
                         Mma<T>::pack2(p[8 * t + 4], p[8 * t + 5]), Mma<T>::pack2(p[8 * t + 6], p[8 * t + 7])};
+      // the row sum is taken over the rounded probabilities, the ones that multiply V
+#pragma unroll
+      for (int d = 0; d < 4; ++d) l_part = Mma<T>::add_pair(pf[d], l_part);
 #pragma unroll
       for (int hb = 0; hb < NB; ++hb) {
         const u32x4 vf = lds_read_transposed_split(v_lds[buf], VS, 32 * kb + 16 * t, 32 * hb, lane);
@@ -183,7 +187,7 @@ __global__ __launch_bounds__(kThreads, 2) void attention_forward_kernel(
   };
 
   fetch(kc_lo);
-  stash(kc_lo, 0);
+  stash(0);
   __syncthreads();
   for (int kc = kc_lo; kc <= kc_hi; ++kc) {
     const int buf = (kc - kc_lo) & 1;
@@ -199,7 +203,7 @@ __global__ __launch_bounds__(kThreads, 2) void attention_forward_kernel(
       else
         block(buf, kb, c0, std::true_type());
     }
-    stash(kc + 1, buf ^ 1);
+    stash(buf ^ 1);
     __syncthreads();
   }
 

@@ -140,22 +140,21 @@ __global__ __launch_bounds__(kThreads, NB <= 2 ? 2 : 1) void attention_backward_
     l_col[u] = (p % (N / 8)) * 8;
   }
   u32x4 kreg[SLOTS], vreg[SLOTS];
+  // loads only; rows past the sequence are clamped to its last row (they are masked out below)
   auto fetch = [&](int kc) {
+    const int base = min(kc, kc_hi) * AB_KC;
 #pragma unroll
     for (int u = 0; u < SLOTS; ++u) {
-      const int key = kc * AB_KC + l_row[u];
-      const bool ok = key < M && kc <= kc_hi;
-      kreg[u] = fetch_row_chunk(Kb + (int64_t)key * ksr + l_col[u], K, ok);
-      vreg[u] = fetch_row_chunk(Vb + (int64_t)key * vsr + l_col[u], V, ok);
+      const int key = min(base + l_row[u], M - 1);
+      kreg[u] = *reinterpret_cast<const u32x4 *>(Kb + (int64_t)key * ksr + l_col[u]);
+      vreg[u] = *reinterpret_cast<const u32x4 *>(Vb + (int64_t)key * vsr + l_col[u]);
     }
   };
-  auto stash = [&](int kc, int buf) {
+  auto stash = [&](int buf) {
 #pragma unroll
     for (int u = 0; u < SLOTS; ++u) {
-      const int key = kc * AB_KC + l_row[u];
-      const bool ok = key < M && kc <= kc_hi;
-      *reinterpret_cast<u32x4 *>(&k_lds[buf][l_row[u] * TS + l_col[u]]) = mask_row_chunk(kreg[u], ok);
-      *reinterpret_cast<u32x4 *>(&v_lds[buf][l_row[u] * TS + l_col[u]]) = mask_row_chunk(vreg[u], ok);
+      *reinterpret_cast<u32x4 *>(&k_lds[buf][l_row[u] * TS + l_col[u]]) = kreg[u];
+      *reinterpret_cast<u32x4 *>(&v_lds[buf][l_row[u] * TS + l_col[u]]) = vreg[u];
     }
   };
 
@@ -179,13 +178,14 @@ __global__ __launch_bounds__(kThreads, NB <= 2 ? 2 : 1) void attention_backward_
     }
     // accumulator v of this lane: key c0 + 8 (v / 4) + 4 half + v % 4, query qi
     if (EDGE) {
-      const int d0 = c0 + 4 * half - qi;
-      const int klim = M - c0 - 4 * half;
+      const int d0 = c0 + 4 * half - qi;  // key - query at offset 0; valid offsets: first..last
+      const int first = -w - d0, last = min(w - d0, M - 1 - c0 - 4 * half);
+      const int origin = last < first ? 0x100000 : first;
+      const unsigned span = last < first ? 0u : (unsigned)(last - first);
 #pragma unroll
       for (int v = 0; v < 16; ++v) {
         const int ofs = 8 * (v / 4) + v % 4;
-        const bool valid = (unsigned)(d0 + ofs + w) <= (unsigned)(2 * w) && ofs < klim;
-        s[v] = valid ? s[v] : ninf;
+        s[v] = (unsigned)(ofs - origin) <= span ? s[v] : ninf;
       }
     }
     float ds[16];
@@ -204,7 +204,7 @@ __global__ __launch_bounds__(kThreads, NB <= 2 ? 2 : 1) void attention_backward_
   };
 
   fetch(kc_lo);
-  stash(kc_lo, 0);
+  stash(0);
   __syncthreads();
   for (int kc = kc_lo; kc <= kc_hi; ++kc) {
     const int buf = (kc - kc_lo) & 1;
@@ -219,7 +219,7 @@ __global__ __launch_bounds__(kThreads, NB <= 2 ? 2 : 1) void attention_backward_
       else
         block(buf, kb, c0, std::true_type());
     }
-    stash(kc + 1, buf ^ 1);
+    stash(buf ^ 1);
     __syncthreads();
   }
   if (q_ok) store_rows<T, NB>(dQ + (int64_t)b * dqsb + (int64_t)qi * dqsr, dq, half);
@@ -279,30 +279,24 @@ __global__ __launch_bounds__(kThreads, NB <= 2 ? 2 : 1) void attention_backward_
   u32x4 qreg[SLOTS], greg[SLOTS];
   float stat = 0.0f;  // threads 0..63 carry L of one query of the chunk, threads 64..127 carry D
   auto fetch = [&](int qc) {
+    const int base = min(qc, qc_hi) * AB_KC;
 #pragma unroll
     for (int u = 0; u < SLOTS; ++u) {
-      const int r = qc * AB_KC + l_row[u];
-      const bool ok = r < M && qc <= qc_hi;
-      qreg[u] = fetch_row_chunk(Qb + (int64_t)r * qsr + l_col[u], Q, ok);
-      greg[u] = fetch_row_chunk(Gb + (int64_t)r * gsr + l_col[u], dO, ok);
+      const int r = min(base + l_row[u], M - 1);
+      qreg[u] = *reinterpret_cast<const u32x4 *>(Qb + (int64_t)r * qsr + l_col[u]);
+      greg[u] = *reinterpret_cast<const u32x4 *>(Gb + (int64_t)r * gsr + l_col[u]);
     }
-    const int r = qc * AB_KC + (tid & 63);
-    const bool ok = r < M && qc <= qc_hi && tid < 128;
-    const float *src = tid < 64 ? Lb : Db;
-    stat = *(ok ? src + r : L);
+    const int r = min(base + (tid & 63), M - 1);
+    stat = (tid < 64 ? Lb : Db)[r];
   };
-  auto stash = [&](int qc, int buf) {
+  auto stash = [&](int buf) {
 #pragma unroll
     for (int u = 0; u < SLOTS; ++u) {
-      const int r = qc * AB_KC + l_row[u];
-      const bool ok = r < M && qc <= qc_hi;
-      *reinterpret_cast<u32x4 *>(&q_lds[buf][l_row[u] * TS + l_col[u]]) = mask_row_chunk(qreg[u], ok);
-      *reinterpret_cast<u32x4 *>(&g_lds[buf][l_row[u] * TS + l_col[u]]) = mask_row_chunk(greg[u], ok);
+      *reinterpret_cast<u32x4 *>(&q_lds[buf][l_row[u] * TS + l_col[u]]) = qreg[u];
+      *reinterpret_cast<u32x4 *>(&g_lds[buf][l_row[u] * TS + l_col[u]]) = greg[u];
     }
-    const int r = qc * AB_KC + (tid & 63);
-    const bool ok = r < M && qc <= qc_hi;
-    if (tid < 64) l_lds[buf][tid] = ok ? stat * 1.4426950408889634f : 0.0f;
-    else if (tid < 128) d_lds[buf][tid - 64] = ok ? stat * scale : 0.0f;
+    if (tid < 64) l_lds[buf][tid] = stat * 1.4426950408889634f;
+    else if (tid < 128) d_lds[buf][tid - 64] = stat * scale;
   };
 
   f32x16 dk[NB], dv[NB];
@@ -325,13 +319,14 @@ __global__ __launch_bounds__(kThreads, NB <= 2 ? 2 : 1) void attention_backward_
     }
     // accumulator v of this lane: query r0 + 8 (v / 4) + 4 half + v % 4, key kj
     if (EDGE) {
-      const int d0 = r0 + 4 * half - kj;
-      const int rlim = M - r0 - 4 * half;
+      const int d0 = r0 + 4 * half - kj;  // query - key at offset 0; valid offsets: first..last
+      const int first = -w - d0, last = min(w - d0, M - 1 - r0 - 4 * half);
+      const int origin = last < first ? 0x100000 : first;
+      const unsigned span = last < first ? 0u : (unsigned)(last - first);
 #pragma unroll
       for (int v = 0; v < 16; ++v) {
         const int ofs = 8 * (v / 4) + v % 4;
-        const bool valid = (unsigned)(d0 + ofs + w) <= (unsigned)(2 * w) && ofs < rlim;
-        s[v] = valid ? s[v] : ninf;
+        s[v] = (unsigned)(ofs - origin) <= span ? s[v] : ninf;
       }
     }
     float p[16], ds[16];
@@ -358,7 +353,7 @@ __global__ __launch_bounds__(kThreads, NB <= 2 ? 2 : 1) void attention_backward_
   };
 
   fetch(qc_lo);
-  stash(qc_lo, 0);
+  stash(0);
   __syncthreads();
   for (int qc = qc_lo; qc <= qc_hi; ++qc) {
     const int buf = (qc - qc_lo) & 1;
@@ -373,7 +368,7 @@ __global__ __launch_bounds__(kThreads, NB <= 2 ? 2 : 1) void attention_backward_
       else
         block(buf, qb, r0, std::true_type());
     }
-    stash(qc + 1, buf ^ 1);
+    stash(buf ^ 1);
     __syncthreads();
   }
   if (k_ok) {

@@ -102,6 +102,11 @@ struct Mma<bf16_t> {
     f32x2 v = {lo, hi};
     return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2));  // v_cvt_pk_bf16_f32, RNE
   }
+  // acc + lo + hi of a packed pair (v_dot2c_f32_bf16 with a pair of ones)
+  static __device__ __forceinline__ float add_pair(uint32_t pair, float acc) {
+    const bf16x2 ones = {(__bf16)1.0f, (__bf16)1.0f};
+    return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, pair), ones, acc, false);
+  }
 };
 template <>
 struct Mma<f16_t> {
@@ -112,6 +117,11 @@ struct Mma<f16_t> {
   static __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
     const uint16_t l = __builtin_bit_cast(uint16_t, (_Float16)lo), h = __builtin_bit_cast(uint16_t, (_Float16)hi);
     return (uint32_t)l | ((uint32_t)h << 16);
+  }
+  static __device__ __forceinline__ float add_pair(uint32_t pair, float acc) {
+    typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+    const f16x2 ones = {(_Float16)1.0f, (_Float16)1.0f};
+    return __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2, pair), ones, acc, false);
   }
 };
 
