@@ -154,7 +154,7 @@ def main():
     if not torch.cuda.is_available():
         sys.exit("bench.py: no GPU visible")
     import wm_ctypes as abi
-    from window_matmul import band_softmax, unwindow_matmul, window_matmul
+    from window_matmul import band_softmax, unwindow_matmul, window_attention, window_matmul
 
     cfg = WORKLOADS[args.workload]
     B, M, N, w = cfg["B"], cfg["M"], cfg["N"], cfg["w"]
@@ -201,6 +201,23 @@ def main():
         torch.cuda.synchronize()
         band_ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
 
+        # and the whole chain as one call: fused kernels, the band never reaches memory
+        def fused_step():
+            out = window_attention(q, k, v, w, scale=1.0)
+            if cfg["backward"]:
+                q.grad = k.grad = v.grad = None
+                out.backward(go)
+            return out
+
+        for _ in range(args.warmup):
+            fused_step()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            fused_step()
+        torch.cuda.synchronize()
+        fused_ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+
     # per-kernel timing through the C ABI (one launch per call), same tensors, same stream
     with torch.no_grad():
         kt = k.detach().transpose(1, 2)
@@ -232,6 +249,11 @@ def main():
         bs_bwd_ms = time_gpu(lambda: abi.band_softmax_backward(probs, ga if ga is not None else att, 1.0, out=sm_out),
                              max(args.steps, 10), 3)
         del sm_out
+        fo, flse = abi.attention_forward(qd, k.detach(), vd, w, 1.0)
+        fused_fwd_ms = time_gpu(lambda: abi.attention_forward(qd, k.detach(), vd, w, 1.0), max(args.steps, 10), 3)
+        fused_bwd_ms = (time_gpu(lambda: abi.attention_backward(qd, k.detach(), vd, fo, flse, go, w, 1.0),
+                                 max(args.steps, 10), 3) if cfg["backward"] else None)
+        del fo, flse
         # device-to-device copy of the band as the achievable-bandwidth yardstick
         scratch = torch.empty_like(att)
         copy_ms = time_gpu(lambda: scratch.copy_(att), 20, 3)
@@ -265,6 +287,12 @@ def main():
             "fwd_ms": round(bs_fwd_ms, 4), "fwd_GBps": round(2 * band_bytes / bs_fwd_ms / 1e6, 1),
             "bwd_ms": round(bs_bwd_ms, 4), "bwd_GBps": round(3 * band_bytes / bs_bwd_ms / 1e6, 1),
             "note": "same chain with window_matmul.band_softmax replacing torch.softmax"},
+        "fused_attention": None if args.kernels_only else {
+            "ms_per_step": round(fused_ms_per_step, 4), "TFLOPs": round(flops / fused_ms_per_step / 1e9, 2),
+            "fwd_ms": round(fused_fwd_ms, 4), "bwd_ms": None if fused_bwd_ms is None else round(fused_bwd_ms, 4),
+            "mfma_frac": round(flops / fused_ms_per_step / 1e9 / 2500.0, 4),
+            "note": "same chain as one call, window_matmul.window_attention; band FLOPs credited as for the "
+                    "separate ops (recomputation in the backward not counted); mfma_frac against 2.5 PFLOP/s"},
         "copy_yardstick_GBps": round(copy_gbs, 1),
         "kernel_sum_GBps": round(len(per_kernel) * kb / sum(v["ms"] for v in per_kernel.values()) / 1e6, 1),
     }
