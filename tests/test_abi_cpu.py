@@ -2,6 +2,7 @@
 declares, validates arguments before touching the device, and the Python layer
 mirrors the reference's surface and error behaviour."""
 import ctypes
+import os
 import inspect
 
 import pytest
@@ -108,3 +109,21 @@ def test_only_one_hip_runtime_is_mapped():
 
     paths = {line.split()[-1] for line in open("/proc/self/maps") if "libamdhip64" in line}
     assert len(paths) == 1, paths
+
+
+def test_setup_py_builds_an_importable_tree(tmp_path):
+    """setup.py (packaging in the manner of reference setup.py:22-116) produces a directory from
+    which the package and its native module import without any sys.path help from this repo."""
+    import subprocess
+    import sys
+
+    pkg = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "pytorch-window-matmul_amd")
+    subprocess.check_call([sys.executable, "setup.py", "-q", "build", "--build-base", str(tmp_path)], cwd=pkg)
+    (lib,) = [d for d in os.listdir(tmp_path) if d.startswith("lib")]
+    code = ("import window_matmul, window_matmul_kernel, wm_ctypes; "
+            "assert window_matmul.__all__ == ['window_matmul', 'unwindow_matmul']; "
+            "assert window_matmul_kernel.abi_version() == wm_ctypes.lib().wm_abi_version(); "
+            "print(window_matmul.__file__)")
+    out = subprocess.check_output([sys.executable, "-c", code], cwd=str(tmp_path),
+                                  env={**os.environ, "PYTHONPATH": os.path.join(str(tmp_path), lib)}, text=True)
+    assert str(tmp_path) in out
