@@ -275,6 +275,7 @@ bool attention_supports(int64_t M, int64_t N, int64_t w, int dtype, double scale
   if (dtype != WM_DTYPE_BF16 && dtype != WM_DTYPE_F16) return false;
   if (N % 32 != 0 || N < 32 || N > 128) return false;
   if (M < 1 || w < 1 || w > 0x3fffffff) return false;
+  if (M > 0x7fffffff - w - 2 * AT_TM) return false;  // row and key indices are 32-bit in the kernels
   return scale > 0.0 && scale < 1.0e30;
 }
 

@@ -98,7 +98,7 @@ __device__ __forceinline__ bf16_t narrow<bf16_t>(float v) {
 // Valid band columns of sequence row i: [lo, hi) (reference tests/utils.py:79-81).
 __device__ __forceinline__ void valid_columns(int i, int M, int w, int *lo, int *hi) {
   *lo = max(w - i, 0);
-  *hi = min(2 * w + 1, M + w - i);
+  *hi = (int)min((int64_t)(2 * w + 1), (int64_t)M + w - i);  // M + w may exceed 32 bits
 }
 
 // ---------------------------------------------------------------------------------------------
