@@ -19,6 +19,7 @@ the count but its time is inside the step).  Next to it:
                 restatement, one thread, on a slice of the batch.
 
 Usage: python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c2|c4] [--no-cpu]
+       python bench.py --kernels-only [--shape B M N w] [--dtype bf16|fp16] [--family auto|wide|strided]
 """
 import argparse
 import json
@@ -140,6 +141,12 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="c3", choices=sorted(WORKLOADS))
+    ap.add_argument("--shape", type=int, nargs=4, metavar=("B", "M", "N", "w"),
+                    help="time this shape instead of a named workload (forward + backward)")
+    ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp16"], help="storage type for --shape")
+    ap.add_argument("--family", default="auto", choices=["auto", "wide", "strided"],
+                    help="kernel family for the per-kernel timings: the library's choice, the wide-band MFMA "
+                         "kernels even for a narrow band, or the strided kernels (A/B measurements)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--kernels-only", action="store_true",
                     help="launch each of the six kernels --steps times and a reference copy, nothing else "
@@ -157,6 +164,12 @@ def main():
     from window_matmul import band_softmax, unwindow_matmul, window_attention, window_matmul
 
     cfg = WORKLOADS[args.workload]
+    if args.shape:
+        sb, sm, sn, sw = args.shape
+        cfg = dict(B=sb, M=sm, N=sn, w=sw, dtype=args.dtype, qk_scale=sn ** -0.25, backward=True,
+                   label=f"B{sb} M{sm} N{sn} w{sw} {args.dtype}, window->softmax->unwindow, fwd+bwd")
+        args.workload = "custom"
+    fam = {"auto": 0, "wide": abi.NO_NARROW_BAND, "strided": abi.FORCE_STRIDED}[args.family]
     B, M, N, w = cfg["B"], cfg["M"], cfg["N"], cfg["w"]
     dtype = {"bf16": torch.bfloat16, "fp16": torch.float16}[cfg["dtype"]]
     es = 2
@@ -226,15 +239,15 @@ def main():
         ga = torch.randn(B, M, 2 * w + 1, generator=g).to(dtype).to(dev) if cfg["backward"] else None
         qd, vd = q.detach(), v.detach()
         launches = {
-            "window_fwd(P1)": lambda: abi.window_forward(qd, kt, w, out=att),
-            "unwindow_fwd(P2)": lambda: abi.unwindow_forward(probs, vd, w),
+            "window_fwd(P1)": lambda: abi.window_forward(qd, kt, w, fam, out=att),
+            "unwindow_fwd(P2)": lambda: abi.unwindow_forward(probs, vd, w, fam),
         }
         if cfg["backward"]:
             launches.update({
-                "grad_a(P1)": lambda: abi.unwindow_backward(probs, vd, w, go, want_v=False),
-                "grad_v(P3)": lambda: abi.unwindow_backward(probs, vd, w, go, want_a=False),
-                "grad_q(P2)": lambda: abi.window_backward(qd, kt, w, ga, want_k=False),
-                "grad_k(P3)": lambda: abi.window_backward(qd, kt, w, ga, want_q=False),
+                "grad_a(P1)": lambda: abi.unwindow_backward(probs, vd, w, go, fam, want_v=False),
+                "grad_v(P3)": lambda: abi.unwindow_backward(probs, vd, w, go, fam, want_a=False),
+                "grad_q(P2)": lambda: abi.window_backward(qd, kt, w, ga, fam, want_k=False),
+                "grad_k(P3)": lambda: abi.window_backward(qd, kt, w, ga, fam, want_q=False),
             })
         kb = kernel_bytes(B, M, N, w, es)
         per_kernel = {}
@@ -297,7 +310,8 @@ def main():
         "kernel_sum_GBps": round(len(per_kernel) * kb / sum(v["ms"] for v in per_kernel.values()) / 1e6, 1),
     }
     if args.kernels_only:
-        print(json.dumps({"kernels": per_kernel, "copy_yardstick_GBps": round(copy_gbs, 1),
+        print(json.dumps({"workload": cfg["label"], "family": args.family, "kernels": per_kernel,
+                          "copy_yardstick_GBps": round(copy_gbs, 1),
                           "copy_bytes_each_way": att.numel() * es}), flush=True)
         return
     if not args.no_cpu:

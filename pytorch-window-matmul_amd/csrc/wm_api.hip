@@ -46,7 +46,7 @@ int p2(const Problem &p, const View &a, const View &y, const View &c) {
   return run_primitive(try_launch_small_p2, try_launch_mfma_p2, try_launch_f32_p2, launch_strided_p2, p, a, y, c);
 }
 int p3(const Problem &p, const View &a, const View &y, const View &c) {
-  return run_primitive(nullptr, try_launch_mfma_p3, try_launch_f32_p3, launch_strided_p3, p, a, y, c);
+  return run_primitive(try_launch_small_p3, try_launch_mfma_p3, try_launch_f32_p3, launch_strided_p3, p, a, y, c);
 }
 
 }  // namespace

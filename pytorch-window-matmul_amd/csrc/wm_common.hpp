@@ -44,9 +44,10 @@ hipError_t launch_strided_p3(const Problem &p, const View &a, const View &y, con
 bool try_launch_mfma_p1(const Problem &p, const View &x, const View &y, const View &c, hipError_t *err);
 bool try_launch_mfma_p2(const Problem &p, const View &a, const View &y, const View &c, hipError_t *err);
 bool try_launch_mfma_p3(const Problem &p, const View &a, const View &y, const View &c, hipError_t *err);
-// Narrow-band family (w <= 32): P1 for any such w, P2 for w % 4 == 0.
+// Narrow-band family (w <= 32): P1 for any such w, P2 and P3 for w % 4 == 0.
 bool try_launch_small_p1(const Problem &p, const View &x, const View &y, const View &c, hipError_t *err);
 bool try_launch_small_p2(const Problem &p, const View &a, const View &y, const View &c, hipError_t *err);
+bool try_launch_small_p3(const Problem &p, const View &a, const View &y, const View &c, hipError_t *err);
 bool small_supports(int op, int64_t M, int64_t N, int64_t w, int dtype);
 // float32 MFMA family (N multiple of 8 up to 128, w >= 4).
 bool try_launch_f32_p1(const Problem &p, const View &x, const View &y, const View &c, hipError_t *err);

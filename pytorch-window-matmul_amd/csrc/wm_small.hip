@@ -255,6 +255,134 @@ __global__ __launch_bounds__(kThreads) void small_p2_kernel(const uint16_t *__re
 }
 
 // ------------------------------------------------------------------------------------------
+// P3 narrow: C[b,c,h] = sum_r A[b,r,c-r+w] * Y[b,r,h]      (w % 4 == 0)
+// ------------------------------------------------------------------------------------------
+// Output-stationary like the wide kernel, staged like the narrow P2: a workgroup owns ROWS
+// output rows c and copies the band rows r in [c_first - w, c_last + w] flat into LDS, plus
+// the Y rows of the same range.  Band entry (r, c) has flat element index r*2w + c + w (+ base),
+// so with 2w a multiple of 8 the image is a matrix Mat[r][c] with row stride 2w whose 16-byte
+// chunk grid along c is the same in every row: output tiles are laid on that grid (shifted by
+// `shift` = (base + w) mod 8 against c = 0, the same for all workgroups of a batch element) and
+// ds_read_b64_tr_b16 then delivers, per lane c, the entries of 8 consecutive r: the B operand.
+template <typename T, int NT, int RW>  // N <= 32 NT; RW output rows per wave (64 or 32)
+__global__ __launch_bounds__(kThreads) void small_p3_kernel(const uint16_t *__restrict__ A,
+                                                            const uint16_t *__restrict__ Y,
+                                                            uint16_t *__restrict__ C, int B, int M, int N, int w,
+                                                            int nblk, int64_t asb, int64_t ysb, int64_t ysr,
+                                                            int64_t csb, int64_t csr) {
+  constexpr int ROWS = 4 * RW;
+  constexpr int SY = lds_stride_tr(32 * NT);
+  extern __shared__ __attribute__((aligned(16))) uint16_t lds[];
+  const int W = 2 * w + 1;
+  const int span = ROWS + 2 * w;                         // band / Y rows a workgroup can touch
+  const int a_elems = ((span * W + 16 + 7) >> 3) << 3;   // flat band image, whole 16-byte chunks
+  uint16_t *aimg = lds;
+  // Y rows r_org .. r_org + span + 15 (the last 16-row step may run past the span), stride SY, zero
+  // outside the sequence and all initialised: they meet masked zeros of the band inside the MFMA
+  uint16_t *yimg = lds + a_elems;
+
+  int b, blk;
+  if (!decode_block(nblk, B, &b, &blk)) return;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int64_t base_el = (int64_t)(reinterpret_cast<uintptr_t>(A) >> 1) + (int64_t)b * asb;
+  const int shift = (int)((base_el + w) & 7);
+  const int c_first = blk * ROWS - shift;  // first output row of this workgroup (may be < 0)
+  if (c_first >= M) return;
+  const int r_org = c_first - w;           // band row that image row 0 stands for (may be < 0)
+  const int r_s = max(r_org, 0), r_e = min(r_org + span - 1, M - 1);  // rows that exist
+  const uint16_t *Yb = Y + (int64_t)b * ysb;
+  // global element index of image element 0, rounded down to a chunk: g0 = base + r_org * W - delta
+  const int64_t g_org = base_el + (int64_t)r_org * W;
+  const int delta = (int)(g_org & 7);
+  const uint16_t *img_src = A + ((g_org - delta) - (int64_t)(reinterpret_cast<uintptr_t>(A) >> 1));
+
+  // flat band rows r_s..r_e: whole aligned chunks (neighbours' entries at both ends are masked later)
+  const int q_lo = (delta + (r_s - r_org) * W) >> 3;
+  const int q_hi = (delta + (r_e + 1 - r_org) * W + 7) >> 3;  // exclusive
+  const int chunks = max(q_hi - q_lo, 0);
+  const int ncg = N >> 3;
+  const int ychunks = (span + 16) * ncg;
+  constexpr int BATCH = 8;
+  for (int base = 0; base < chunks + ychunks; base += BATCH * kThreads) {
+    u32x4 reg[BATCH];
+#pragma unroll
+    for (int s = 0; s < BATCH; ++s) {
+      const int q = base + s * kThreads + tid;
+      const int qy = q - chunks, yr = qy / ncg, hg = qy - yr * ncg, r = r_org + yr;
+      const uint16_t *src = q < chunks ? img_src + 8 * (int64_t)(q_lo + q) : Yb + (int64_t)r * ysr + 8 * hg;
+      const bool ok = q < chunks || (q < chunks + ychunks && r >= 0 && r < M);
+      reg[s] = *reinterpret_cast<const u32x4 *>(ok ? src : A);
+    }
+#pragma unroll
+    for (int s = 0; s < BATCH; ++s) {
+      const int q = base + s * kThreads + tid;
+      const int qy = q - chunks, yr = qy / ncg, hg = qy - yr * ncg, r = r_org + yr;
+      if (q < chunks)
+        *reinterpret_cast<u32x4 *>(aimg + 8 * (q_lo + q)) = reg[s];
+      else if (q < chunks + ychunks)
+        *reinterpret_cast<u32x4 *>(yimg + yr * SY + 8 * hg) = mask_row_chunk(reg[s], (r >= 0) & (r < M));
+    }
+  }
+  __syncthreads();
+
+  const int nks = (32 + 2 * w + 15) >> 4;  // 16-row steps covering the band rows of one 32-row output tile
+  u32x2 outp[RW / 32][NT][4];
+#pragma unroll
+  for (int nt = 0; nt < RW / 32; ++nt) {
+    const int t0 = RW * wave + 32 * nt;        // first output row of the tile, relative to c_first
+    const int c = c_first + t0 + (lane & 31);  // this lane's output row
+    f32x16 acc[NT];
+#pragma unroll
+    for (int t = 0; t < NT; ++t)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[t][v] = 0.f;
+    // Mat[k][x]: k = r - r_org, x = c - r_org + w = t0 + (lane & 31) + 2w; element delta + k*2w + x
+    for (int ks = 0; ks < nks; ++ks) {
+      const int k0 = t0 + 16 * ks;                       // image row of band row c_tile - w + 16 ks
+      const int r_g = r_org + k0 + 8 * (lane >> 5);      // band row of this lane's element 0
+      u32x4 bop = lds_read_transposed(aimg + delta, 2 * w, k0, t0 + 2 * w, lane);
+      // element e is band row r_g + e: valid iff |r - c| <= w and 0 <= r < M
+      const int e_lo = max(c - w - r_g, -r_g);
+      const int e_hi = min(c + w - r_g, M - 1 - r_g);
+      bop = mask_band_chunk(bop, e_lo, e_hi);
+#pragma unroll
+      for (int t = 0; t < NT; ++t) {
+        const u32x4 aop = lds_read_transposed(yimg, SY, k0, 32 * t, lane);
+        acc[t] = Mma<T>::run(aop, bop, acc[t]);
+      }
+    }
+#pragma unroll
+    for (int t = 0; t < NT; ++t)
+#pragma unroll
+      for (int q4 = 0; q4 < 4; ++q4) {
+        outp[nt][t][q4][0] = Mma<T>::pack2(acc[t][4 * q4], acc[t][4 * q4 + 1]);
+        outp[nt][t][q4][1] = Mma<T>::pack2(acc[t][4 * q4 + 2], acc[t][4 * q4 + 3]);
+      }
+  }
+  // results leave through LDS as row-contiguous 16-byte stores; the staging area reuses the images
+  __syncthreads();
+  constexpr int SO = 32 * NT + 8;
+  uint16_t *stage = lds + wave * (RW * SO);
+#pragma unroll
+  for (int nt = 0; nt < RW / 32; ++nt)
+#pragma unroll
+    for (int t = 0; t < NT; ++t)
+#pragma unroll
+      for (int q4 = 0; q4 < 4; ++q4)
+        *reinterpret_cast<u32x2 *>(stage + (32 * nt + (lane & 31)) * SO + 32 * t + 8 * q4 + 4 * (lane >> 5)) =
+            outp[nt][t][q4];
+  wave_sync_lds();
+  const int per_row = N >> 3;
+  for (int q = lane; q < RW * per_row; q += 64) {
+    const int r = q / per_row, hg = q - r * per_row;
+    const int c = c_first + RW * wave + r;
+    if (c >= 0 && c < M)
+      *reinterpret_cast<u32x4 *>(C + (int64_t)b * csb + (int64_t)c * csr + 8 * hg) =
+          *reinterpret_cast<const u32x4 *>(stage + r * SO + 8 * hg);
+  }
+}
+
+// ------------------------------------------------------------------------------------------
 // host side
 // ------------------------------------------------------------------------------------------
 bool small_shape_ok(int64_t M, int64_t N, int64_t w, int dtype) {
@@ -295,27 +423,69 @@ hipError_t launch_small_p1(const Problem &p, const View &x, const View &y, const
   return hipGetLastError();
 }
 
+// LDS bytes of the P2 kernel: flat band image of `rows` rows plus the Y rows they reach.
+size_t small_p2_lds(int64_t rows, int64_t w, int64_t NT) {
+  const int64_t W = 2 * w + 1;
+  const size_t a_elems = (size_t)(((rows * W + 16 + 7) >> 3) << 3);
+  return (a_elems + (size_t)(rows + 2 * w + 32) * (32 * NT + 16)) * 2;
+}
+constexpr size_t kSmallLdsLimit = 65536;  // default limit for dynamic LDS
+// Rows per wave: 64 for N <= 64 while the two images fit, else 32.
+int small_p2_rows_per_wave(int64_t w, int64_t NT) {
+  return NT <= 2 && small_p2_lds(256, w, NT) <= kSmallLdsLimit ? 64 : 32;
+}
+
 template <typename T>
 hipError_t launch_small_p2(const Problem &p, const View &a, const View &y, const View &c) {
   const int NT = (int)((p.N + 31) / 32);
-  const int RW = NT <= 2 ? 64 : 32;
+  const int RW = small_p2_rows_per_wave(p.w, NT);
   const int rows = 4 * RW;
   const int nblk = (int)((p.M + rows - 1) / rows);
   const dim3 grid(small_grid(p.B, nblk)), block(kThreads);
-  const int64_t W = 2 * p.w + 1;
-  const size_t a_elems = (size_t)(((rows * W + 16 + 7) >> 3) << 3);
-  const size_t lds = (a_elems + (size_t)(rows + 2 * p.w + 32) * (32 * NT + 16)) * 2;
+  const size_t lds = small_p2_lds(rows, p.w, NT);
 #define WM_SP2(NT_, RW_)                                                                                       \
   hipLaunchKernelGGL((small_p2_kernel<T, NT_, RW_>), grid, block, lds, p.stream, (const uint16_t *)a.data,     \
                      (const uint16_t *)y.data, (uint16_t *)c.data, (int)p.B, (int)p.M, (int)p.N, (int)p.w, nblk, \
                      a.sb, y.sb, y.sr, c.sb, c.sr)
   switch (NT) {
-    case 1: WM_SP2(1, 64); break;
-    case 2: WM_SP2(2, 64); break;
+    case 1: if (RW == 64) WM_SP2(1, 64); else WM_SP2(1, 32); break;
+    case 2: if (RW == 64) WM_SP2(2, 64); else WM_SP2(2, 32); break;
     case 3: WM_SP2(3, 32); break;
     default: WM_SP2(4, 32); break;
   }
 #undef WM_SP2
+  return hipGetLastError();
+}
+
+// LDS bytes of the P3 kernel: flat image of rows + 2w band rows plus as many Y rows.
+size_t small_p3_lds(int64_t rows, int64_t w, int64_t NT) {
+  const int64_t W = 2 * w + 1, span = rows + 2 * w;
+  const size_t a_elems = (size_t)(((span * W + 16 + 7) >> 3) << 3);
+  return (a_elems + (size_t)(span + 16) * (32 * NT + 16)) * 2;
+}
+int small_p3_rows_per_wave(int64_t w, int64_t NT) {
+  return NT <= 2 && small_p3_lds(256, w, NT) <= kSmallLdsLimit ? 64 : 32;
+}
+
+template <typename T>
+hipError_t launch_small_p3(const Problem &p, const View &a, const View &y, const View &c) {
+  const int NT = (int)((p.N + 31) / 32);
+  const int RW = small_p3_rows_per_wave(p.w, NT);
+  const int rows = 4 * RW;
+  const int nblk = (int)((p.M + 7 + rows - 1) / rows);  // output tiles start up to 7 rows before row 0
+  const dim3 grid(small_grid(p.B, nblk)), block(kThreads);
+  const size_t lds = small_p3_lds(rows, p.w, NT);
+#define WM_SP3(NT_, RW_)                                                                                       \
+  hipLaunchKernelGGL((small_p3_kernel<T, NT_, RW_>), grid, block, lds, p.stream, (const uint16_t *)a.data,     \
+                     (const uint16_t *)y.data, (uint16_t *)c.data, (int)p.B, (int)p.M, (int)p.N, (int)p.w, nblk, \
+                     a.sb, y.sb, y.sr, c.sb, c.sr)
+  switch (NT) {
+    case 1: if (RW == 64) WM_SP3(1, 64); else WM_SP3(1, 32); break;
+    case 2: if (RW == 64) WM_SP3(2, 64); else WM_SP3(2, 32); break;
+    case 3: WM_SP3(3, 32); break;
+    default: WM_SP3(4, 32); break;
+  }
+#undef WM_SP3
   return hipGetLastError();
 }
 
@@ -326,7 +496,15 @@ bool band_contiguous(const View &v, int64_t W) { return v.sc == 1 && v.sr == W &
 bool small_supports(int op, int64_t M, int64_t N, int64_t w, int dtype) {
   if (!small_shape_ok(M, N, w, dtype)) return false;
   if (op == 1) return true;
-  if (op == 2) return w % 4 == 0;
+  if (op == 2) {
+    // the two LDS images must fit the default 64 KB dynamic limit; wider cases go to the wide-band family
+    const int64_t NT = (N + 31) / 32;
+    return w % 4 == 0 && small_p2_lds(4 * small_p2_rows_per_wave(w, NT), w, NT) <= kSmallLdsLimit;
+  }
+  if (op == 3) {
+    const int64_t NT = (N + 31) / 32;
+    return w % 4 == 0 && small_p3_lds(4 * small_p3_rows_per_wave(w, NT), w, NT) <= kSmallLdsLimit;
+  }
   return false;
 }
 
@@ -339,12 +517,15 @@ bool try_launch_small_p1(const Problem &p, const View &x, const View &y, const V
 
 bool try_launch_small_p2(const Problem &p, const View &a, const View &y, const View &c, hipError_t *err) {
   if (!small_supports(2, p.M, p.N, p.w, p.dtype)) return false;
-  {  // the two LDS images must fit the default 64 KB dynamic limit; wider cases go to the wide-band family
-    const int64_t NT = (p.N + 31) / 32, rows = NT <= 2 ? 256 : 128, W = 2 * p.w + 1;
-    if ((rows * W + 24 + (rows + 2 * p.w + 32) * (32 * NT + 16)) * 2 > 65536) return false;
-  }
   if (!band_contiguous(a, 2 * p.w + 1) || !fast_layout(y, p.dtype) || !fast_layout(c, p.dtype)) return false;
   *err = p.dtype == WM_DTYPE_BF16 ? launch_small_p2<bf16_t>(p, a, y, c) : launch_small_p2<f16_t>(p, a, y, c);
+  return true;
+}
+
+bool try_launch_small_p3(const Problem &p, const View &a, const View &y, const View &c, hipError_t *err) {
+  if (!small_supports(3, p.M, p.N, p.w, p.dtype)) return false;
+  if (!band_contiguous(a, 2 * p.w + 1) || !fast_layout(y, p.dtype) || !fast_layout(c, p.dtype)) return false;
+  *err = p.dtype == WM_DTYPE_BF16 ? launch_small_p3<bf16_t>(p, a, y, c) : launch_small_p3<f16_t>(p, a, y, c);
   return true;
 }
 

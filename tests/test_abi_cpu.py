@@ -51,13 +51,16 @@ def test_kernel_choice_names():
     assert L.wm_kernel_choice(1, 2, 128, 64, 4, 0, 1, abi.FORCE_STRIDED) == b"strided_p1"
     assert L.wm_kernel_choice(3, 2, 128, 64, 4, 3, 1, 0) == b"strided_p3"  # float64 has no MFMA path
     assert L.wm_kernel_choice(9, 2, 128, 64, 4, 0, 1, 0) == b"invalid"
-    # per family: float32 MFMA, 16-bit wide band, 16-bit narrow band (P1 any w <= 32, P2 for w % 4 == 0)
+    # per family: float32 MFMA, 16-bit wide band, 16-bit narrow band (P1 any w <= 32, P2 and P3 for w % 4 == 0)
     assert L.wm_kernel_choice(1, 7, 3001, 80, 1500, 0, 1, 0) == b"f32_mfma_p1"
     assert L.wm_kernel_choice(2, 96, 4096, 64, 256, 2, 1, 0) == b"mfma_p2"
     assert L.wm_kernel_choice(1, 96, 16384, 64, 8, 2, 1, 0) == b"narrow_p1"
     assert L.wm_kernel_choice(2, 96, 16384, 64, 8, 1, 1, 0) == b"narrow_p2"
     assert L.wm_kernel_choice(2, 96, 16384, 64, 9, 2, 1, 0) == b"mfma_p2"
-    assert L.wm_kernel_choice(3, 96, 16384, 64, 8, 2, 1, 0) == b"mfma_p3"
+    assert L.wm_kernel_choice(3, 96, 16384, 64, 8, 2, 1, 0) == b"narrow_p3"
+    assert L.wm_kernel_choice(3, 96, 16384, 64, 10, 2, 1, 0) == b"mfma_p3"
+    assert L.wm_kernel_choice(2, 96, 16384, 64, 32, 2, 1, 0) == b"narrow_p2"  # 32 rows per wave still fit LDS
+    assert L.wm_kernel_choice(3, 96, 16384, 128, 32, 2, 1, 0) == b"mfma_p3"   # images beyond 64 KB of LDS
     assert L.wm_kernel_choice(1, 96, 16384, 64, 8, 2, 1, abi.NO_NARROW_BAND) == b"mfma_p1"
     assert L.wm_kernel_choice(1, 2, 128, 3, 4, 0, 1, 0) == b"strided_p1"  # N not a multiple of 8
     assert L.wm_kernel_choice(1, 2, 128, 64, 4, 2, 0, 0) == b"strided_p1"  # layout not vector friendly
