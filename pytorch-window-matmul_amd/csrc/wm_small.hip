@@ -248,9 +248,9 @@ __global__ __launch_bounds__(kThreads) void small_p2_kernel(const uint16_t *__re
   for (int q = lane; q < RW * per_row; q += 64) {
     const int r = q / per_row, hg = q - r * per_row;
     const int i = i0 + RW * wave + r;
-    if (i < M)
-      *reinterpret_cast<u32x4 *>(C + (int64_t)b * csb + (int64_t)i * csr + 8 * hg) =
-          *reinterpret_cast<const u32x4 *>(stage + r * SO + 8 * hg);
+    if (i < M)  // whole 128-byte lines, written once and not read again here: non-temporal
+      store_chunk_streaming(C + (int64_t)b * csb + (int64_t)i * csr + 8 * hg,
+                            *reinterpret_cast<const u32x4 *>(stage + r * SO + 8 * hg));
   }
 }
 
@@ -377,8 +377,8 @@ __global__ __launch_bounds__(kThreads) void small_p3_kernel(const uint16_t *__re
     const int r = q / per_row, hg = q - r * per_row;
     const int c = c_first + RW * wave + r;
     if (c >= 0 && c < M)
-      *reinterpret_cast<u32x4 *>(C + (int64_t)b * csb + (int64_t)c * csr + 8 * hg) =
-          *reinterpret_cast<const u32x4 *>(stage + r * SO + 8 * hg);
+      store_chunk_streaming(C + (int64_t)b * csb + (int64_t)c * csr + 8 * hg,
+                            *reinterpret_cast<const u32x4 *>(stage + r * SO + 8 * hg));
   }
 }
 
