@@ -160,3 +160,28 @@ def test_python_function_falls_back_to_the_separate_ops(device):
     # window_size 0: the value itself
     q = seeded((2, 5, 64), 85, torch.bfloat16).to(device)
     torch.testing.assert_close(window_attention(q, q, q, 0), q)
+
+
+def test_long_sequence_wide_head_against_separate_ops(device):
+    """B=16 M=32768 N=128 w=512 float16 (the widest kernels, one wavefront per SIMD in the backward):
+    fused forward and backward against the chain of the separate ops with torch autograd."""
+    from window_matmul import unwindow_matmul, window_attention, window_matmul
+
+    B, M, N, w = 16, 32768, 128, 512
+    g = torch.Generator().manual_seed(11)
+    q0, k0, v0, go = ((torch.randn(B, M, N, generator=g) * s).to(torch.float16).to(device) for s in (1, 1, 1, 1))
+    scale = 1.0 / math.sqrt(N)
+    res = {}
+    for name in ("chain", "fused"):
+        q, k, v = (t.clone().requires_grad_(True) for t in (q0, k0, v0))
+        if name == "chain":
+            att = window_matmul(q, k.transpose(1, 2), w).float() * scale
+            out = unwindow_matmul(torch.softmax(att, -1).to(torch.float16), v, w)
+            del att
+        else:
+            out = window_attention(q, k, v, w)
+        out.backward(go)
+        res[name] = (out.detach(), q.grad, k.grad, v.grad)
+    for x, y in zip(res["fused"], res["chain"]):
+        torch.testing.assert_close(x.float(), y.float(), **TOL)
+        assert torch.isfinite(x).all()
