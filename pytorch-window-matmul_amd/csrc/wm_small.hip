@@ -3,12 +3,14 @@
 // With a narrow band the whole band of a block of rows is small (256 rows x 17 entries =
 // 8.7 KB at w = 8), the op is a pure stream over Q/K (P1) or V/O (P2), and the dense tiles of
 // the wide-band kernels would waste most of their work and all of their barriers.  Here a
-// wave owns 64 (or 32) consecutive rows and everything it needs:
+// wave owns 64 (P1) or 32 (P2, P3) consecutive rows and everything it needs:
 //
 //   P1  the wave loads its rows of X and the rows [r0-w, r0+64+w) of Y straight from HBM
 //       into MFMA operand registers (no LDS, no barrier), forms the 32x32 tiles that touch
 //       the band, and scatters the band entries into a flat LDS image of the workgroup's
 //       band rows, which then leaves as aligned 16-byte stores.
+//       (Staging the operands in LDS with coalesced loads, 32 rows per wave, and replacing the
+//       scatter by dense staging tiles were both measured: within 5 % either way, not kept.)
 //   P2  the workgroup copies its band rows flat into LDS (aligned 16-byte loads) and the
 //       rows [i0-w, i0+rows+w) of Y row-major into LDS; each wave then multiplies its rows:
 //       the skewed tile is read back with ds_read_b128 (the flat image keeps 8-column groups
@@ -430,10 +432,10 @@ size_t small_p2_lds(int64_t rows, int64_t w, int64_t NT) {
   return (a_elems + (size_t)(rows + 2 * w + 32) * (32 * NT + 16)) * 2;
 }
 constexpr size_t kSmallLdsLimit = 65536;  // default limit for dynamic LDS
-// Rows per wave: 64 for N <= 64 while the two images fit, else 32.
-int small_p2_rows_per_wave(int64_t w, int64_t NT) {
-  return NT <= 2 && small_p2_lds(256, w, NT) <= kSmallLdsLimit ? 64 : 32;
-}
+// Rows per wave.  64 (256-row workgroups) were measured 20-30 % slower than 32 at every narrow
+// window: the LDS images of a 256-row workgroup allow two workgroups per CU, and these kernels
+// (load everything, barrier, multiply, barrier, store) need more of them in flight to overlap.
+int small_p2_rows_per_wave(int64_t, int64_t) { return 32; }
 
 template <typename T>
 hipError_t launch_small_p2(const Problem &p, const View &a, const View &y, const View &c) {
@@ -448,8 +450,8 @@ hipError_t launch_small_p2(const Problem &p, const View &a, const View &y, const
                      (const uint16_t *)y.data, (uint16_t *)c.data, (int)p.B, (int)p.M, (int)p.N, (int)p.w, nblk, \
                      a.sb, y.sb, y.sr, c.sb, c.sr)
   switch (NT) {
-    case 1: if (RW == 64) WM_SP2(1, 64); else WM_SP2(1, 32); break;
-    case 2: if (RW == 64) WM_SP2(2, 64); else WM_SP2(2, 32); break;
+    case 1: WM_SP2(1, 32); break;
+    case 2: WM_SP2(2, 32); break;
     case 3: WM_SP2(3, 32); break;
     default: WM_SP2(4, 32); break;
   }
@@ -463,9 +465,7 @@ size_t small_p3_lds(int64_t rows, int64_t w, int64_t NT) {
   const size_t a_elems = (size_t)(((span * W + 16 + 7) >> 3) << 3);
   return (a_elems + (size_t)(span + 16) * (32 * NT + 16)) * 2;
 }
-int small_p3_rows_per_wave(int64_t w, int64_t NT) {
-  return NT <= 2 && small_p3_lds(256, w, NT) <= kSmallLdsLimit ? 64 : 32;
-}
+int small_p3_rows_per_wave(int64_t, int64_t) { return 32; }
 
 template <typename T>
 hipError_t launch_small_p3(const Problem &p, const View &a, const View &y, const View &c) {
@@ -480,8 +480,8 @@ hipError_t launch_small_p3(const Problem &p, const View &a, const View &y, const
                      (const uint16_t *)y.data, (uint16_t *)c.data, (int)p.B, (int)p.M, (int)p.N, (int)p.w, nblk, \
                      a.sb, y.sb, y.sr, c.sb, c.sr)
   switch (NT) {
-    case 1: if (RW == 64) WM_SP3(1, 64); else WM_SP3(1, 32); break;
-    case 2: if (RW == 64) WM_SP3(2, 64); else WM_SP3(2, 32); break;
+    case 1: WM_SP3(1, 32); break;
+    case 2: WM_SP3(2, 32); break;
     case 3: WM_SP3(3, 32); break;
     default: WM_SP3(4, 32); break;
   }
