@@ -157,7 +157,9 @@ int wm_window_attention_forward(const wm_operand *q, const wm_operand *k, const 
  * lse, and the upstream gradient grad_o, writes grad_q, grad_k, grad_v (all (B, M, N) operands,
  * k and grad_k as key rows).  delta is a caller-owned float32 workspace of B * M values (it
  * receives sum_h grad_o * o per row).  The masking choice of the forward is carried by lse and
- * needs no argument here.  Two kernels are enqueued on the stream; no atomics, so results are
+ * needs no argument here.  Any of grad_q, grad_k, grad_v may be NULL to skip that gradient
+ * (grad_q NULL shortens the first kernel to the delta pass, grad_k and grad_v both NULL drop the
+ * second).  Up to two kernels are enqueued on the stream; no atomics, so results are
  * reproducible run to run.  Same support rule and WM_ERR_UNSUPPORTED behaviour as the forward.
  * No counterpart in the reference's native module (see the forward). */
 int wm_window_attention_backward(const wm_operand *q, const wm_operand *k, const wm_operand *v,

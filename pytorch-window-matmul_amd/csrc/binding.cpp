@@ -258,9 +258,10 @@ std::tuple<torch::Tensor, torch::Tensor> window_attention_forward(torch::Tensor 
   return std::make_tuple(o, lse);
 }
 
-std::tuple<torch::Tensor, torch::Tensor, torch::Tensor> window_attention_backward(
-    torch::Tensor q, torch::Tensor k, torch::Tensor v, torch::Tensor o, torch::Tensor lse, torch::Tensor grad_output,
-    int64_t window_size, double scale) {
+std::tuple<c10::optional<torch::Tensor>, c10::optional<torch::Tensor>, c10::optional<torch::Tensor>>
+window_attention_backward(torch::Tensor q, torch::Tensor k, torch::Tensor v, torch::Tensor o, torch::Tensor lse,
+                          torch::Tensor grad_output, int64_t window_size, double scale, bool need_q, bool need_k,
+                          bool need_v) {
   check_attention_inputs(q, k, v);
   check_grad(grad_output, q, q.sizes().vec());
   check_grad(o, q, q.sizes().vec());
@@ -272,14 +273,16 @@ std::tuple<torch::Tensor, torch::Tensor, torch::Tensor> window_attention_backwar
   const int64_t B = q.size(0), M = q.size(1), N = q.size(2);
   auto qq = vector_friendly(q), kk = vector_friendly(k), vv = vector_friendly(v), oo = vector_friendly(o),
        go = vector_friendly(grad_output);
-  auto gq = torch::empty({B, M, N}, q.options()), gk = torch::empty({B, M, N}, q.options()),
-       gv = torch::empty({B, M, N}, q.options());
+  c10::optional<torch::Tensor> gq, gk, gv;
+  wm_operand f{}, g{}, h{};
+  if (need_q) gq = torch::empty({B, M, N}, q.options()), f = operand(*gq);
+  if (need_k) gk = torch::empty({B, M, N}, q.options()), g = operand(*gk);
+  if (need_v) gv = torch::empty({B, M, N}, q.options()), h = operand(*gv);
   auto delta = torch::empty({B, M}, lse.options());
-  wm_operand a = operand(qq), b = operand(kk), c = operand(vv), d = operand(oo), e = operand(go), f = operand(gq),
-             g = operand(gk), h = operand(gv);
-  raise_on_error(wm_window_attention_backward(&a, &b, &c, &d, lse.data_ptr<float>(), &e, &f, &g, &h,
-                                              delta.data_ptr<float>(), B, M, N, window_size, scale, dtype, 0,
-                                              current_stream(q)),
+  wm_operand a = operand(qq), b = operand(kk), c = operand(vv), d = operand(oo), e = operand(go);
+  raise_on_error(wm_window_attention_backward(&a, &b, &c, &d, lse.data_ptr<float>(), &e, need_q ? &f : nullptr,
+                                              need_k ? &g : nullptr, need_v ? &h : nullptr, delta.data_ptr<float>(),
+                                              B, M, N, window_size, scale, dtype, 0, current_stream(q)),
                  "window_attention_backward");
   return std::make_tuple(gq, gk, gv);
 }
@@ -306,6 +309,7 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
         py::arg("mask_out_of_range") = false);
   m.def("window_attention_backward", &window_attention_backward, "fused window attention backward -> (gq, gk, gv)",
         py::arg("q"), py::arg("k"), py::arg("v"), py::arg("o"), py::arg("lse"), py::arg("grad_output"),
-        py::arg("window_size"), py::arg("scale"));
+        py::arg("window_size"), py::arg("scale"), py::arg("need_q") = true, py::arg("need_k") = true,
+        py::arg("need_v") = true);
   m.def("abi_version", []() { return wm_abi_version(); }, "ABI version of libwindow_matmul_hip.so");
 }

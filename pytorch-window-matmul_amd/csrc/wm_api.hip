@@ -154,13 +154,16 @@ int wm_window_attention_backward(const wm_operand *q, const wm_operand *k, const
   if (int st = check_common(B, M, N, w, dtype, flags)) return st;
   if (!(scale == scale)) return WM_ERR_BAD_SHAPE;
   if (B == 0 || M == 0) return WM_OK;
-  if (missing(q) || missing(k) || missing(v) || missing(o) || missing(grad_o) || missing(grad_q) || missing(grad_k) ||
-      missing(grad_v) || lse == nullptr || delta == nullptr)
+  if (missing(q) || missing(k) || missing(v) || missing(o) || missing(grad_o) || lse == nullptr || delta == nullptr)
     return WM_ERR_NULL_POINTER;
+  if (grad_q == nullptr && grad_k == nullptr && grad_v == nullptr) return WM_OK;
+  if ((grad_q && !grad_q->data) || (grad_k && !grad_k->data) || (grad_v && !grad_v->data)) return WM_ERR_NULL_POINTER;
   const Problem prob{B, M, N, w, dtype, flags, static_cast<hipStream_t>(stream)};
+  const View none{nullptr, 0, 0, 0};
   hipError_t err = hipSuccess;
   if (!try_launch_attention_backward(prob, make_view(q), make_view(k), make_view(v), make_view(o), make_view(grad_o),
-                                     lse, delta, make_view(grad_q), make_view(grad_k), make_view(grad_v), scale, &err))
+                                     lse, delta, grad_q ? make_view(grad_q) : none, grad_k ? make_view(grad_k) : none,
+                                     grad_v ? make_view(grad_v) : none, scale, &err))
     return WM_ERR_UNSUPPORTED;
   return to_status(err);
 }

@@ -87,7 +87,7 @@ __device__ __forceinline__ void store_rows(uint16_t *row, const f32x16 (&acc)[NB
 // ---------------------------------------------------------------------------------------------
 // query kernel: dQ and D
 // ---------------------------------------------------------------------------------------------
-template <typename T, int NB>
+template <typename T, int NB, bool WITH_DQ>  // WITH_DQ false: only D is wanted (grad_q not requested)
 __global__ __launch_bounds__(kThreads, NB <= 2 ? 2 : 1) void attention_backward_query_kernel(
     const uint16_t *__restrict__ Q, const uint16_t *__restrict__ K, const uint16_t *__restrict__ V,
     const uint16_t *__restrict__ O, const uint16_t *__restrict__ dO, const float *__restrict__ L,
@@ -127,6 +127,7 @@ __global__ __launch_bounds__(kThreads, NB <= 2 ? 2 : 1) void attention_backward_
   }
   delta = halves_sum(delta);
   if (q_ok && half == 0) D[(int64_t)b * M + qi] = delta;
+  if (!WITH_DQ) return;
   const float l2 = (q_ok ? L[(int64_t)b * M + qi] : 0.0f) * 1.4426950408889634f;
   const float delta_s = delta * scale;
 
@@ -371,9 +372,9 @@ __global__ __launch_bounds__(kThreads, NB <= 2 ? 2 : 1) void attention_backward_
     stash(buf ^ 1);
     __syncthreads();
   }
-  if (k_ok) {
-    store_rows<T, NB>(dK + (int64_t)b * dksb + (int64_t)kj * dksr, dk, half);
-    store_rows<T, NB>(dV + (int64_t)b * dvsb + (int64_t)kj * dvsr, dv, half);
+  if (k_ok) {  // either output may be absent (gradient not requested)
+    if (dK != nullptr) store_rows<T, NB>(dK + (int64_t)b * dksb + (int64_t)kj * dksr, dk, half);
+    if (dV != nullptr) store_rows<T, NB>(dV + (int64_t)b * dvsb + (int64_t)kj * dvsr, dv, half);
   }
 }
 
@@ -387,12 +388,20 @@ hipError_t launch_backward(const Problem &p, const View &q, const View &k, const
   const dim3 grid((unsigned)(groups * 8 * nblk)), block(kThreads);
   typedef const uint16_t *in_t;
   typedef uint16_t *out_t;
-  hipLaunchKernelGGL((attention_backward_query_kernel<T, NB>), grid, block, 0, p.stream, (in_t)q.data, (in_t)k.data,
-                     (in_t)v.data, (in_t)o.data, (in_t)go.data, lse, (out_t)gq.data, delta, (int)p.B, (int)p.M,
-                     (int)p.w, nblk, (float)scale, q.sb, q.sr, k.sb, k.sr, v.sb, v.sr, o.sb, o.sr, go.sb, go.sr, gq.sb,
-                     gq.sr);
+#define WM_ABQ(WITH_DQ)                                                                                              \
+  hipLaunchKernelGGL((attention_backward_query_kernel<T, NB, WITH_DQ>), grid, block, 0, p.stream, (in_t)q.data,      \
+                     (in_t)k.data, (in_t)v.data, (in_t)o.data, (in_t)go.data, lse, (out_t)gq.data, delta, (int)p.B,  \
+                     (int)p.M, (int)p.w, nblk, (float)scale, q.sb, q.sr, k.sb, k.sr, v.sb, v.sr, o.sb, o.sr, go.sb,  \
+                     go.sr, gq.sb, gq.sr)
+  // D is needed by the key kernel even when grad_q is not: the query kernel then stops after writing it
+  if (gq.data != nullptr)
+    WM_ABQ(true);
+  else if (gk.data != nullptr || gv.data != nullptr)
+    WM_ABQ(false);
+#undef WM_ABQ
   hipError_t err = hipGetLastError();
   if (err != hipSuccess) return err;
+  if (gk.data == nullptr && gv.data == nullptr) return hipSuccess;
   hipLaunchKernelGGL((attention_backward_key_kernel<T, NB>), grid, block, 0, p.stream, (in_t)q.data, (in_t)k.data,
                      (in_t)v.data, (in_t)go.data, lse, (const float *)delta, (out_t)gk.data, (out_t)gv.data, (int)p.B,
                      (int)p.M, (int)p.w, nblk, (float)scale, q.sb, q.sr, k.sb, k.sr, v.sb, v.sr, go.sb, go.sr, gk.sb,
@@ -421,7 +430,7 @@ bool try_launch_attention_backward(const Problem &p, const View &q, const View &
   if (!attention_supports(p.M, p.N, p.w, p.dtype, scale)) return false;
   const View *all[] = {&q, &k, &v, &o, &go, &gq, &gk, &gv};
   for (const View *t : all)
-    if (!fast_layout(*t, p.dtype)) return false;
+    if (t->data != nullptr && !fast_layout(*t, p.dtype)) return false;  // absent outputs have no layout
   *err = p.dtype == WM_DTYPE_BF16 ? backward_by_width<bf16_t>(p, q, k, v, o, go, lse, delta, gq, gk, gv, scale)
                                   : backward_by_width<f16_t>(p, q, k, v, o, go, lse, delta, gq, gk, gv, scale);
   return true;

@@ -33,7 +33,8 @@ class WindowAttentionFunc(torch.autograd.Function):
     @staticmethod
     def backward(ctx, grad_output):
         q, k, v, out, lse = ctx.saved_tensors
-        gq, gk, gv = _native.window_attention_backward(q, k, v, out, lse, grad_output, ctx.window_size, ctx.scale)
+        gq, gk, gv = _native.window_attention_backward(q, k, v, out, lse, grad_output, ctx.window_size, ctx.scale,
+                                                       *ctx.needs_input_grad[:3])
         return gq, gk, gv, None, None, None
 
 

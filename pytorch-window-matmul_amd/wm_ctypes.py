@@ -153,10 +153,10 @@ def attention_forward(q, k, v, w, scale=1.0, mask=False, flags=0, want_lse=True)
     return o, lse
 
 
-def attention_backward(q, k, v, o, lse, go, w, scale=1.0, flags=0):
-    """Gradients (gq, gk, gv), all (B,M,N) row-major, from the forward's o and lse."""
+def attention_backward(q, k, v, o, lse, go, w, scale=1.0, flags=0, want=(True, True, True)):
+    """Gradients (gq, gk, gv), all (B,M,N) row-major, from the forward's o and lse; None where not wanted."""
     B, M, N = q.shape
-    gq, gk, gv = (torch.empty(B, M, N, dtype=q.dtype, device=q.device) for _ in range(3))
+    gq, gk, gv = (torch.empty(B, M, N, dtype=q.dtype, device=q.device) if x else None for x in want)
     delta = torch.empty(B, M, dtype=torch.float32, device=q.device)
     _check(lib().wm_window_attention_backward(op(q), op(k), op(v), op(o), ctypes.c_void_p(lse.data_ptr()), op(go),
                                              op(gq), op(gk), op(gv), ctypes.c_void_p(delta.data_ptr()), B, M, N, w,

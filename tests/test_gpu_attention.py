@@ -185,3 +185,27 @@ def test_long_sequence_wide_head_against_separate_ops(device):
     for x, y in zip(res["fused"], res["chain"]):
         torch.testing.assert_close(x.float(), y.float(), **TOL)
         assert torch.isfinite(x).all()
+
+
+@pytest.mark.parametrize("want", [(True, False, False), (False, True, True), (False, False, True), (True, True, False)],
+                         ids=lambda t: "".join("qkv"[i] for i in range(3) if t[i]))
+def test_backward_of_some_inputs_only(device, want):
+    """Gradients that are not asked for are skipped and the others do not change by a bit."""
+    from window_matmul import window_attention
+
+    B, M, N, w = 3, 300, 64, 40
+    q, k, v, go = (seeded((B, M, N), s, torch.bfloat16).to(device) for s in (95, 96, 97, 98))
+    o, lse = abi.attention_forward(q, k, v, w, 0.125)
+    full = abi.attention_backward(q, k, v, o, lse, go, w, 0.125)
+    part = abi.attention_backward(q, k, v, o, lse, go, w, 0.125, want=want)
+    for wanted, x, y in zip(want, part, full):
+        assert (x is None) == (not wanted)
+        if wanted:
+            assert torch.equal(x, y)
+    # through autograd: inputs that do not require a gradient get none
+    qq, kk, vv = (t.clone().requires_grad_(r) for t, r in zip((q, k, v), want))
+    window_attention(qq, kk, vv, w, 0.125).backward(go)
+    for wanted, t, y in zip(want, (qq, kk, vv), full):
+        assert (t.grad is None) == (not wanted)
+        if wanted:
+            assert torch.equal(t.grad, y)
