@@ -146,7 +146,7 @@ const char *wm_band_softmax_kernel_choice(int64_t w, int dtype, int contiguous, 
  * window op takes).  lse, if not NULL, receives the natural-log sum of exponentials of every
  * row as float32 (B * M values, contiguous) for use by a backward pass.
  * Returns WM_ERR_UNSUPPORTED, having launched nothing, unless dtype is float16 / bfloat16,
- * N is a multiple of 32 up to 128, w >= 1, scale > 0 and all four operands have unit column
+ * N is a multiple of 16 up to 128, w >= 1, scale > 0 and all four operands have unit column
  * stride and 16-byte aligned rows (see wm_window_attention_supported). */
 int wm_window_attention_forward(const wm_operand *q, const wm_operand *k, const wm_operand *v,
                                 const wm_operand *o, float *lse, int64_t B, int64_t M, int64_t N,

@@ -61,15 +61,16 @@ __device__ __forceinline__ float across_halves_sum(float v) {
   return __uint_as_float(r[0]) + __uint_as_float(r[1]);
 }
 
-template <typename T, int NB, bool MASK>
-__global__ __launch_bounds__(kThreads, NB <= 2 ? 4 : 2) void attention_forward_kernel(
+template <typename T, int NK, bool MASK>  // N = 16 NK
+__global__ __launch_bounds__(kThreads, NK <= 4 ? 4 : 2) void attention_forward_kernel(
     const uint16_t *__restrict__ Q, const uint16_t *__restrict__ K, const uint16_t *__restrict__ V,
     uint16_t *__restrict__ O, float *__restrict__ L, int B, int M, int w, int nblk, float c, int64_t qsb, int64_t qsr,
     int64_t ksb, int64_t ksr, int64_t vsb, int64_t vsr, int64_t osb, int64_t osr) {
-  constexpr int N = 32 * NB, NK = N / 16;
-  constexpr int KS = N + 8;   // key rows 16 (mod 128) bytes apart in banks: conflict-free b128 reads
-  constexpr int VS = N + 16;  // value rows 32 (mod 128) bytes apart: what the transposed reads want
-  constexpr int SLOTS = AT_KC * N / 8 / kThreads;  // 16-byte pieces per thread, chunk and tensor
+  constexpr int N = 16 * NK, NB = (NK + 1) / 2;  // NB blocks of 32 output columns; the last may be half used
+  constexpr int KS = N + 8;         // key rows 16 (mod 128) bytes apart in banks: conflict-free b128 reads
+  constexpr int VS = 32 * NB + 16;  // value rows 32 or 96 (mod 128) bytes apart: what the transposed reads want
+  constexpr int PIECES = AT_KC * N / 8;                       // 16-byte pieces of a chunk, per tensor
+  constexpr int SLOTS = (PIECES + kThreads - 1) / kThreads;   // pieces per thread (the last slot may be idle)
   __shared__ __attribute__((aligned(16))) uint16_t k_lds[2][AT_KC * KS];
   __shared__ __attribute__((aligned(16))) uint16_t v_lds[2][AT_KC * VS];
 
@@ -97,7 +98,7 @@ __global__ __launch_bounds__(kThreads, NB <= 2 ? 4 : 2) void attention_forward_k
   int l_row[SLOTS], l_col[SLOTS];
 #pragma unroll
   for (int u = 0; u < SLOTS; ++u) {
-    const int p = tid + kThreads * u;
+    const int p = min(tid + kThreads * u, PIECES - 1);  // an idle slot repeats the last piece
     l_row[u] = p / (N / 8);
     l_col[u] = (p % (N / 8)) * 8;
   }
@@ -233,12 +234,12 @@ __global__ __launch_bounds__(kThreads, NB <= 2 ? 4 : 2) void attention_forward_k
     for (int g = 0; g < 4; ++g) {
       const u32x2 out = {Mma<T>::pack2(o[hb][4 * g] * inv, o[hb][4 * g + 1] * inv),
                          Mma<T>::pack2(o[hb][4 * g + 2] * inv, o[hb][4 * g + 3] * inv)};
-      *reinterpret_cast<u32x2 *>(orow + 32 * hb + 8 * g) = out;
+      if (32 * hb + 8 * g + 4 * half < N) *reinterpret_cast<u32x2 *>(orow + 32 * hb + 8 * g) = out;
     }
   if (L != nullptr && half == 0) L[(int64_t)b * M + qi] = (m_used + __builtin_amdgcn_logf(l)) * kLn2F;
 }
 
-template <typename T, int NB>
+template <typename T, int NK>
 hipError_t launch_forward(const Problem &p, const View &q, const View &k, const View &v, const View &o, float *lse,
                           double scale, int mask) {
   const int nblk = (int)((p.M + AT_TM - 1) / AT_TM);
@@ -247,7 +248,7 @@ hipError_t launch_forward(const Problem &p, const View &q, const View &k, const 
   const dim3 grid((unsigned)(groups * 8 * nblk)), block(kThreads);
   const float c = (float)(scale * 1.4426950408889634);
 #define WM_AT(MASKED)                                                                                                 \
-  hipLaunchKernelGGL((attention_forward_kernel<T, NB, MASKED>), grid, block, 0, p.stream, (const uint16_t *)q.data,   \
+  hipLaunchKernelGGL((attention_forward_kernel<T, NK, MASKED>), grid, block, 0, p.stream, (const uint16_t *)q.data,   \
                      (const uint16_t *)k.data, (const uint16_t *)v.data, (uint16_t *)o.data, lse, (int)p.B, (int)p.M, \
                      (int)p.w, nblk, c, q.sb, q.sr, k.sb, k.sr, v.sb, v.sr, o.sb, o.sr)
   if (mask)
@@ -261,11 +262,15 @@ hipError_t launch_forward(const Problem &p, const View &q, const View &k, const 
 template <typename T>
 hipError_t forward_by_width(const Problem &p, const View &q, const View &k, const View &v, const View &o, float *lse,
                             double scale, int mask) {
-  switch (p.N / 32) {
+  switch (p.N / 16) {
     case 1: return launch_forward<T, 1>(p, q, k, v, o, lse, scale, mask);
     case 2: return launch_forward<T, 2>(p, q, k, v, o, lse, scale, mask);
     case 3: return launch_forward<T, 3>(p, q, k, v, o, lse, scale, mask);
-    default: return launch_forward<T, 4>(p, q, k, v, o, lse, scale, mask);
+    case 4: return launch_forward<T, 4>(p, q, k, v, o, lse, scale, mask);
+    case 5: return launch_forward<T, 5>(p, q, k, v, o, lse, scale, mask);
+    case 6: return launch_forward<T, 6>(p, q, k, v, o, lse, scale, mask);
+    case 7: return launch_forward<T, 7>(p, q, k, v, o, lse, scale, mask);
+    default: return launch_forward<T, 8>(p, q, k, v, o, lse, scale, mask);
   }
 }
 
@@ -273,7 +278,7 @@ hipError_t forward_by_width(const Problem &p, const View &q, const View &k, cons
 
 bool attention_supports(int64_t M, int64_t N, int64_t w, int dtype, double scale) {
   if (dtype != WM_DTYPE_BF16 && dtype != WM_DTYPE_F16) return false;
-  if (N % 32 != 0 || N < 32 || N > 128) return false;
+  if (N % 16 != 0 || N < 16 || N > 128) return false;
   if (M < 1 || w < 1 || w > 0x3fffffff) return false;
   if (M > 0x7fffffff - w - 2 * AT_TM) return false;  // row and key indices are 32-bit in the kernels
   return scale > 0.0 && scale < 1.0e30;

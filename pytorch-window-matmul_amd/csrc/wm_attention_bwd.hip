@@ -71,32 +71,33 @@ __device__ __forceinline__ u32x4 pack8(const float *x) {
 }
 
 // Stores a 32-row accumulator block set, transposed layout (lane = row lane % 32, accumulator v =
-// column 32 hb + 8 (v / 4) + 4 half + v % 4), as 16-bit rows.
+// column 32 hb + 8 (v / 4) + 4 half + v % 4), as 16-bit rows of N columns (the last block may be half used).
 template <typename T, int NB>
-__device__ __forceinline__ void store_rows(uint16_t *row, const f32x16 (&acc)[NB], int half) {
+__device__ __forceinline__ void store_rows(uint16_t *row, const f32x16 (&acc)[NB], int half, int N) {
 #pragma unroll
   for (int hb = 0; hb < NB; ++hb)
 #pragma unroll
     for (int g = 0; g < 4; ++g) {
       const u32x2 out = {Mma<T>::pack2(acc[hb][4 * g], acc[hb][4 * g + 1]),
                          Mma<T>::pack2(acc[hb][4 * g + 2], acc[hb][4 * g + 3])};
-      *reinterpret_cast<u32x2 *>(row + 32 * hb + 8 * g + 4 * half) = out;
+      if (32 * hb + 8 * g + 4 * half < N) *reinterpret_cast<u32x2 *>(row + 32 * hb + 8 * g + 4 * half) = out;
     }
 }
 
 // ---------------------------------------------------------------------------------------------
 // query kernel: dQ and D
 // ---------------------------------------------------------------------------------------------
-template <typename T, int NB, bool WITH_DQ>  // WITH_DQ false: only D is wanted (grad_q not requested)
-__global__ __launch_bounds__(kThreads, NB <= 2 ? 2 : 1) void attention_backward_query_kernel(
+template <typename T, int NK, bool WITH_DQ>  // N = 16 NK; WITH_DQ false: only D is wanted (grad_q not requested)
+__global__ __launch_bounds__(kThreads, NK <= 4 ? 2 : 1) void attention_backward_query_kernel(
     const uint16_t *__restrict__ Q, const uint16_t *__restrict__ K, const uint16_t *__restrict__ V,
     const uint16_t *__restrict__ O, const uint16_t *__restrict__ dO, const float *__restrict__ L,
     uint16_t *__restrict__ dQ, float *__restrict__ D, int B, int M, int w, int nblk, float scale, int64_t qsb,
     int64_t qsr, int64_t ksb, int64_t ksr, int64_t vsb, int64_t vsr, int64_t osb, int64_t osr, int64_t gsb, int64_t gsr,
     int64_t dqsb, int64_t dqsr) {
-  constexpr int N = 32 * NB, NK = N / 16;
-  constexpr int TS = N + 16;  // tile rows 32 (mod 128) bytes apart: good for row reads and transposed reads
-  constexpr int SLOTS = AB_KC * N / 8 / kThreads;
+  constexpr int N = 16 * NK, NB = (NK + 1) / 2;
+  constexpr int TS = 32 * NB + 16;  // tile rows 32 or 96 (mod 128) bytes apart: row reads and transposed reads
+  constexpr int PIECES = AB_KC * N / 8;
+  constexpr int SLOTS = (PIECES + kThreads - 1) / kThreads;  // the last slot may be idle
   __shared__ __attribute__((aligned(16))) uint16_t k_lds[2][AB_KC * TS];
   __shared__ __attribute__((aligned(16))) uint16_t v_lds[2][AB_KC * TS];
 
@@ -136,7 +137,7 @@ __global__ __launch_bounds__(kThreads, NB <= 2 ? 2 : 1) void attention_backward_
   int l_row[SLOTS], l_col[SLOTS];
 #pragma unroll
   for (int u = 0; u < SLOTS; ++u) {
-    const int p = tid + kThreads * u;
+    const int p = min(tid + kThreads * u, PIECES - 1);  // an idle slot repeats the last piece
     l_row[u] = p / (N / 8);
     l_col[u] = (p % (N / 8)) * 8;
   }
@@ -223,22 +224,23 @@ __global__ __launch_bounds__(kThreads, NB <= 2 ? 2 : 1) void attention_backward_
     stash(buf ^ 1);
     __syncthreads();
   }
-  if (q_ok) store_rows<T, NB>(dQ + (int64_t)b * dqsb + (int64_t)qi * dqsr, dq, half);
+  if (q_ok) store_rows<T, NB>(dQ + (int64_t)b * dqsb + (int64_t)qi * dqsr, dq, half, N);
 }
 
 // ---------------------------------------------------------------------------------------------
 // key kernel: dK and dV
 // ---------------------------------------------------------------------------------------------
-template <typename T, int NB>
-__global__ __launch_bounds__(kThreads, NB <= 2 ? 2 : 1) void attention_backward_key_kernel(
+template <typename T, int NK>  // N = 16 NK
+__global__ __launch_bounds__(kThreads, NK <= 4 ? 2 : 1) void attention_backward_key_kernel(
     const uint16_t *__restrict__ Q, const uint16_t *__restrict__ K, const uint16_t *__restrict__ V,
     const uint16_t *__restrict__ dO, const float *__restrict__ L, const float *__restrict__ D,
     uint16_t *__restrict__ dK, uint16_t *__restrict__ dV, int B, int M, int w, int nblk, float scale, int64_t qsb,
     int64_t qsr, int64_t ksb, int64_t ksr, int64_t vsb, int64_t vsr, int64_t gsb, int64_t gsr, int64_t dksb,
     int64_t dksr, int64_t dvsb, int64_t dvsr) {
-  constexpr int N = 32 * NB, NK = N / 16;
-  constexpr int TS = N + 16;
-  constexpr int SLOTS = AB_KC * N / 8 / kThreads;
+  constexpr int N = 16 * NK, NB = (NK + 1) / 2;
+  constexpr int TS = 32 * NB + 16;
+  constexpr int PIECES = AB_KC * N / 8;
+  constexpr int SLOTS = (PIECES + kThreads - 1) / kThreads;
   __shared__ __attribute__((aligned(16))) uint16_t q_lds[2][AB_KC * TS];
   __shared__ __attribute__((aligned(16))) uint16_t g_lds[2][AB_KC * TS];
   __shared__ __attribute__((aligned(16))) float l_lds[2][AB_KC];  // L * log2(e) of the chunk's queries
@@ -273,7 +275,7 @@ __global__ __launch_bounds__(kThreads, NB <= 2 ? 2 : 1) void attention_backward_
   int l_row[SLOTS], l_col[SLOTS];
 #pragma unroll
   for (int u = 0; u < SLOTS; ++u) {
-    const int p = tid + kThreads * u;
+    const int p = min(tid + kThreads * u, PIECES - 1);  // an idle slot repeats the last piece
     l_row[u] = p / (N / 8);
     l_col[u] = (p % (N / 8)) * 8;
   }
@@ -373,12 +375,12 @@ __global__ __launch_bounds__(kThreads, NB <= 2 ? 2 : 1) void attention_backward_
     __syncthreads();
   }
   if (k_ok) {  // either output may be absent (gradient not requested)
-    if (dK != nullptr) store_rows<T, NB>(dK + (int64_t)b * dksb + (int64_t)kj * dksr, dk, half);
-    if (dV != nullptr) store_rows<T, NB>(dV + (int64_t)b * dvsb + (int64_t)kj * dvsr, dv, half);
+    if (dK != nullptr) store_rows<T, NB>(dK + (int64_t)b * dksb + (int64_t)kj * dksr, dk, half, N);
+    if (dV != nullptr) store_rows<T, NB>(dV + (int64_t)b * dvsb + (int64_t)kj * dvsr, dv, half, N);
   }
 }
 
-template <typename T, int NB>
+template <typename T, int NK>
 hipError_t launch_backward(const Problem &p, const View &q, const View &k, const View &v, const View &o,
                            const View &go, const float *lse, float *delta, const View &gq, const View &gk,
                            const View &gv, double scale) {
@@ -389,7 +391,7 @@ hipError_t launch_backward(const Problem &p, const View &q, const View &k, const
   typedef const uint16_t *in_t;
   typedef uint16_t *out_t;
 #define WM_ABQ(WITH_DQ)                                                                                              \
-  hipLaunchKernelGGL((attention_backward_query_kernel<T, NB, WITH_DQ>), grid, block, 0, p.stream, (in_t)q.data,      \
+  hipLaunchKernelGGL((attention_backward_query_kernel<T, NK, WITH_DQ>), grid, block, 0, p.stream, (in_t)q.data,      \
                      (in_t)k.data, (in_t)v.data, (in_t)o.data, (in_t)go.data, lse, (out_t)gq.data, delta, (int)p.B,  \
                      (int)p.M, (int)p.w, nblk, (float)scale, q.sb, q.sr, k.sb, k.sr, v.sb, v.sr, o.sb, o.sr, go.sb,  \
                      go.sr, gq.sb, gq.sr)
@@ -402,7 +404,7 @@ hipError_t launch_backward(const Problem &p, const View &q, const View &k, const
   hipError_t err = hipGetLastError();
   if (err != hipSuccess) return err;
   if (gk.data == nullptr && gv.data == nullptr) return hipSuccess;
-  hipLaunchKernelGGL((attention_backward_key_kernel<T, NB>), grid, block, 0, p.stream, (in_t)q.data, (in_t)k.data,
+  hipLaunchKernelGGL((attention_backward_key_kernel<T, NK>), grid, block, 0, p.stream, (in_t)q.data, (in_t)k.data,
                      (in_t)v.data, (in_t)go.data, lse, (const float *)delta, (out_t)gk.data, (out_t)gv.data, (int)p.B,
                      (int)p.M, (int)p.w, nblk, (float)scale, q.sb, q.sr, k.sb, k.sr, v.sb, v.sr, go.sb, go.sr, gk.sb,
                      gk.sr, gv.sb, gv.sr);
@@ -413,11 +415,15 @@ template <typename T>
 hipError_t backward_by_width(const Problem &p, const View &q, const View &k, const View &v, const View &o,
                              const View &go, const float *lse, float *delta, const View &gq, const View &gk,
                              const View &gv, double scale) {
-  switch (p.N / 32) {
+  switch (p.N / 16) {
     case 1: return launch_backward<T, 1>(p, q, k, v, o, go, lse, delta, gq, gk, gv, scale);
     case 2: return launch_backward<T, 2>(p, q, k, v, o, go, lse, delta, gq, gk, gv, scale);
     case 3: return launch_backward<T, 3>(p, q, k, v, o, go, lse, delta, gq, gk, gv, scale);
-    default: return launch_backward<T, 4>(p, q, k, v, o, go, lse, delta, gq, gk, gv, scale);
+    case 4: return launch_backward<T, 4>(p, q, k, v, o, go, lse, delta, gq, gk, gv, scale);
+    case 5: return launch_backward<T, 5>(p, q, k, v, o, go, lse, delta, gq, gk, gv, scale);
+    case 6: return launch_backward<T, 6>(p, q, k, v, o, go, lse, delta, gq, gk, gv, scale);
+    case 7: return launch_backward<T, 7>(p, q, k, v, o, go, lse, delta, gq, gk, gv, scale);
+    default: return launch_backward<T, 8>(p, q, k, v, o, go, lse, delta, gq, gk, gv, scale);
   }
 }
 

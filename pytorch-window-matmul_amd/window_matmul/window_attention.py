@@ -3,7 +3,7 @@
 The reference package stops at the two banded matmuls; its callers write the chain above
 themselves (reference tests/test_attention.py:57-63).  This function is that chain with the
 same semantics, as an addition next to the unchanged two-function API.  For float16 /
-bfloat16 inputs whose last dimension is a multiple of 32 up to 128 it runs fused kernels that
+bfloat16 inputs whose last dimension is a multiple of 16 up to 128 it runs fused kernels that
 never write the ``(…, M, 2w+1)`` band to memory (forward keeps only the log-sum-exp of every
 row, backward recomputes the probabilities); everything else runs the chain of the separate
 ops of this package, on the GPU as well.
