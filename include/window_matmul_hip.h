@@ -144,7 +144,8 @@ const char *wm_band_softmax_kernel_choice(int64_t w, int dtype, int contiguous, 
  * contribute no value row; with mask_out_of_range != 0 they are left out.
  * q, k, v, o are (B, M, N) operands (k holds key ROWS here, unlike the (B, N, M) view the
  * window op takes).  lse, if not NULL, receives the natural-log sum of exponentials of every
- * row as float32 (B * M values, contiguous) for use by a backward pass.
+ * row as float32 (B * M values, contiguous) for use by a backward pass; the sum is taken over
+ * the probabilities as rounded to the storage type, the values that multiply v.
  * Returns WM_ERR_UNSUPPORTED, having launched nothing, unless dtype is float16 / bfloat16,
  * N is a multiple of 16 up to 128, w >= 1, scale > 0 and all four operands have unit column
  * stride and 16-byte aligned rows (see wm_window_attention_supported). */
