@@ -239,6 +239,151 @@ __global__ __launch_bounds__(kThreads, NK <= 4 ? 4 : 2) void attention_forward_k
   if (L != nullptr && half == 0) L[(int64_t)b * M + qi] = (m_used + __builtin_amdgcn_logf(l)) * kLn2F;
 }
 
+// ---------------------------------------------------------------------------------------------
+// Narrow windows (w <= 16 (NKB - 1)): one pass, no key loop
+// ---------------------------------------------------------------------------------------------
+// A wavefront's 32 queries reach at most 32 NKB keys, so all of S^T (NKB tiles) sits in registers
+// at once and the softmax is the plain two-pass one.  Queries go straight from memory into MFMA
+// operand registers; the key and value rows of the workgroup are fetched as coalesced 16-byte
+// pieces, every load in flight before the first use, and pass through one LDS region in turn
+// (keys for S^T, then values for the second product, then the output rows, which leave as whole
+// non-temporal lines).  What bounds this kernel is HBM: it reads q, k, v and writes o, nothing else.
+template <typename T, int NK, int NKB, bool MASK>
+__global__ __launch_bounds__(kThreads, 2) void attention_forward_narrow_kernel(
+    const uint16_t *__restrict__ Q, const uint16_t *__restrict__ K, const uint16_t *__restrict__ V,
+    uint16_t *__restrict__ O, float *__restrict__ L, int B, int M, int w, int nblk, float c, int64_t qsb, int64_t qsr,
+    int64_t ksb, int64_t ksr, int64_t vsb, int64_t vsr, int64_t osb, int64_t osr) {
+  constexpr int N = 16 * NK, NB = (NK + 1) / 2;
+  constexpr int PADW = 16 * (NKB - 1);         // keys staged before the first and after the last query
+  constexpr int ROWS = AT_TM + 2 * PADW;       // key / value rows of the workgroup
+  constexpr int KS = N + 8;                    // key tile: plain b128 operand reads
+  constexpr int VS = 32 * NB + 16;             // value tile: transposed reads
+  constexpr int PIECES = ROWS * N / 8, SLOTS = (PIECES + kThreads - 1) / kThreads;
+  // one LDS region, used three times: key tile, then value tile, then output staging
+  __shared__ __attribute__((aligned(16))) uint16_t tile[ROWS * VS];
+  static_assert(KS <= VS, "the key tile must fit the region of the value tile");
+
+  int b, blk;
+  if (!decode_block(nblk, B, &b, &blk)) return;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, half = lane >> 5;
+  const int i0 = blk * AT_TM;
+  const int qw0 = i0 + 32 * wave, qi = qw0 + (lane & 31);
+  const int kw0 = qw0 - PADW;  // first key of this wavefront's tiles
+
+  // every load of the workgroup is issued before the first use: queries in operand layout, key and
+  // value rows as coalesced 16-byte pieces (rows outside the sequence read a safe address, zeroed later)
+  u32x4 qf[NK], kreg[SLOTS], vreg[SLOTS];
+  {
+    const uint16_t *qr = Q + (int64_t)b * qsb + (int64_t)qi * qsr + 8 * half;
+#pragma unroll
+    for (int ks = 0; ks < NK; ++ks) qf[ks] = fetch_row_chunk(qr + 16 * ks, Q, qi < M);
+    const uint16_t *Kb = K + (int64_t)b * ksb, *Vb = V + (int64_t)b * vsb;
+#pragma unroll
+    for (int u = 0; u < SLOTS; ++u) {
+      const int p = min(tid + kThreads * u, PIECES - 1);
+      const int key = i0 - PADW + p / (N / 8), col = (p % (N / 8)) * 8;
+      const bool ok = (key >= 0) & (key < M);
+      kreg[u] = fetch_row_chunk(Kb + (int64_t)key * ksr + col, K, ok);
+      vreg[u] = fetch_row_chunk(Vb + (int64_t)key * vsr + col, V, ok);
+    }
+#pragma unroll
+    for (int ks = 0; ks < NK; ++ks) qf[ks] = mask_row_chunk(qf[ks], qi < M);
+#pragma unroll
+    for (int u = 0; u < SLOTS; ++u) {
+      const int p = min(tid + kThreads * u, PIECES - 1);
+      const int row = p / (N / 8), key = i0 - PADW + row;
+      *reinterpret_cast<u32x4 *>(&tile[row * KS + (p % (N / 8)) * 8]) = mask_row_chunk(kreg[u], (key >= 0) & (key < M));
+    }
+  }
+  __syncthreads();
+
+  // S^T tiles: accumulator v of tile j: key kw0 + 32 j + 8 (v / 4) + 4 half + v % 4, query qi
+  const float ninf = -__builtin_huge_valf();
+  f32x16 s[NKB];
+  float top = ninf;
+#pragma unroll
+  for (int j = 0; j < NKB; ++j) {
+#pragma unroll
+    for (int v = 0; v < 16; ++v) s[j][v] = 0.0f;
+    const uint16_t *krow = &tile[(32 * wave + 32 * j + (lane & 31)) * KS + 8 * half];
+#pragma unroll
+    for (int ks = 0; ks < NK; ++ks) s[j] = Mma<T>::run(*reinterpret_cast<const u32x4 *>(krow + 16 * ks), qf[ks], s[j]);
+    // valid key offsets of this lane in tile j: first..last (band and sequence), as in the wide kernel
+    const int k0 = kw0 + 32 * j + 4 * half;  // key at offset 0
+    const int first = max(qi - w, 0) - k0, last = min(qi + w, M - 1) - k0;
+    const int origin = last < first ? 0x100000 : first;
+    const unsigned span = last < first ? 0u : (unsigned)(last - first);
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+      const int ofs = 8 * (v / 4) + v % 4;
+      s[j][v] = (unsigned)(ofs - origin) <= span ? s[j][v] : ninf;
+      top = fmaxf(top, s[j][v]);
+    }
+  }
+  __syncthreads();  // the key tile has been read by everyone: the value tile takes its place
+#pragma unroll
+  for (int u = 0; u < SLOTS; ++u) {
+    const int p = min(tid + kThreads * u, PIECES - 1);
+    const int row = p / (N / 8), key = i0 - PADW + row;
+    *reinterpret_cast<u32x4 *>(&tile[row * VS + (p % (N / 8)) * 8]) = mask_row_chunk(vreg[u], (key >= 0) & (key < M));
+  }
+  __syncthreads();
+  top = across_halves_max(top) * c;  // log2 units
+  const int n_out = MASK ? 0 : max(0, w - qi) + max(0, qi + w - (M - 1));  // zero-score entries outside the sequence
+  if (n_out > 0) top = fmaxf(top, 0.0f);
+  if (qi >= M) top = 0.0f;  // rows past the end: keep the arithmetic finite, nothing is stored
+  float l_part = 0.0f;
+  f32x16 o[NB];
+#pragma unroll
+  for (int hb = 0; hb < NB; ++hb)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) o[hb][v] = 0.0f;
+#pragma unroll
+  for (int j = 0; j < NKB; ++j) {
+    float p[16];
+#pragma unroll
+    for (int v = 0; v < 16; ++v) p[v] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[j][v], c, -top));
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      const u32x4 pf = {Mma<T>::pack2(p[8 * t + 0], p[8 * t + 1]), Mma<T>::pack2(p[8 * t + 2], p[8 * t + 3]),
+                        Mma<T>::pack2(p[8 * t + 4], p[8 * t + 5]), Mma<T>::pack2(p[8 * t + 6], p[8 * t + 7])};
+#pragma unroll
+      for (int d = 0; d < 4; ++d) l_part = Mma<T>::add_pair(pf[d], l_part);
+#pragma unroll
+      for (int hb = 0; hb < NB; ++hb) {
+        const u32x4 vf = lds_read_transposed_split(tile, VS, 32 * wave + 32 * j + 16 * t, 32 * hb, lane);
+        o[hb] = Mma<T>::run(vf, pf, o[hb]);
+      }
+    }
+  }
+  float l = across_halves_sum(l_part);
+  if (n_out > 0) l += (float)n_out * __builtin_amdgcn_exp2f(-top);
+  const float inv = 1.0f / l;
+  if (L != nullptr && half == 0 && qi < M) L[(int64_t)b * M + qi] = (top + __builtin_amdgcn_logf(l)) * kLn2F;
+  // The result leaves through LDS (the value tile is no longer needed) as row-contiguous,
+  // non-temporal 16-byte stores: whole 128-byte lines instead of 8 bytes per lane over 32 rows.
+  __syncthreads();
+  constexpr int SO = 32 * NB + 8;
+  static_assert(4 * 32 * SO <= ROWS * VS, "output staging must fit the value tile");
+  uint16_t *stage = tile + wave * (32 * SO);
+#pragma unroll
+  for (int hb = 0; hb < NB; ++hb)
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      const u32x2 out = {Mma<T>::pack2(o[hb][4 * g] * inv, o[hb][4 * g + 1] * inv),
+                         Mma<T>::pack2(o[hb][4 * g + 2] * inv, o[hb][4 * g + 3] * inv)};
+      *reinterpret_cast<u32x2 *>(stage + (lane & 31) * SO + 32 * hb + 8 * g + 4 * half) = out;
+    }
+  wave_sync_lds();
+  constexpr int PER_ROW = N / 8;
+  for (int p = lane; p < 32 * PER_ROW; p += 64) {
+    const int r = p / PER_ROW, hg = p - r * PER_ROW;
+    if (qw0 + r < M)
+      store_chunk_streaming(O + (int64_t)b * osb + (int64_t)(qw0 + r) * osr + 8 * hg,
+                            *reinterpret_cast<const u32x4 *>(stage + r * SO + 8 * hg));
+  }
+}
+
 template <typename T, int NK>
 hipError_t launch_forward(const Problem &p, const View &q, const View &k, const View &v, const View &o, float *lse,
                           double scale, int mask) {
@@ -247,14 +392,27 @@ hipError_t launch_forward(const Problem &p, const View &q, const View &k, const 
   if (groups * 8 * nblk > 0x7fffffff) return hipErrorInvalidValue;
   const dim3 grid((unsigned)(groups * 8 * nblk)), block(kThreads);
   const float c = (float)(scale * 1.4426950408889634);
-#define WM_AT(MASKED)                                                                                                 \
-  hipLaunchKernelGGL((attention_forward_kernel<T, NK, MASKED>), grid, block, 0, p.stream, (const uint16_t *)q.data,   \
-                     (const uint16_t *)k.data, (const uint16_t *)v.data, (uint16_t *)o.data, lse, (int)p.B, (int)p.M, \
-                     (int)p.w, nblk, c, q.sb, q.sr, k.sb, k.sr, v.sb, v.sr, o.sb, o.sr)
-  if (mask)
-    WM_AT(true);
-  else
-    WM_AT(false);
+#define WM_AT(KERNEL)                                                                                              \
+  hipLaunchKernelGGL(KERNEL, grid, block, 0, p.stream, (const uint16_t *)q.data, (const uint16_t *)k.data,         \
+                     (const uint16_t *)v.data, (uint16_t *)o.data, lse, (int)p.B, (int)p.M, (int)p.w, nblk, c,     \
+                     q.sb, q.sr, k.sb, k.sr, v.sb, v.sr, o.sb, o.sr)
+  // narrow windows take the one-pass kernel (two key tiles per wavefront up to w = 16, three up to 32)
+  if (p.w <= 16 && !(p.flags & WM_FLAG_NO_NARROW_BAND)) {
+    if (mask)
+      WM_AT((attention_forward_narrow_kernel<T, NK, 2, true>));
+    else
+      WM_AT((attention_forward_narrow_kernel<T, NK, 2, false>));
+  } else if (p.w <= 32 && NK <= 4 && !(p.flags & WM_FLAG_NO_NARROW_BAND)) {
+    if (mask)
+      WM_AT((attention_forward_narrow_kernel<T, NK, 3, true>));
+    else
+      WM_AT((attention_forward_narrow_kernel<T, NK, 3, false>));
+  } else {
+    if (mask)
+      WM_AT((attention_forward_kernel<T, NK, true>));
+    else
+      WM_AT((attention_forward_kernel<T, NK, false>));
+  }
 #undef WM_AT
   return hipGetLastError();
 }

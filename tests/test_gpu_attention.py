@@ -233,3 +233,16 @@ def test_ragged_shape_with_zero_query_rows(device, w):
     # a zero query row attends uniformly over its 2w+1 band entries (out-of-sequence ones included)
     uniform = torch.from_numpy(want_o)[:, zero_rows]
     torch.testing.assert_close(o[:, zero_rows].cpu().to(torch.float64), uniform, **TOL)
+
+
+@pytest.mark.parametrize("w", [3, 8, 16, 24, 32])
+def test_narrow_and_chunked_forward_agree(device, w):
+    """Windows up to 32 take the one-pass kernel; WM_FLAG_NO_NARROW_BAND forces the chunked one.  Both
+    must agree with each other to rounding (and each is checked against the oracle elsewhere)."""
+    B, M, N = 5, 700, 64
+    q, k, v = (seeded((B, M, N), s, torch.bfloat16).to(device) for s in (121, 122, 123))
+    for mask in (False, True):
+        o1, l1 = abi.attention_forward(q, k, v, w, 0.125, mask)
+        o2, l2 = abi.attention_forward(q, k, v, w, 0.125, mask, flags=abi.NO_NARROW_BAND)
+        torch.testing.assert_close(o1.float(), o2.float(), rtol=1e-2, atol=1e-2)
+        torch.testing.assert_close(l1, l2, rtol=5e-3, atol=5e-3)
