@@ -246,3 +246,32 @@ def test_narrow_and_chunked_forward_agree(device, w):
         o2, l2 = abi.attention_forward(q, k, v, w, 0.125, mask, flags=abi.NO_NARROW_BAND)
         torch.testing.assert_close(o1.float(), o2.float(), rtol=1e-2, atol=1e-2)
         torch.testing.assert_close(l1, l2, rtol=5e-3, atol=5e-3)
+
+
+def _graph_nodes(t):
+    seen, todo = set(), [t.grad_fn]
+    while todo:
+        fn = todo.pop()
+        if fn is None or fn in seen:
+            continue
+        seen.add(fn)
+        todo.extend(f for f, _ in fn.next_functions)
+    return {type(fn).__name__ for fn in seen}
+
+
+def test_narrow_window_training_goes_through_the_separate_ops(device):
+    """Same values either way; the choice only shows in which autograd nodes produced the result."""
+    from window_matmul import window_attention
+
+    q, k, v, go = (seeded((2, 200, 64), s, torch.bfloat16).to(device) for s in (131, 132, 133, 134))
+    with torch.no_grad():
+        want = window_attention(q, k, v, 8)          # fused one-pass forward
+    qq, kk, vv = (t.clone().requires_grad_(True) for t in (q, k, v))
+    out = window_attention(qq, kk, vv, 8)             # separate ops (w <= 12 and gradients wanted)
+    assert "UnwindowMatmulFuncBackward" in _graph_nodes(out)
+    torch.testing.assert_close(out.float(), want.float(), **TOL)
+    out.backward(go)
+    want_g = ao.window_attention_backward(q.cpu(), k.cpu(), v.cpu(), 8, go.cpu(), 1.0 / math.sqrt(64))
+    for x, y in zip((qq.grad, kk.grad, vv.grad), want_g):
+        close(x, y)
+    assert "WindowAttentionFuncBackward" in _graph_nodes(window_attention(qq, kk, vv, 16))  # wider: fused
