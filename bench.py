@@ -180,7 +180,8 @@ def main():
         return (torch.randn(B, M, N, generator=g) * scale).to(dtype).to(dev)
 
     q, k, v, go = synth(cfg["qk_scale"]), synth(cfg["qk_scale"]), synth(), synth()
-    q.requires_grad_(True), k.requires_grad_(True), v.requires_grad_(True)
+    if cfg["backward"]:  # forward-only workloads are inference: no autograd graph is recorded
+        q.requires_grad_(True), k.requires_grad_(True), v.requires_grad_(True)
 
     def step(softmax=lambda att: torch.softmax(att, dim=-1)):
         att = window_matmul(q, k.transpose(1, 2), w)
