@@ -137,7 +137,8 @@ __global__ __launch_bounds__(kThreads, NK <= 4 ? 2 : 1) void attention_backward_
   int l_row[SLOTS], l_col[SLOTS];
 #pragma unroll
   for (int u = 0; u < SLOTS; ++u) {
-    const int p = min(tid + kThreads * u, PIECES - 1);  // an idle slot repeats the last piece
+    // an idle slot repeats the last piece; widths that fill every slot keep the plain affine index
+    const int p = PIECES % kThreads == 0 ? tid + kThreads * u : min(tid + kThreads * u, PIECES - 1);
     l_row[u] = p / (N / 8);
     l_col[u] = (p % (N / 8)) * 8;
   }
@@ -275,7 +276,8 @@ __global__ __launch_bounds__(kThreads, NK <= 4 ? 2 : 1) void attention_backward_
   int l_row[SLOTS], l_col[SLOTS];
 #pragma unroll
   for (int u = 0; u < SLOTS; ++u) {
-    const int p = min(tid + kThreads * u, PIECES - 1);  // an idle slot repeats the last piece
+    // an idle slot repeats the last piece; widths that fill every slot keep the plain affine index
+    const int p = PIECES % kThreads == 0 ? tid + kThreads * u : min(tid + kThreads * u, PIECES - 1);
     l_row[u] = p / (N / 8);
     l_col[u] = (p % (N / 8)) * 8;
   }
