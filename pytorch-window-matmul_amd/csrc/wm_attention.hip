@@ -225,18 +225,12 @@ __global__ __launch_bounds__(kThreads, NK <= 4 ? 4 : 2) void attention_forward_k
       }
     }
   }
-  if (qi >= M) return;
+  if (qi >= M) l = 1.0f;  // rows past the end: keep the arithmetic finite, nothing is stored
   const float inv = 1.0f / l;
-  uint16_t *orow = O + (int64_t)b * osb + (int64_t)qi * osr + 4 * half;
-#pragma unroll
-  for (int hb = 0; hb < NB; ++hb)
-#pragma unroll
-    for (int g = 0; g < 4; ++g) {
-      const u32x2 out = {Mma<T>::pack2(o[hb][4 * g] * inv, o[hb][4 * g + 1] * inv),
-                         Mma<T>::pack2(o[hb][4 * g + 2] * inv, o[hb][4 * g + 3] * inv)};
-      if (32 * hb + 8 * g + 4 * half < N) *reinterpret_cast<u32x2 *>(orow + 32 * hb + 8 * g) = out;
-    }
-  if (L != nullptr && half == 0) L[(int64_t)b * M + qi] = (m_used + __builtin_amdgcn_logf(l)) * kLn2F;
+  if (L != nullptr && half == 0 && qi < M) L[(int64_t)b * M + qi] = (m_used + __builtin_amdgcn_logf(l)) * kLn2F;
+  // every wave is past the last barrier: the value buffers are free and stage the result rows
+  static_assert(4 * RowStage<NB>::ELEMS <= 2 * AT_KC * VS, "the four staging areas must fit the value buffers");
+  store_wave_rows<T, NB>(&v_lds[0][0] + wave * RowStage<NB>::ELEMS, o, inv, O + (int64_t)b * osb, osr, qw0, M, N, lane);
 }
 
 // ---------------------------------------------------------------------------------------------

@@ -70,25 +70,11 @@ __device__ __forceinline__ u32x4 pack8(const float *x) {
   return r;
 }
 
-// Stores a 32-row accumulator block set, transposed layout (lane = row lane % 32, accumulator v =
-// column 32 hb + 8 (v / 4) + 4 half + v % 4), as 16-bit rows of N columns (the last block may be half used).
-template <typename T, int NB>
-__device__ __forceinline__ void store_rows(uint16_t *row, const f32x16 (&acc)[NB], int half, int N) {
-#pragma unroll
-  for (int hb = 0; hb < NB; ++hb)
-#pragma unroll
-    for (int g = 0; g < 4; ++g) {
-      const u32x2 out = {Mma<T>::pack2(acc[hb][4 * g], acc[hb][4 * g + 1]),
-                         Mma<T>::pack2(acc[hb][4 * g + 2], acc[hb][4 * g + 3])};
-      if (32 * hb + 8 * g + 4 * half < N) *reinterpret_cast<u32x2 *>(row + 32 * hb + 8 * g + 4 * half) = out;
-    }
-}
-
 // ---------------------------------------------------------------------------------------------
 // query kernel: dQ and D
 // ---------------------------------------------------------------------------------------------
 template <typename T, int NK, bool WITH_DQ>  // N = 16 NK; WITH_DQ false: only D is wanted (grad_q not requested)
-__global__ __launch_bounds__(kThreads, NK <= 4 ? 2 : 1) void attention_backward_query_kernel(
+__global__ __launch_bounds__(kThreads, NK <= 4 ? 3 : 1) void attention_backward_query_kernel(
     const uint16_t *__restrict__ Q, const uint16_t *__restrict__ K, const uint16_t *__restrict__ V,
     const uint16_t *__restrict__ O, const uint16_t *__restrict__ dO, const float *__restrict__ L,
     uint16_t *__restrict__ dQ, float *__restrict__ D, int B, int M, int w, int nblk, float scale, int64_t qsb,
@@ -225,7 +211,10 @@ __global__ __launch_bounds__(kThreads, NK <= 4 ? 2 : 1) void attention_backward_
     stash(buf ^ 1);
     __syncthreads();
   }
-  if (q_ok) store_rows<T, NB>(dQ + (int64_t)b * dqsb + (int64_t)qi * dqsr, dq, half, N);
+  // every wave is past the last barrier: the key buffers are free and stage the result rows
+  static_assert(4 * RowStage<NB>::ELEMS <= 2 * AB_KC * TS, "the four staging areas must fit the key buffers");
+  store_wave_rows<T, NB>(&k_lds[0][0] + wave * RowStage<NB>::ELEMS, dq, 1.0f, dQ + (int64_t)b * dqsb, dqsr, qw0, M, N,
+                         lane);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -376,10 +365,12 @@ __global__ __launch_bounds__(kThreads, NK <= 4 ? 2 : 1) void attention_backward_
     stash(buf ^ 1);
     __syncthreads();
   }
-  if (k_ok) {  // either output may be absent (gradient not requested)
-    if (dK != nullptr) store_rows<T, NB>(dK + (int64_t)b * dksb + (int64_t)kj * dksr, dk, half, N);
-    if (dV != nullptr) store_rows<T, NB>(dV + (int64_t)b * dvsb + (int64_t)kj * dvsr, dv, half, N);
-  }
+  // every wave is past the last barrier: the query buffers are free and stage the result rows;
+  // either output may be absent (gradient not requested)
+  static_assert(4 * RowStage<NB>::ELEMS <= 2 * AB_KC * TS, "the four staging areas must fit the query buffers");
+  uint16_t *stage = &q_lds[0][0] + wave * RowStage<NB>::ELEMS;
+  if (dK != nullptr) store_wave_rows<T, NB>(stage, dk, 1.0f, dK + (int64_t)b * dksb, dksr, kw0, M, N, lane);
+  if (dV != nullptr) store_wave_rows<T, NB>(stage, dv, 1.0f, dV + (int64_t)b * dvsb, dvsr, kw0, M, N, lane);
 }
 
 template <typename T, int NK>

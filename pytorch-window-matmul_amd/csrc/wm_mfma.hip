@@ -180,22 +180,11 @@ __global__ __launch_bounds__(kThreads, NT <= 2 ? 3 : 2) void mfma_p2_kernel(cons
   }
   if (k < nk) slot(k, t_reg[0], y_reg[0], t_reg[1], y_reg[1]);
 
-  // acc[nt][v]: h = 32 nt + 8 (v / 4) + 4 (lane / 32) + v % 4, row = wave * 32 + lane % 32
-  const int i = i0 + wave * 32 + (lane & 31);
-  if (i < M) {
-    uint16_t *crow = C + (int64_t)b * csb + (int64_t)i * csr;
-#pragma unroll
-    for (int nt = 0; nt < NT; ++nt)
-#pragma unroll
-      for (int q4 = 0; q4 < 4; ++q4) {
-        const int h = 32 * nt + 8 * q4 + 4 * (lane >> 5);
-        if (h < N) {
-          u32x2 o = {Mma<T>::pack2(acc[nt][4 * q4], acc[nt][4 * q4 + 1]),
-                     Mma<T>::pack2(acc[nt][4 * q4 + 2], acc[nt][4 * q4 + 3])};
-          *reinterpret_cast<u32x2 *>(crow + h) = o;
-        }
-      }
-  }
+  // acc[nt][v]: h = 32 nt + 8 (v / 4) + 4 (lane / 32) + v % 4, row = wave * 32 + lane % 32; every
+  // wave is past the last barrier, so the tile buffers are free
+  static_assert(4 * RowStage<NT>::ELEMS <= 2 * TM * KC, "the four staging areas must fit the band tile buffers");
+  store_wave_rows<T, NT>(&t_lds[0][0] + wave * RowStage<NT>::ELEMS, acc, 1.0f, C + (int64_t)b * csb, csr,
+                         i0 + wave * 32, M, N, lane);
 }
 
 // ------------------------------------------------------------------------------------------
@@ -320,21 +309,9 @@ __global__ __launch_bounds__(kThreads, NT <= 2 ? 3 : 2) void mfma_p3_kernel(cons
   }
   if (k < nk) slot(k, t_reg[0], y_reg[0], t_reg[1], y_reg[1]);
 
-  const int c = c0 + wave * 32 + (lane & 31);
-  if (c >= 0 && c < M) {
-    uint16_t *crow = C + (int64_t)b * csb + (int64_t)c * csr;
-#pragma unroll
-    for (int nt = 0; nt < NT; ++nt)
-#pragma unroll
-      for (int q4 = 0; q4 < 4; ++q4) {
-        const int h = 32 * nt + 8 * q4 + 4 * (lane >> 5);
-        if (h < N) {
-          u32x2 o = {Mma<T>::pack2(acc[nt][4 * q4], acc[nt][4 * q4 + 1]),
-                     Mma<T>::pack2(acc[nt][4 * q4 + 2], acc[nt][4 * q4 + 3])};
-          *reinterpret_cast<u32x2 *>(crow + h) = o;
-        }
-      }
-  }
+  static_assert(4 * RowStage<NT>::ELEMS <= 2 * TM * KC, "the four staging areas must fit the band tile buffers");
+  store_wave_rows<T, NT>(&t_lds[0][0] + wave * RowStage<NT>::ELEMS, acc, 1.0f, C + (int64_t)b * csb, csr,
+                         c0 + wave * 32, M, N, lane);
 }
 
 // ------------------------------------------------------------------------------------------

@@ -175,6 +175,48 @@ __device__ __forceinline__ void wave_sync_lds() {
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
+// Result rows of a wave that holds 32 rows x 32 NB columns transposed: lane = row (lane % 32),
+// accumulator v of block hb = column 32 hb + 8 (v / 4) + 4 (lane / 32) + v % 4.  Stored from
+// there a row would leave as 8-byte pieces, sixteen per 128 bytes.  The rows go through a
+// wave-private LDS area instead (RowStage<NB>::ELEMS elements, e.g. part of the operand buffers
+// once the last chunk is multiplied) and leave as 16-byte pieces, consecutive lanes on
+// consecutive pieces of a row: whole 128-byte lines per 8 lanes, non-temporal so that they do
+// not displace streamed operands on their way through the caches.  `mul` scales the lane's row.
+template <int NB>
+struct RowStage {
+  static constexpr int SW = NB == 1 ? 32 : 64;  // columns staged at a time
+  static constexpr int STRIDE = SW + 8;         // staged rows 16 bytes apart mod 128 (SW = 64)
+  static constexpr int ELEMS = 32 * STRIDE;     // per wave
+};
+template <typename T, int NB>
+__device__ __forceinline__ void store_wave_rows(uint16_t *stage, const f32x16 (&acc)[NB], float mul, uint16_t *Cb,
+                                                int64_t csr, int row0, int M, int N, int lane) {
+  constexpr int SW = RowStage<NB>::SW, STRIDE = RowStage<NB>::STRIDE;
+  constexpr int CPR = SW / 8, RPP = 64 / CPR;  // 16-byte pieces per staged row, rows per 64-lane pass
+  const int r = lane & 31, half = lane >> 5;
+#pragma unroll
+  for (int n0 = 0; n0 < NB; n0 += SW / 32) {
+    wave_sync_lds();  // whatever the wave still reads from the area has been read
+#pragma unroll
+    for (int hb = n0; hb < n0 + SW / 32 && hb < NB; ++hb)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const u32x2 o = {Mma<T>::pack2(acc[hb][4 * g] * mul, acc[hb][4 * g + 1] * mul),
+                         Mma<T>::pack2(acc[hb][4 * g + 2] * mul, acc[hb][4 * g + 3] * mul)};
+        *reinterpret_cast<u32x2 *>(stage + r * STRIDE + 32 * (hb - n0) + 8 * g + 4 * half) = o;
+      }
+    wave_sync_lds();
+#pragma unroll
+    for (int s = 0; s < 32 / RPP; ++s) {
+      const int rr = lane / CPR + RPP * s, piece = lane % CPR;
+      const int row = row0 + rr, h = 32 * n0 + 8 * piece;
+      if (row >= 0 && row < M && h < N)
+        __builtin_nontemporal_store(*reinterpret_cast<const u32x4 *>(stage + rr * STRIDE + 8 * piece),
+                                    reinterpret_cast<u32x4 *>(Cb + (int64_t)row * csr + h));
+    }
+  }
+}
+
 // Workgroup -> (batch, block).  Workgroups are dealt round-robin to the 8 XCDs, each with
 // its own L2; all blocks of one batch element are given to one XCD so that neighbouring
 // blocks find the rows they share (the +-w halo) in that L2.
