@@ -19,7 +19,7 @@ the count but its time is inside the step).  Next to it:
                 restatement, one thread, on a slice of the batch.
 
 Usage: python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c2|c4] [--no-cpu]
-       python bench.py --kernels-only [--shape B M N w] [--dtype bf16|fp16] [--family auto|wide|strided]
+       python bench.py --kernels-only [--shape B M N w] [--dtype bf16|fp16|fp32] [--family auto|wide|strided]
 """
 import argparse
 import json
@@ -102,7 +102,7 @@ def cpu_baseline(cfg, seconds_budget=20.0):
     impl = ref if ref is not None else oracle
     M, N, w = cfg["M"], cfg["N"], cfg["w"]
     g = torch.Generator().manual_seed(0)
-    rnd = {"bf16": torch.bfloat16, "fp16": torch.float16}[cfg["dtype"]]
+    rnd = {"bf16": torch.bfloat16, "fp16": torch.float16, "fp32": torch.float32}[cfg["dtype"]]
 
     def rounded(*shape, scale=1.0):
         return (torch.randn(*shape, generator=g) * scale).to(rnd).float()
@@ -143,7 +143,8 @@ def main():
     ap.add_argument("--workload", default="c3", choices=sorted(WORKLOADS))
     ap.add_argument("--shape", type=int, nargs=4, metavar=("B", "M", "N", "w"),
                     help="time this shape instead of a named workload (forward + backward)")
-    ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp16"], help="storage type for --shape")
+    ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp16", "fp32"],
+                    help="storage type for --shape")
     ap.add_argument("--family", default="auto", choices=["auto", "wide", "strided"],
                     help="kernel family for the per-kernel timings: the library's choice, the wide-band MFMA "
                          "kernels even for a narrow band, or the strided kernels (A/B measurements)")
@@ -171,8 +172,8 @@ def main():
         args.workload = "custom"
     fam = {"auto": 0, "wide": abi.NO_NARROW_BAND, "strided": abi.FORCE_STRIDED}[args.family]
     B, M, N, w = cfg["B"], cfg["M"], cfg["N"], cfg["w"]
-    dtype = {"bf16": torch.bfloat16, "fp16": torch.float16}[cfg["dtype"]]
-    es = 2
+    dtype = {"bf16": torch.bfloat16, "fp16": torch.float16, "fp32": torch.float32}[cfg["dtype"]]
+    es = 4 if dtype == torch.float32 else 2
     dev = torch.device("cuda:0")
     g = torch.Generator().manual_seed(0)
 
@@ -263,11 +264,14 @@ def main():
         bs_bwd_ms = time_gpu(lambda: abi.band_softmax_backward(probs, ga if ga is not None else att, 1.0, out=sm_out),
                              max(args.steps, 10), 3)
         del sm_out
-        fo, flse = abi.attention_forward(qd, k.detach(), vd, w, 1.0)
-        fused_fwd_ms = time_gpu(lambda: abi.attention_forward(qd, k.detach(), vd, w, 1.0), max(args.steps, 10), 3)
-        fused_bwd_ms = (time_gpu(lambda: abi.attention_backward(qd, k.detach(), vd, fo, flse, go, w, 1.0),
-                                 max(args.steps, 10), 3) if cfg["backward"] else None)
-        del fo, flse
+        fused_fwd_ms = fused_bwd_ms = None
+        if es == 2:  # the fused kernels are 16-bit only; float32 runs the chain of separate ops
+            fo, flse = abi.attention_forward(qd, k.detach(), vd, w, 1.0)
+            fused_fwd_ms = time_gpu(lambda: abi.attention_forward(qd, k.detach(), vd, w, 1.0), max(args.steps, 10), 3)
+            if cfg["backward"]:
+                fused_bwd_ms = time_gpu(lambda: abi.attention_backward(qd, k.detach(), vd, fo, flse, go, w, 1.0),
+                                        max(args.steps, 10), 3)
+            del fo, flse
         # device-to-device copy of the band as the achievable-bandwidth yardstick
         scratch = torch.empty_like(att)
         copy_ms = time_gpu(lambda: scratch.copy_(att), 20, 3)
@@ -303,7 +307,8 @@ def main():
             "note": "same chain with window_matmul.band_softmax replacing torch.softmax"},
         "fused_attention": None if args.kernels_only else {
             "ms_per_step": round(fused_ms_per_step, 4), "TFLOPs": round(flops / fused_ms_per_step / 1e9, 2),
-            "fwd_ms": round(fused_fwd_ms, 4), "bwd_ms": None if fused_bwd_ms is None else round(fused_bwd_ms, 4),
+            "fwd_ms": None if fused_fwd_ms is None else round(fused_fwd_ms, 4),
+            "bwd_ms": None if fused_bwd_ms is None else round(fused_bwd_ms, 4),
             "mfma_frac": round(flops / fused_ms_per_step / 1e9 / 2500.0, 4),
             "note": "same chain as one call, window_matmul.window_attention; band FLOPs credited as for the "
                     "separate ops (recomputation in the backward not counted); mfma_frac against 2.5 PFLOP/s"},

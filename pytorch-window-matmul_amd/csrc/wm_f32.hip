@@ -49,6 +49,18 @@ __device__ __forceinline__ f32x4 load_row4(const float *p, const float *safe, bo
   f32x4 z = {0.f, 0.f, 0.f, 0.f};
   return valid ? v : z;
 }
+__device__ __forceinline__ bool band_any(int e_lo, int e_hi) { return (e_hi >= 0) & (e_lo <= 3) & (e_lo <= e_hi); }
+// Keeps a loaded value opaque until here, so that whatever is computed from it (masks) is not
+// scheduled right behind the load.
+__device__ __forceinline__ f32x4 pin(f32x4 v) {
+  asm volatile("" : "+v"(v));
+  return v;
+}
+__device__ __forceinline__ void wave_sync_lds() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
 __device__ __forceinline__ f32x16 mma(float a, float b, f32x16 c) {
   return __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, 0, 0, 0);
 }
@@ -62,9 +74,16 @@ __device__ __forceinline__ bool decode_block(int nblk, int B, int *b, int *blk) 
 // ------------------------------------------------------------------------------------------
 // P2: C[b,i,h] = sum_c T[i][c] Y[b,c,h]          P3: C[b,c,h] = sum_r T[r][c] Y[b,r,h]
 // acc(m = h, n = output row): A operand Y[k][h] (4-byte LDS reads along h), B operand T.
+//
+// Pipeline: chunk k+2 is requested (loads only, into one of two register sets) before chunk k is
+// multiplied; chunk k+1, requested a whole slot earlier, is masked and moved to LDS after the
+// multiply.  Loads and the masking of what they return are kept apart on purpose: a mask right
+// behind its load would make the wave wait for the load where it is issued.
 // ------------------------------------------------------------------------------------------
+constexpr int kStage = 32 + 4;  // staged result row: 32 floats, rows 16 bytes apart mod 128
+
 template <int NT, bool TRANSPOSED>
-__global__ __launch_bounds__(kThreads, 2) void f32_band_in_kernel(const float *__restrict__ A,
+__global__ __launch_bounds__(kThreads, NT <= 2 ? 3 : 2) void f32_band_in_kernel(const float *__restrict__ A,
                                                                   const float *__restrict__ Y,
                                                                   float *__restrict__ C, int B, int M, int N, int w,
                                                                   int nblk, int64_t asb, int64_t ysb, int64_t ysr,
@@ -75,6 +94,7 @@ __global__ __launch_bounds__(kThreads, 2) void f32_band_in_kernel(const float *_
   constexpr int SY = NP + 4;
   __shared__ __attribute__((aligned(16))) float t_lds[2][TROWS * ST];
   __shared__ __attribute__((aligned(16))) float y_lds[2][KC * SY];
+  static_assert(4 * 32 * kStage <= 2 * TROWS * ST, "the four staging areas must fit the band tile buffers");
 
   int b, blk;
   if (!decode_block(nblk, B, &b, &blk)) return;
@@ -87,42 +107,104 @@ __global__ __launch_bounds__(kThreads, 2) void f32_band_in_kernel(const float *_
   const float *Ab = A + (int64_t)b * asb;
   const float *Yb = Y + (int64_t)b * ysb;
   const int ncg = N >> 2, ychunks = KC * ncg;
+  int y_row[NT], y_col[NT];  // this thread's pieces of a Y chunk; row KC = none
+#pragma unroll
+  for (int s = 0; s < NT; ++s) {
+    const int q = tid + kThreads * s;
+    y_row[s] = q < ychunks ? q / ncg : KC;
+    y_col[s] = q < ychunks ? (q % ncg) * 4 : 0;
+  }
 
-  f32x4 t_reg[4], y_reg[NT];
-  auto fetch = [&](int k) {
-    const int kb = k_lo + k * KC;
+  // Band piece s of this thread: its address in chunk 0 (advanced by `t_step` elements per chunk)
+  // and what decides its valid element range [e_lo, e_hi] (0..3) in a chunk.
+  const float *t_ptr[4];
+  int t_fix[4];  // P2: band row i of the piece; P3: first output column c4 of the piece
+  const int64_t t_step = TRANSPOSED ? (int64_t)KC * (W - 1) : KC;
 #pragma unroll
-    for (int s = 0; s < 4; ++s) {
-      const int q = tid + kThreads * s;
-      if (!TRANSPOSED) {  // tile row = band row i, 4 consecutive dense columns c
-        const int i = o0 + (q >> 3), c4 = kb + 4 * (q & 7);
-        const int lo = max(i - w, 0), hi = i <= o1 ? min(i + w, k_hi) : -1;
-        t_reg[s] = load_band4(Ab + (int64_t)i * W + (w - i) + c4, A, lo - c4, hi - c4);
-      } else {  // tile row = band row r (the contraction index), 4 consecutive output columns c
-        const int r = kb + (q >> 5), c4 = o0 + 4 * (q & 31);
-        const int lo = max(r - w, o0), hi = r <= k_hi ? min(r + w, o1) : -1;
-        t_reg[s] = load_band4(Ab + (int64_t)r * W + (w - r) + c4, A, lo - c4, hi - c4);
-      }
+  for (int s = 0; s < 4; ++s) {
+    const int q = tid + kThreads * s;
+    if (!TRANSPOSED) {  // tile row = band row i, 4 consecutive dense columns c
+      const int i = o0 + (q >> 3);
+      t_fix[s] = i;
+      t_ptr[s] = Ab + (int64_t)i * W + (w - i) + k_lo + 4 * (q & 7);
+    } else {  // tile row = band row r (the contraction index), 4 consecutive output columns c
+      const int r = k_lo + (q >> 5), c4 = o0 + 4 * (q & 31);
+      t_fix[s] = c4;
+      t_ptr[s] = Ab + (int64_t)r * W + (w - r) + c4;
     }
-#pragma unroll
-    for (int s = 0; s < NT; ++s) {
-      const int q = tid + kThreads * s;
-      const int kr = kb + q / ncg;
-      y_reg[s] = load_row4(Yb + (int64_t)kr * ysr + (q % ncg) * 4, Y, (q < ychunks) & (kr <= k_hi));
+  }
+  auto piece_range = [&](int kb, int s, int &e_lo, int &e_hi) {
+    const int q = tid + kThreads * s;
+    if (!TRANSPOSED) {
+      const int i = t_fix[s], c4 = kb + 4 * (q & 7);
+      const int lo = max(i - w, 0), hi = i <= o1 ? min(i + w, k_hi) : -1;
+      e_lo = lo - c4, e_hi = hi - c4;
+    } else {
+      const int r = kb + (q >> 5), c4 = t_fix[s];
+      const int lo = max(r - w, o0), hi = r <= k_hi ? min(r + w, o1) : -1;
+      e_lo = lo - c4, e_hi = hi - c4;
     }
   };
-  auto stash = [&](int buf) {
+  // A chunk is interior when every band element of its tile and every Y row is valid: no address
+  // selection, no masks (most chunks of a wide band).
+  const bool block_whole = o1 == o0 + TM - 1;
+  auto interior = [&](int k) {
+    const int kb = k_lo + k * KC;
+    return block_whole && kb + KC - 1 <= k_hi && kb + KC - 1 - w <= o0 && o1 <= kb + w &&
+           (TRANSPOSED || kb >= o1 - w) && (!TRANSPOSED || kb + KC - 1 - w <= o0);
+  };
+  auto fetch = [&](int k, f32x4(&tr)[4], f32x4(&yr)[NT]) {  // loads only; chunks past the end read the safe address
+    const int kb = k_lo + k * KC;
+    if (interior(k)) {
+#pragma unroll
+      for (int s = 0; s < 4; ++s) tr[s] = load4(t_ptr[s] + k * t_step);
+#pragma unroll
+      for (int s = 0; s < NT; ++s)
+        yr[s] = *reinterpret_cast<const f32x4 *>(y_row[s] < KC ? Yb + (int64_t)(kb + y_row[s]) * ysr + y_col[s] : Y);
+    } else {
+#pragma unroll
+      for (int s = 0; s < 4; ++s) {
+        int e_lo, e_hi;
+        piece_range(kb, s, e_lo, e_hi);
+        tr[s] = load4(band_any(e_lo, e_hi) ? t_ptr[s] + k * t_step : A);
+      }
+#pragma unroll
+      for (int s = 0; s < NT; ++s) {
+        const int kr = kb + y_row[s];
+        const bool ok = (y_row[s] < KC) & (kr <= k_hi);
+        yr[s] = *reinterpret_cast<const f32x4 *>(ok ? Yb + (int64_t)kr * ysr + y_col[s] : Y);
+      }
+    }
+  };
+  auto stash = [&](int k, f32x4(&tr)[4], f32x4(&yr)[NT]) {  // mask, then to LDS buffer k & 1
+    const int kb = k_lo + k * KC, buf = k & 1;
+    f32x4 tv[4], yv[NT];
+#pragma unroll
+    for (int s = 0; s < 4; ++s) tv[s] = pin(tr[s]);
+#pragma unroll
+    for (int s = 0; s < NT; ++s) yv[s] = pin(yr[s]);
+    if (!interior(k)) {
+#pragma unroll
+      for (int s = 0; s < 4; ++s) {
+        int e_lo, e_hi;
+        piece_range(kb, s, e_lo, e_hi);
+        tv[s] = keep4(tv[s], band_any(e_lo, e_hi) ? e_lo : 4, e_hi);
+      }
+#pragma unroll
+      for (int s = 0; s < NT; ++s) {
+        const f32x4 z = {0.f, 0.f, 0.f, 0.f};
+        yv[s] = kb + y_row[s] <= k_hi ? yv[s] : z;
+      }
+    }
 #pragma unroll
     for (int s = 0; s < 4; ++s) {
       const int q = tid + kThreads * s;
       float *dst = TRANSPOSED ? &t_lds[buf][(q >> 5) * ST + 4 * (q & 31)] : &t_lds[buf][(q >> 3) * ST + 4 * (q & 7)];
-      *reinterpret_cast<f32x4 *>(dst) = t_reg[s];
+      *reinterpret_cast<f32x4 *>(dst) = tv[s];
     }
 #pragma unroll
-    for (int s = 0; s < NT; ++s) {
-      const int q = tid + kThreads * s;
-      if (q < ychunks) *reinterpret_cast<f32x4 *>(&y_lds[buf][(q / ncg) * SY + (q % ncg) * 4]) = y_reg[s];
-    }
+    for (int s = 0; s < NT; ++s)
+      if (y_row[s] < KC) *reinterpret_cast<f32x4 *>(&y_lds[buf][y_row[s] * SY + y_col[s]]) = yv[s];
   };
 
   f32x16 acc[NT];
@@ -131,13 +213,17 @@ __global__ __launch_bounds__(kThreads, 2) void f32_band_in_kernel(const float *_
 #pragma unroll
     for (int v = 0; v < 16; ++v) acc[t][v] = 0.f;
 
-  fetch(0);
-  stash(0);
+  f32x4 t_reg[2][4], y_reg[2][NT];
+  fetch(0, t_reg[0], y_reg[0]);
+  fetch(1, t_reg[1], y_reg[1]);
+  __builtin_amdgcn_sched_barrier(0);
+  stash(0, t_reg[0], y_reg[0]);
   __syncthreads();
   const int half = lane >> 5, col = lane & 31;
-  for (int k = 0; k < nk; ++k) {
+  auto slot = [&](int k, f32x4(&mine_t)[4], f32x4(&mine_y)[NT], f32x4(&next_t)[4], f32x4(&next_y)[NT]) {
     const int buf = k & 1;
-    if (k + 1 < nk) fetch(k + 1);
+    fetch(k + 2, mine_t, mine_y);
+    __builtin_amdgcn_sched_barrier(0);
     const float *tl = t_lds[buf];
     const float *yl = y_lds[buf];
 #pragma unroll
@@ -151,34 +237,54 @@ __global__ __launch_bounds__(kThreads, 2) void f32_band_in_kernel(const float *_
         for (int j = 0; j < 4; ++j) bop[j] = tl[(kk + j) * ST + wave * 32 + col];
       }
 #pragma unroll
-      for (int t = 0; t < NT; ++t)
+      for (int j = 0; j < 4; ++j)
 #pragma unroll
-        for (int j = 0; j < 4; ++j) acc[t] = mma(yl[(kk + j) * SY + 32 * t + col], bop[j], acc[t]);
+        for (int t = 0; t < NT; ++t) acc[t] = mma(yl[(kk + j) * SY + 32 * t + col], bop[j], acc[t]);
     }
-    if (k + 1 < nk) stash(buf ^ 1);
+    __builtin_amdgcn_sched_barrier(0);
+    stash(k + 1, next_t, next_y);
     __syncthreads();
+  };
+  // Slots run in pairs inside the loop, an odd last one after it: one loop exit, one back edge, so
+  // the compiler's count of outstanding loads is the same on every way into a slot.
+  int k = 0;
+  for (; k + 1 < nk; k += 2) {
+    slot(k, t_reg[0], y_reg[0], t_reg[1], y_reg[1]);
+    slot(k + 1, t_reg[1], y_reg[1], t_reg[0], y_reg[0]);
   }
+  if (k < nk) slot(k, t_reg[0], y_reg[0], t_reg[1], y_reg[1]);
 
-  // acc[t][v]: h = 32 t + 8 (v / 4) + 4 (lane / 32) + v % 4, output row = wave * 32 + lane % 32
-  const int o = o0 + wave * 32 + col;
-  if (o <= o1) {
-    float *crow = C + (int64_t)b * csb + (int64_t)o * csr;
+  // acc[t][v]: h = 32 t + 8 (v / 4) + 4 (lane / 32) + v % 4, output row = wave * 32 + lane % 32.
+  // Every wave is past the last barrier, so the tile buffers are free: each wave stages 32 columns
+  // of its rows at a time in a private area and the rows leave as 16-byte pieces, 8 consecutive
+  // lanes on one 128-byte line (non-temporal: the result is not read again here).
+  float *stage = &t_lds[0][0] + wave * (32 * kStage);
+  float *Cb = C + (int64_t)b * csb;
 #pragma unroll
-    for (int t = 0; t < NT; ++t)
+  for (int t = 0; t < NT; ++t) {
+    wave_sync_lds();
 #pragma unroll
-      for (int q4 = 0; q4 < 4; ++q4) {
-        const int h = 32 * t + 8 * q4 + 4 * half;
-        if (h < N) {
-          f32x4 out = {acc[t][4 * q4], acc[t][4 * q4 + 1], acc[t][4 * q4 + 2], acc[t][4 * q4 + 3]};
-          *reinterpret_cast<f32x4 *>(crow + h) = out;
-        }
-      }
+    for (int q4 = 0; q4 < 4; ++q4) {
+      const f32x4 out = {acc[t][4 * q4], acc[t][4 * q4 + 1], acc[t][4 * q4 + 2], acc[t][4 * q4 + 3]};
+      *reinterpret_cast<f32x4 *>(stage + col * kStage + 8 * q4 + 4 * half) = out;
+    }
+    wave_sync_lds();
+#pragma unroll
+    for (int s = 0; s < 4; ++s) {
+      const int rr = (lane >> 3) + 8 * s, h = 32 * t + 4 * (lane & 7);
+      const int o = o0 + wave * 32 + rr;
+      if (o <= o1 && h < N)
+        __builtin_nontemporal_store(*reinterpret_cast<const f32x4 *>(stage + rr * kStage + 4 * (lane & 7)),
+                                    reinterpret_cast<f32x4 *>(Cb + (int64_t)o * csr + h));
+    }
   }
 }
 
 // ------------------------------------------------------------------------------------------
 // P1: band[b,i,c-i+w] = sum_h X[b,i,h] Y[b,c,h]   (+0.0 where c is outside the sequence)
 // acc(m = c, n = i): A operand Y chunk (LDS, k = h along memory), B operand X rows (registers).
+// The 32 x 32 result of a wave and chunk is staged in wave-private LDS and leaves as 16-byte
+// pieces, 8 consecutive lanes on 128 consecutive bytes of one band row.
 // ------------------------------------------------------------------------------------------
 template <int NK8>  // N = 8 NK8
 __global__ __launch_bounds__(kThreads, 2) void f32_band_out_kernel(const float *__restrict__ X,
@@ -188,8 +294,10 @@ __global__ __launch_bounds__(kThreads, 2) void f32_band_out_kernel(const float *
                                                                    int64_t ysr, int64_t csb) {
   constexpr int N = 8 * NK8;
   constexpr int SY = N + 4;
-  constexpr int YS = (KC * N / 4 + kThreads - 1) / kThreads;
+  constexpr int PIECES = KC * N / 4;
+  constexpr int YS = (PIECES + kThreads - 1) / kThreads;
   __shared__ __attribute__((aligned(16))) float y_lds[2][KC * SY];
+  __shared__ __attribute__((aligned(16))) float stage_lds[4][32 * kStage];
 
   int b, blk;
   if (!decode_block(nblk, B, &b, &blk)) return;
@@ -210,31 +318,47 @@ __global__ __launch_bounds__(kThreads, 2) void f32_band_out_kernel(const float *
   for (int u = 0; u < NK8; ++u)
     xop[u] = load_row4(X + (int64_t)b * xsb + (int64_t)i * xsr + 8 * u + 4 * half, X, i < M);
 
-  f32x4 y_reg[YS];
-  auto fetch = [&](int k) {
+  int y_row[YS], y_col[YS];  // this thread's pieces of a Y chunk; row KC = none
+#pragma unroll
+  for (int s = 0; s < YS; ++s) {
+    const int q = tid + kThreads * s;
+    y_row[s] = q < PIECES ? q / (N / 4) : KC;
+    y_col[s] = q < PIECES ? (q % (N / 4)) * 4 : 0;
+  }
+  auto fetch = [&](int k, f32x4(&yr)[YS]) {  // loads only; rows outside the sequence read the safe address
     const int cb = c_lo + k * KC;
 #pragma unroll
     for (int s = 0; s < YS; ++s) {
-      const int q = tid + kThreads * s;
-      const int c = cb + q / (N / 4);
-      y_reg[s] = load_row4(Yb + (int64_t)c * ysr + (q % (N / 4)) * 4, Y, (q < KC * N / 4) & (c >= 0) & (c < M));
+      const int c = cb + y_row[s];
+      const bool ok = (y_row[s] < KC) & (c >= 0) & (c < M);
+      yr[s] = *reinterpret_cast<const f32x4 *>(ok ? Yb + (int64_t)c * ysr + y_col[s] : Y);
     }
   };
-  auto stash = [&](int buf) {
+  auto stash = [&](int k, f32x4(&yr)[YS]) {
+    const int cb = c_lo + k * KC, buf = k & 1;
+    f32x4 yv[YS];
+#pragma unroll
+    for (int s = 0; s < YS; ++s) yv[s] = pin(yr[s]);
 #pragma unroll
     for (int s = 0; s < YS; ++s) {
-      const int q = tid + kThreads * s;
-      if (q < KC * N / 4) *reinterpret_cast<f32x4 *>(&y_lds[buf][(q / (N / 4)) * SY + (q % (N / 4)) * 4]) = y_reg[s];
+      const int c = cb + y_row[s];
+      const f32x4 z = {0.f, 0.f, 0.f, 0.f};
+      if (y_row[s] < KC) *reinterpret_cast<f32x4 *>(&y_lds[buf][y_row[s] * SY + y_col[s]]) = (c >= 0) & (c < M) ? yv[s] : z;
     }
   };
 
-  fetch(0);
-  stash(0);
+  f32x4 y_reg[2][YS];
+  fetch(0, y_reg[0]);
+  fetch(1, y_reg[1]);
+  __builtin_amdgcn_sched_barrier(0);
+  stash(0, y_reg[0]);
   __syncthreads();
-  for (int k = 0; k < nk; ++k) {
+  float *stage = stage_lds[wave];
+  auto slot = [&](int k, f32x4(&mine)[YS], f32x4(&next)[YS]) {
     const int buf = k & 1;
     const int cb = c_lo + k * KC;
-    if (k + 1 < nk) fetch(k + 1);
+    fetch(k + 2, mine);
+    __builtin_amdgcn_sched_barrier(0);
     f32x16 acc;
 #pragma unroll
     for (int v = 0; v < 16; ++v) acc[v] = 0.f;
@@ -246,27 +370,43 @@ __global__ __launch_bounds__(kThreads, 2) void f32_band_out_kernel(const float *
       for (int j = 0; j < 4; ++j) acc = mma(aop[j], xop[u][j], acc);
     }
     // acc[v]: dense column c = cb + 8 (v / 4) + 4 half + v % 4, row i; band column j = c - i + w
-    if (i < M) {
-      float *brow = Cb + (int64_t)i * W + (w - i);  // address of dense column 0 of row i
+    wave_sync_lds();  // the pieces of the previous chunk have been read
 #pragma unroll
-      for (int q4 = 0; q4 < 4; ++q4) {
-        const int c = cb + 8 * q4 + 4 * half;
-        f32x4 out;
+    for (int q4 = 0; q4 < 4; ++q4) {
+      const int c = cb + 8 * q4 + 4 * half;
+      f32x4 out;
 #pragma unroll
-        for (int e = 0; e < 4; ++e) out[e] = (c + e >= 0 && c + e < M) ? acc[4 * q4 + e] : 0.f;  // +0.0 outside
-        const int e_lo = (i - w) - c, e_hi = (i + w) - c;
+      for (int e = 0; e < 4; ++e) out[e] = (c + e >= 0 && c + e < M) ? acc[4 * q4 + e] : 0.f;  // +0.0 outside
+      *reinterpret_cast<f32x4 *>(stage + col * kStage + 8 * q4 + 4 * half) = out;
+    }
+    wave_sync_lds();
+#pragma unroll
+    for (int s = 0; s < 4; ++s) {
+      const int rr = (lane >> 3) + 8 * s;
+      const int i2 = i0 + wave * 32 + rr, c = cb + 4 * (lane & 7);
+      const int e_lo = (i2 - w) - c, e_hi = (i2 + w) - c;
+      if (i2 < M && e_hi >= 0 && e_lo <= 3) {
+        const f32x4 out = *reinterpret_cast<const f32x4 *>(stage + rr * kStage + 4 * (lane & 7));
+        float *dst = Cb + (int64_t)i2 * W + (w - i2) + c;
         if (e_lo <= 0 && e_hi >= 3) {
-          store4(brow + c, out);
+          store4(dst, out);
         } else {
 #pragma unroll
           for (int e = 0; e < 4; ++e)
-            if (e >= e_lo && e <= e_hi) brow[c + e] = out[e];
+            if (e >= e_lo && e <= e_hi) dst[e] = out[e];
         }
       }
     }
-    if (k + 1 < nk) stash(buf ^ 1);
+    __builtin_amdgcn_sched_barrier(0);
+    stash(k + 1, next);
     __syncthreads();
+  };
+  int k = 0;
+  for (; k + 1 < nk; k += 2) {
+    slot(k, y_reg[0], y_reg[1]);
+    slot(k + 1, y_reg[1], y_reg[0]);
   }
+  if (k < nk) slot(k, y_reg[0], y_reg[1]);
 }
 
 // ------------------------------------------------------------------------------------------
