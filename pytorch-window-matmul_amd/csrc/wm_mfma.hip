@@ -118,7 +118,16 @@ __global__ __launch_bounds__(kThreads, NT <= 2 ? 3 : 2) void mfma_p2_kernel(cons
 #pragma unroll
       for (int s = 0; s < TS; ++s) {
         const int c8 = cb + 8 * ((tid + kThreads * s) & (GPR - 1));
-        tv[s] = mask_band_chunk(tv[s], t_lo[s] - c8, t_hi[s] - c8);
+        const int e_lo = t_lo[s] - c8, e_hi = t_hi[s] - c8;
+        // the 64 chunks of one wave instruction are 8 consecutive rows: in an edge chunk half of
+        // these groups are whole (nothing to mask) or empty (one select), wave-uniformly
+        const bool whole = (e_lo <= 0) & (e_hi >= 7), any = band_chunk_any(e_lo, e_hi);
+        if (__builtin_amdgcn_ballot_w64(!whole) == 0) continue;
+        if (__builtin_amdgcn_ballot_w64(any & !whole) == 0) {
+          tv[s] = mask_row_chunk(tv[s], any);
+        } else {
+          tv[s] = mask_band_chunk(tv[s], e_lo, e_hi);
+        }
       }
 #pragma unroll
       for (int s = 0; s < YS; ++s) {
