@@ -1,0 +1,87 @@
+"""Seeded random shapes: the tuned kernel families against the untuned one, on the GPU.
+
+The parity tests proper compare against the CPU oracle at hand-picked shapes.  This file adds
+breadth: shapes, dtypes and windows drawn from a fixed seed, the library's own kernel choice
+(narrow-band, wide-band MFMA, float32 MFMA) against the strided family, which shares no tiling,
+staging or masking code with them and is itself checked against the oracle in
+``test_gpu_parity.py``; and the fused attention kernels against the chain of the separate ops in
+float32.  Tolerances as everywhere: float32 1e-3, 16-bit 2e-2 (here relative to the largest
+reference magnitude, since both sides round).
+"""
+import random
+
+import pytest
+import torch
+
+import wm_ctypes as abi
+
+pytestmark = pytest.mark.gpu
+
+B_SET = [1, 2, 3, 5, 9]
+M_SET = [1, 7, 31, 64, 100, 128, 129, 255, 300, 513, 1000, 1500]
+W_SET = [1, 2, 3, 4, 5, 8, 9, 12, 16, 17, 24, 32, 33, 40, 64, 100, 128, 200, 256, 700]
+
+
+def _draw(seed, n, n_set, dtypes):
+    rng = random.Random(seed)
+    return [(rng.choice(dtypes), rng.choice(B_SET), rng.choice(M_SET), rng.choice(n_set), rng.choice(W_SET))
+            for _ in range(n)]
+
+
+def _randn(shape, g, dtype, dev, scale=1.0):
+    return (torch.randn(*shape, generator=g) * scale).to(dtype).to(dev)
+
+
+def _assert_close(got, want, tol, what):
+    got, want = got.float(), want.float()
+    assert torch.isfinite(got).all(), what
+    if got.numel():
+        err = (got - want).abs().max().item()
+        assert err <= tol * max(1.0, want.abs().max().item()), f"{what}: max error {err}"
+
+
+MATMUL_CASES = _draw(1, 60, [8, 16, 24, 32, 48, 64, 80, 96, 112, 128],
+                     [torch.bfloat16, torch.float16, torch.float32])
+
+
+@pytest.mark.parametrize("dtype,B,M,N,w", MATMUL_CASES,
+                         ids=[f"{str(d)[6:]}-B{B}-M{M}-N{N}-w{w}" for d, B, M, N, w in MATMUL_CASES])
+def test_kernel_choice_agrees_with_strided_family(device, dtype, B, M, N, w):
+    g = torch.Generator().manual_seed(B * 1000003 + M * 1009 + N * 31 + w)
+    q, k, v, go = (_randn((B, M, N), g, dtype, device) for _ in range(4))
+    a = _randn((B, M, 2 * w + 1), g, dtype, device, 0.2)
+    kt = k.transpose(1, 2)
+    tol = 1e-3 if dtype == torch.float32 else 2e-2
+    results = []
+    for flags in (0, abi.FORCE_STRIDED):
+        att = abi.window_forward(q, kt, w, flags)
+        out = abi.unwindow_forward(a, v, w, flags)
+        ga, gv = abi.unwindow_backward(a, v, w, go, flags)
+        gq, gk = abi.window_backward(q, kt, w, a, flags)
+        results.append(dict(window_fwd=att, unwindow_fwd=out, grad_a=ga, grad_v=gv, grad_q=gq, grad_k=gk))
+    for name in results[0]:
+        _assert_close(results[0][name], results[1][name], tol, name)
+
+
+ATTENTION_CASES = _draw(2, 40, [16, 32, 48, 64, 80, 96, 112, 128], [torch.bfloat16, torch.float16])
+
+
+@pytest.mark.parametrize("dtype,B,M,N,w", ATTENTION_CASES,
+                         ids=[f"{str(d)[6:]}-B{B}-M{M}-N{N}-w{w}" for d, B, M, N, w in ATTENTION_CASES])
+def test_fused_attention_agrees_with_chain_of_ops(device, dtype, B, M, N, w):
+    rng = random.Random(B * 7919 + M * 104729 + N * 13 + w)
+    mask = rng.choice([False, True])
+    scale = rng.choice([1.0, 2.0]) / N ** 0.5  # the usual 1 / sqrt(N), and scores twice as wide
+    g = torch.Generator().manual_seed(rng.randrange(1 << 30))
+    q, k, v, go = (_randn((B, M, N), g, dtype, device) for _ in range(4))
+    o, lse = abi.attention_forward(q, k, v, w, scale, mask)
+    gq, gk, gv = abi.attention_backward(q, k, v, o, lse, go, w, scale)
+    # the same chain on float32 copies of the rounded inputs
+    qf, kf, vf, gof = (t.float() for t in (q, k, v, go))
+    p = abi.band_softmax_forward(abi.window_forward(qf, kf.transpose(1, 2), w), scale, mask)
+    _assert_close(o, abi.unwindow_forward(p, vf, w), 2e-2, "output")
+    gp, gv_ref = abi.unwindow_backward(p, vf, w, gof)
+    gq_ref, gk_ref = abi.window_backward(qf, kf.transpose(1, 2), w, abi.band_softmax_backward(p, gp, scale, mask))
+    _assert_close(gq, gq_ref, 2e-2, "grad_q")
+    _assert_close(gk, gk_ref.transpose(1, 2), 2e-2, "grad_k")
+    _assert_close(gv, gv_ref, 2e-2, "grad_v")
