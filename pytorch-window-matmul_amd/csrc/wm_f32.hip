@@ -226,20 +226,25 @@ __global__ __launch_bounds__(kThreads, NT <= 2 ? 3 : 2) void f32_band_in_kernel(
     __builtin_amdgcn_sched_barrier(0);
     const float *tl = t_lds[buf];
     const float *yl = y_lds[buf];
+    // the wave's 32 output rows meet the chunk's 32 contraction indices only where |row - index| <= w:
+    // a chunk that lies wholly outside that range for this wave is all zeros in its part of the tile
+    const int kb = k_lo + k * KC, ow = o0 + wave * 32;
+    if (kb <= ow + 31 + w && kb + KC - 1 >= ow - w) {
 #pragma unroll
-    for (int u = 0; u < KC / 8; ++u) {
-      const int kk = 8 * u + 4 * half;  // this half-wave's 4 k values of the group
-      f32x4 bop;
-      if (!TRANSPOSED) {
-        bop = *reinterpret_cast<const f32x4 *>(tl + (wave * 32 + col) * ST + kk);
-      } else {
+      for (int u = 0; u < KC / 8; ++u) {
+        const int kk = 8 * u + 4 * half;  // this half-wave's 4 k values of the group
+        f32x4 bop;
+        if (!TRANSPOSED) {
+          bop = *reinterpret_cast<const f32x4 *>(tl + (wave * 32 + col) * ST + kk);
+        } else {
 #pragma unroll
-        for (int j = 0; j < 4; ++j) bop[j] = tl[(kk + j) * ST + wave * 32 + col];
+          for (int j = 0; j < 4; ++j) bop[j] = tl[(kk + j) * ST + wave * 32 + col];
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+          for (int t = 0; t < NT; ++t) acc[t] = mma(yl[(kk + j) * SY + 32 * t + col], bop[j], acc[t]);
       }
-#pragma unroll
-      for (int j = 0; j < 4; ++j)
-#pragma unroll
-        for (int t = 0; t < NT; ++t) acc[t] = mma(yl[(kk + j) * SY + 32 * t + col], bop[j], acc[t]);
     }
     __builtin_amdgcn_sched_barrier(0);
     stash(k + 1, next_t, next_y);
@@ -287,7 +292,7 @@ __global__ __launch_bounds__(kThreads, NT <= 2 ? 3 : 2) void f32_band_in_kernel(
 // pieces, 8 consecutive lanes on 128 consecutive bytes of one band row.
 // ------------------------------------------------------------------------------------------
 template <int NK8>  // N = 8 NK8
-__global__ __launch_bounds__(kThreads, 2) void f32_band_out_kernel(const float *__restrict__ X,
+__global__ __launch_bounds__(kThreads, NK8 <= 8 ? 4 : 2) void f32_band_out_kernel(const float *__restrict__ X,
                                                                    const float *__restrict__ Y,
                                                                    float *__restrict__ C, int B, int M, int w,
                                                                    int nblk, int64_t xsb, int64_t xsr, int64_t ysb,
@@ -359,6 +364,9 @@ __global__ __launch_bounds__(kThreads, 2) void f32_band_out_kernel(const float *
     const int cb = c_lo + k * KC;
     fetch(k + 2, mine);
     __builtin_amdgcn_sched_barrier(0);
+    // a wave whose 32 rows have no band entry among the chunk's 32 columns has nothing to compute or store
+    const int iw = i0 + wave * 32;
+    if (cb <= iw + 31 + w && cb + KC - 1 >= iw - w) {
     f32x16 acc;
 #pragma unroll
     for (int v = 0; v < 16; ++v) acc[v] = 0.f;
@@ -396,6 +404,7 @@ __global__ __launch_bounds__(kThreads, 2) void f32_band_out_kernel(const float *
             if (e >= e_lo && e <= e_hi) dst[e] = out[e];
         }
       }
+    }
     }
     __builtin_amdgcn_sched_barrier(0);
     stash(k + 1, next);
