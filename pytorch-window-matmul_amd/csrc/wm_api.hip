@@ -26,13 +26,15 @@ int to_status(hipError_t err) {
 typedef bool (*mfma_fn)(const Problem &, const View &, const View &, const View &, hipError_t *);
 typedef hipError_t (*strided_fn)(const Problem &, const View &, const View &, const View &);
 
-// Kernel choice per primitive: narrow-band family, else wide-band MFMA family (both 16-bit
-// storage), else the float32 MFMA family, else strided.
-int run_primitive(mfma_fn narrow, mfma_fn fast, mfma_fn f32, strided_fn slow, const Problem &p, const View &a,
-                  const View &y, const View &c) {
+// Kernel choice per primitive: narrow-band family (MFMA, or vector ALU for the windows that
+// leaves out), else wide-band MFMA family (all 16-bit storage), else the float32 MFMA family,
+// else strided.
+int run_primitive(mfma_fn narrow, mfma_fn vector, mfma_fn fast, mfma_fn f32, strided_fn slow, const Problem &p,
+                  const View &a, const View &y, const View &c) {
   hipError_t err = hipSuccess;
   if (!(p.flags & WM_FLAG_FORCE_STRIDED)) {
     if (narrow && !(p.flags & WM_FLAG_NO_NARROW_BAND) && narrow(p, a, y, c, &err)) return to_status(err);
+    if (vector && !(p.flags & WM_FLAG_NO_NARROW_BAND) && vector(p, a, y, c, &err)) return to_status(err);
     if (fast(p, a, y, c, &err)) return to_status(err);
     if (f32(p, a, y, c, &err)) return to_status(err);
   }
@@ -40,13 +42,16 @@ int run_primitive(mfma_fn narrow, mfma_fn fast, mfma_fn f32, strided_fn slow, co
 }
 
 int p1(const Problem &p, const View &x, const View &y, const View &c) {
-  return run_primitive(try_launch_small_p1, try_launch_mfma_p1, try_launch_f32_p1, launch_strided_p1, p, x, y, c);
+  return run_primitive(try_launch_small_p1, nullptr, try_launch_mfma_p1, try_launch_f32_p1, launch_strided_p1, p, x, y,
+                       c);
 }
 int p2(const Problem &p, const View &a, const View &y, const View &c) {
-  return run_primitive(try_launch_small_p2, try_launch_mfma_p2, try_launch_f32_p2, launch_strided_p2, p, a, y, c);
+  return run_primitive(try_launch_small_p2, try_launch_vector_p2, try_launch_mfma_p2, try_launch_f32_p2,
+                       launch_strided_p2, p, a, y, c);
 }
 int p3(const Problem &p, const View &a, const View &y, const View &c) {
-  return run_primitive(try_launch_small_p3, try_launch_mfma_p3, try_launch_f32_p3, launch_strided_p3, p, a, y, c);
+  return run_primitive(try_launch_small_p3, try_launch_vector_p3, try_launch_mfma_p3, try_launch_f32_p3,
+                       launch_strided_p3, p, a, y, c);
 }
 
 }  // namespace
@@ -187,6 +192,7 @@ const char *wm_kernel_choice(int op, int64_t B, int64_t M, int64_t N, int64_t w,
       static const char *names[] = {"narrow_p1", "narrow_p2", "narrow_p3"};
       return names[op - 1];
     }
+    if (!(flags & WM_FLAG_NO_NARROW_BAND) && vector_supports(op, M, N, w, dtype)) return op == 2 ? "vector_p2" : "vector_p3";
     if (mfma_supports(op, B, M, N, w, dtype)) {
       static const char *names[] = {"mfma_p1", "mfma_p2", "mfma_p3"};
       return names[op - 1];

@@ -49,6 +49,10 @@ bool try_launch_small_p1(const Problem &p, const View &x, const View &y, const V
 bool try_launch_small_p2(const Problem &p, const View &a, const View &y, const View &c, hipError_t *err);
 bool try_launch_small_p3(const Problem &p, const View &a, const View &y, const View &c, hipError_t *err);
 bool small_supports(int op, int64_t M, int64_t N, int64_t w, int dtype);
+// Vector-ALU band-in kernels for the very narrow windows the narrow-band family leaves out (w % 4 != 0).
+bool try_launch_vector_p2(const Problem &p, const View &a, const View &y, const View &c, hipError_t *err);
+bool try_launch_vector_p3(const Problem &p, const View &a, const View &y, const View &c, hipError_t *err);
+bool vector_supports(int op, int64_t M, int64_t N, int64_t w, int dtype);
 // float32 MFMA family (N multiple of 8 up to 128, w >= 4).
 bool try_launch_f32_p1(const Problem &p, const View &x, const View &y, const View &c, hipError_t *err);
 bool try_launch_f32_p2(const Problem &p, const View &a, const View &y, const View &c, hipError_t *err);
