@@ -42,8 +42,8 @@ int run_primitive(mfma_fn narrow, mfma_fn vector, mfma_fn fast, mfma_fn f32, str
 }
 
 int p1(const Problem &p, const View &x, const View &y, const View &c) {
-  return run_primitive(try_launch_small_p1, nullptr, try_launch_mfma_p1, try_launch_f32_p1, launch_strided_p1, p, x, y,
-                       c);
+  return run_primitive(try_launch_small_p1, try_launch_vector_p1, try_launch_mfma_p1, try_launch_f32_p1,
+                       launch_strided_p1, p, x, y, c);
 }
 int p2(const Problem &p, const View &a, const View &y, const View &c) {
   return run_primitive(try_launch_small_p2, try_launch_vector_p2, try_launch_mfma_p2, try_launch_f32_p2,
@@ -192,7 +192,10 @@ const char *wm_kernel_choice(int op, int64_t B, int64_t M, int64_t N, int64_t w,
       static const char *names[] = {"narrow_p1", "narrow_p2", "narrow_p3"};
       return names[op - 1];
     }
-    if (!(flags & WM_FLAG_NO_NARROW_BAND) && vector_supports(op, M, N, w, dtype)) return op == 2 ? "vector_p2" : "vector_p3";
+    if (!(flags & WM_FLAG_NO_NARROW_BAND) && vector_supports(op, M, N, w, dtype)) {
+      static const char *names[] = {"vector_p1", "vector_p2", "vector_p3"};
+      return names[op - 1];
+    }
     if (mfma_supports(op, B, M, N, w, dtype)) {
       static const char *names[] = {"mfma_p1", "mfma_p2", "mfma_p3"};
       return names[op - 1];

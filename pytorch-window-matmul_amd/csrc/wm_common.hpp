@@ -49,7 +49,9 @@ bool try_launch_small_p1(const Problem &p, const View &x, const View &y, const V
 bool try_launch_small_p2(const Problem &p, const View &a, const View &y, const View &c, hipError_t *err);
 bool try_launch_small_p3(const Problem &p, const View &a, const View &y, const View &c, hipError_t *err);
 bool small_supports(int op, int64_t M, int64_t N, int64_t w, int dtype);
-// Vector-ALU band-in kernels for the very narrow windows the narrow-band family leaves out (w % 4 != 0).
+// Vector-ALU kernels for the very narrow windows the MFMA families leave out: 16-bit band-in products
+// at w % 4 != 0 below 8, float32 (all three products) below the float32 family's range.
+bool try_launch_vector_p1(const Problem &p, const View &x, const View &y, const View &c, hipError_t *err);
 bool try_launch_vector_p2(const Problem &p, const View &a, const View &y, const View &c, hipError_t *err);
 bool try_launch_vector_p3(const Problem &p, const View &a, const View &y, const View &c, hipError_t *err);
 bool vector_supports(int op, int64_t M, int64_t N, int64_t w, int dtype);

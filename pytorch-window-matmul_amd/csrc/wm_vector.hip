@@ -1,28 +1,35 @@
-// Vector-ALU band-in kernels for very narrow bands (16-bit storage, float32 accumulate) on gfx950.
+// Vector-ALU kernels for very narrow bands on gfx950 (16-bit storage and float32, float32 accumulate).
 //
 // The narrow-band MFMA kernels read their skewed tile with 16-byte LDS reads, which needs the flat
-// band image to keep 8-column groups aligned in every row, i.e. w % 4 == 0.  For the other small
-// windows (w = 1, 2, 3, 5, 6, 7, ...) the band-in products
+// band image to keep 8-column groups aligned in every row, i.e. w % 4 == 0, and the float32 MFMA
+// kernels walk 128-row tiles in chunks of 32 columns, mostly empty when the band is a few entries
+// wide.  For these windows the band-in products
 //     P2  C[i,h] = sum_j A[i,j] Y[i+j-w,h]          P3  C[c,h] = sum_r A[r,c-r+w] Y[r,h]
 // are 2w+1 multiply-adds per output element on operands that are streamed once: far too little
-// arithmetic for the matrix pipe to matter, so each thread simply owns 8 consecutive output
-// columns of one row and walks the 2w+1 terms: one 2-byte LDS read of the band entry (the same
-// address for the 8 threads of a row), one 16-byte LDS read of the Y row piece, 8 packed dot
-// products that each pair the entry with one of the 8 values (and a zero with its neighbour).
-// The workgroup first copies what it needs into LDS with coalesced 16-byte loads (its band rows
-// as one flat image, the Y rows they reach row-major, zero outside the sequence); the result
-// leaves as 16-byte non-temporal stores, 8 consecutive threads on one 128-byte row (N = 64).
-// One barrier per workgroup; no atomics.
+// arithmetic for the matrix pipe to matter, so each thread simply owns 16 bytes of one output row
+// (8 or 4 consecutive columns) and walks the 2w+1 terms: one LDS read of the band entry (the same
+// address for the threads of a row), one 16-byte LDS read of the Y row piece, 8 packed dot products
+// that each pair the entry with one of the 8 values and a zero with its neighbour (16-bit), or 4
+// FMAs (float32).  The workgroup first copies what it needs into LDS with coalesced 16-byte loads
+// (its band rows as one flat image, the Y rows they reach row-major, zero outside the sequence);
+// the result leaves as 16-byte non-temporal stores, consecutive threads on consecutive pieces of a row.
+// The float32 band-out product  P1  band[i,j] = sum_h X[i,h] Y[i+j-w,h]  gets the same treatment:
+// X and Y rows in LDS, one thread per band entry, consecutive threads on consecutive entries of
+// the flat band.  One barrier per workgroup; no atomics.
 #include "wm_mfma_common.hpp"
 
 namespace wm {
 namespace {
 
-constexpr int VROWS = 128;  // output rows per workgroup
 #ifndef WM_VECTOR_MAX_W
 #define WM_VECTOR_MAX_W 7
 #endif
 constexpr int VECTOR_MAX_W = WM_VECTOR_MAX_W;
+#ifndef WM_VECTOR_F32_MAX_W
+#define WM_VECTOR_F32_MAX_W 10
+#endif
+constexpr int VECTOR_F32_MAX_W = WM_VECTOR_F32_MAX_W;
+typedef float f32x4v __attribute__((ext_vector_type(4)));
 
 // acc + a.lo * y.lo + a.hi * y.hi on packed pairs (v_dot2_f32_bf16 / v_dot2_f32_f16): with the band
 // entry in one half of `a` and zero in the other, one instruction per multiply-add and no unpacking.
@@ -38,38 +45,52 @@ __device__ __forceinline__ float dot2<f16_t>(uint32_t a, uint32_t y, float acc) 
   return __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2, a), __builtin_bit_cast(f16x2, y), acc, false);
 }
 
+// Storage element of a type tag, and the float32 "tag".
+struct f32_t {};
+template <typename T>
+struct Elem {
+  typedef uint16_t type;
+};
+template <>
+struct Elem<f32_t> {
+  typedef float type;
+};
+
 // TRANSPOSED false: P2 (rows = band rows i).  TRANSPOSED true: P3 (rows = output rows c, the
 // contraction runs over the band rows r = c-w .. c+w).
-template <typename T, int NK, bool TRANSPOSED>  // N = 16 NK
-__global__ __launch_bounds__(kThreads) void vector_band_in_kernel(const uint16_t *__restrict__ A,
-                                                                  const uint16_t *__restrict__ Y,
-                                                                  uint16_t *__restrict__ C, int B, int M, int w,
-                                                                  int nblk, int64_t asb, int64_t ysb, int64_t ysr,
-                                                                  int64_t csb, int64_t csr) {
-  constexpr int N = 16 * NK, NCG = N / 8;  // 16-byte column groups per row
-  constexpr int SY = N + 8;                // Y image rows 16 bytes apart mod 128
-  extern __shared__ __attribute__((aligned(16))) uint16_t lds[];
+template <typename T, int NK, bool TRANSPOSED>  // N = 16 NK (16-bit) or 8 NK (float32): 2 NK pieces per row
+__global__ __launch_bounds__(kThreads) void vector_band_in_kernel(const typename Elem<T>::type *__restrict__ A,
+                                                                  const typename Elem<T>::type *__restrict__ Y,
+                                                                  typename Elem<T>::type *__restrict__ C, int B,
+                                                                  int M, int w, int nblk, int vrows, int64_t asb,
+                                                                  int64_t ysb, int64_t ysr, int64_t csb, int64_t csr) {
+  typedef typename Elem<T>::type E;
+  constexpr int VEC = 16 / sizeof(E);       // elements per 16-byte piece
+  constexpr int NCG = 2 * NK, N = NCG * VEC;  // 16-byte column groups per row
+  constexpr int SY = N + VEC;               // Y image rows 16 bytes apart mod 128
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
+  E *lds = reinterpret_cast<E *>(lds_raw);
 
   int b, blk;
   if (!decode_block(nblk, B, &b, &blk)) return;
   const int tid = threadIdx.x;
   const int W = 2 * w + 1;
-  const int o0 = blk * VROWS;                      // first output row
-  const int orows = min(VROWS, M - o0);
+  const int o0 = blk * vrows;                      // first output row
+  const int orows = min(vrows, M - o0);
   // rows held in LDS: Y rows [y0, y0 + yrows) (may reach outside the sequence: zeros), band rows
   // [a0, a0 + arows) (inside the sequence)
   const int y0 = o0 - w, yrows = orows + 2 * w;
   const int a0 = TRANSPOSED ? max(o0 - w, 0) : o0;
   const int a1 = TRANSPOSED ? min(o0 + orows - 1 + w, M - 1) : o0 + orows - 1;
   const int arows = a1 - a0 + 1;
-  const uint16_t *Ab = A + (int64_t)b * asb + (int64_t)a0 * W;
-  const uint16_t *Yb = Y + (int64_t)b * ysb;
+  const E *Ab = A + (int64_t)b * asb + (int64_t)a0 * W;
+  const E *Yb = Y + (int64_t)b * ysb;
   // flat band image in whole aligned 16-byte chunks: image element e is band element e - delta
-  const int delta = (int)((reinterpret_cast<uintptr_t>(Ab) >> 1) & 7);
+  const int delta = (int)((reinterpret_cast<uintptr_t>(Ab) / sizeof(E)) & (VEC - 1));
   const int n_el = arows * W;
-  const int chunks = (delta + n_el + 7) >> 3;
-  uint16_t *aimg = lds;
-  uint16_t *yimg = lds + (((VROWS + 2 * w) * W + 16 + 7) & ~7);  // sized for the largest image
+  const int chunks = (delta + n_el + VEC - 1) / VEC;
+  E *aimg = lds;
+  E *yimg = lds + (((vrows + 2 * w) * W + 2 * VEC + VEC - 1) & ~(VEC - 1));  // sized for the largest image
   const int ychunks = yrows * NCG;
 
   // loads go out in batches of 8 per thread before any of them is used
@@ -80,7 +101,7 @@ __global__ __launch_bounds__(kThreads) void vector_band_in_kernel(const uint16_t
     for (int s = 0; s < BATCH; ++s) {
       const int q = base + s * kThreads + tid;
       const int qy = q - chunks, yr = qy / NCG, hg = qy - yr * NCG, c = y0 + yr;
-      const uint16_t *src = q < chunks ? Ab - delta + 8 * q : Yb + (int64_t)c * ysr + 8 * hg;
+      const E *src = q < chunks ? Ab - delta + VEC * q : Yb + (int64_t)c * ysr + VEC * hg;
       const bool ok = q < chunks || (q < chunks + ychunks && c >= 0 && c < M);
       reg[s] = *reinterpret_cast<const u32x4 *>(ok ? src : A);
     }
@@ -89,9 +110,9 @@ __global__ __launch_bounds__(kThreads) void vector_band_in_kernel(const uint16_t
       const int q = base + s * kThreads + tid;
       const int qy = q - chunks, yr = qy / NCG, hg = qy - yr * NCG, c = y0 + yr;
       if (q < chunks)
-        *reinterpret_cast<u32x4 *>(aimg + 8 * q) = reg[s];
+        *reinterpret_cast<u32x4 *>(aimg + VEC * q) = reg[s];
       else if (q < chunks + ychunks)
-        *reinterpret_cast<u32x4 *>(yimg + yr * SY + 8 * hg) = mask_row_chunk(reg[s], (c >= 0) & (c < M));
+        *reinterpret_cast<u32x4 *>(yimg + yr * SY + VEC * hg) = mask_row_chunk(reg[s], (c >= 0) & (c < M));
     }
   }
   __syncthreads();
@@ -99,54 +120,161 @@ __global__ __launch_bounds__(kThreads) void vector_band_in_kernel(const uint16_t
   for (int item = tid; item < orows * NCG; item += kThreads) {
     const int r = item / NCG, hg = item - r * NCG;
     const int o = o0 + r;  // output row
-    float acc[8];
+    float acc[VEC];
 #pragma unroll
-    for (int e = 0; e < 8; ++e) acc[e] = 0.f;
+    for (int e = 0; e < VEC; ++e) acc[e] = 0.f;
     // term t = 0 .. 2w: the Y row is o - w + t (image row r + t) in both products
     const int t_lo = max(0, w - o), t_hi = min(2 * w, M - 1 - o + w);  // Y rows inside the sequence
-    const uint16_t *yp = yimg + (r + t_lo) * SY + 8 * hg;
+    const E *yp = yimg + (r + t_lo) * SY + VEC * hg;
     // P2: band entry (o, t) -> image index (o - a0) W + t, next term +1.
     // P3: band entry (o - w + t, 2w - t) -> image index (o - w + t - a0) W + 2w - t, next term +W - 1.
-    const uint16_t *ap = aimg + delta + (TRANSPOSED ? (o - w + t_lo - a0) * W + 2 * w - t_lo : (o - a0) * W + t_lo);
+    const E *ap = aimg + delta + (TRANSPOSED ? (o - w + t_lo - a0) * W + 2 * w - t_lo : (o - a0) * W + t_lo);
     const int a_step = TRANSPOSED ? W - 1 : 1;
     for (int t = t_lo; t <= t_hi; ++t) {
-      const uint32_t a_lo = *ap, a_hi = a_lo << 16;  // (a, 0) and (0, a)
       const u32x4 y = *reinterpret_cast<const u32x4 *>(yp);
+      if constexpr (sizeof(E) == 2) {
+        const uint32_t a_lo = *ap, a_hi = a_lo << 16;  // (a, 0) and (0, a)
 #pragma unroll
-      for (int d = 0; d < 4; ++d) {
-        acc[2 * d] = dot2<T>(a_lo, y[d], acc[2 * d]);
-        acc[2 * d + 1] = dot2<T>(a_hi, y[d], acc[2 * d + 1]);
+        for (int d = 0; d < 4; ++d) {
+          acc[2 * d] = dot2<T>(a_lo, y[d], acc[2 * d]);
+          acc[2 * d + 1] = dot2<T>(a_hi, y[d], acc[2 * d + 1]);
+        }
+      } else {
+        const float a = *ap;
+        const f32x4v yf = __builtin_bit_cast(f32x4v, y);  // (a bit cast of one element y[d] reads element 0)
+#pragma unroll
+        for (int d = 0; d < 4; ++d) acc[d] = __builtin_fmaf(a, yf[d], acc[d]);
       }
       ap += a_step;
       yp += SY;
     }
-    const u32x4 out = {Mma<T>::pack2(acc[0], acc[1]), Mma<T>::pack2(acc[2], acc[3]), Mma<T>::pack2(acc[4], acc[5]),
-                       Mma<T>::pack2(acc[6], acc[7])};
-    __builtin_nontemporal_store(out, reinterpret_cast<u32x4 *>(C + (int64_t)b * csb + (int64_t)o * csr + 8 * hg));
+    u32x4 out;
+    if constexpr (sizeof(E) == 2) {
+      out = u32x4{Mma<T>::pack2(acc[0], acc[1]), Mma<T>::pack2(acc[2], acc[3]), Mma<T>::pack2(acc[4], acc[5]),
+                  Mma<T>::pack2(acc[6], acc[7])};
+    } else {
+      out = u32x4{__builtin_bit_cast(uint32_t, acc[0]), __builtin_bit_cast(uint32_t, acc[1]),
+                  __builtin_bit_cast(uint32_t, acc[2]), __builtin_bit_cast(uint32_t, acc[3])};
+    }
+    __builtin_nontemporal_store(out, reinterpret_cast<u32x4 *>(C + (int64_t)b * csb + (int64_t)o * csr + VEC * hg));
   }
 }
 
-size_t vector_lds(int64_t w, int64_t N) {
-  const int64_t W = 2 * w + 1;
-  return (size_t)((((VROWS + 2 * w) * W + 16 + 7) & ~(int64_t)7) + (VROWS + 2 * w) * (N + 8)) * 2;
+// float32 P1: band[b,i,j] = sum_h X[b,i,h] Y[b,i+j-w,h]  (+0.0 where i+j-w is outside the sequence).
+// One thread per band entry, consecutive threads on consecutive entries of the flat band.
+template <int NK>  // N = 8 NK
+__global__ __launch_bounds__(kThreads) void vector_band_out_f32_kernel(const float *__restrict__ X,
+                                                                       const float *__restrict__ Y,
+                                                                       float *__restrict__ C, int B, int M, int w,
+                                                                       int nblk, int vrows, int64_t xsb, int64_t xsr,
+                                                                       int64_t ysb, int64_t ysr, int64_t csb) {
+  constexpr int N = 8 * NK, NCG = N / 4;
+  constexpr int SX = N + 4;  // rows 16 bytes apart mod 128
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
+  float *ximg = reinterpret_cast<float *>(lds_raw);  // rows i0 .. i0 + rows
+  float *yimg = ximg + vrows * SX;                   // rows i0 - w .. i0 + rows + w, zero outside the sequence
+
+  int b, blk;
+  if (!decode_block(nblk, B, &b, &blk)) return;
+  const int tid = threadIdx.x;
+  const int W = 2 * w + 1;
+  const int i0 = blk * vrows;
+  const int rows = min(vrows, M - i0);
+  const float *Xb = X + (int64_t)b * xsb, *Yb = Y + (int64_t)b * ysb;
+  const int xchunks = rows * NCG, ychunks = (rows + 2 * w) * NCG;
+  constexpr int BATCH = 8;
+  for (int base = 0; base < xchunks + ychunks; base += BATCH * kThreads) {
+    u32x4 reg[BATCH];
+#pragma unroll
+    for (int s = 0; s < BATCH; ++s) {
+      const int q = base + s * kThreads + tid;
+      const int qy = q - xchunks;
+      const int xr = q / NCG, xg = q - xr * NCG, yr = qy / NCG, yg = qy - yr * NCG, c = i0 - w + yr;
+      const float *src = q < xchunks ? Xb + (int64_t)(i0 + xr) * xsr + 4 * xg : Yb + (int64_t)c * ysr + 4 * yg;
+      const bool ok = q < xchunks || (q < xchunks + ychunks && c >= 0 && c < M);
+      reg[s] = *reinterpret_cast<const u32x4 *>(ok ? src : X);
+    }
+#pragma unroll
+    for (int s = 0; s < BATCH; ++s) {
+      const int q = base + s * kThreads + tid;
+      const int qy = q - xchunks;
+      const int xr = q / NCG, xg = q - xr * NCG, yr = qy / NCG, yg = qy - yr * NCG, c = i0 - w + yr;
+      if (q < xchunks)
+        *reinterpret_cast<u32x4 *>(ximg + xr * SX + 4 * xg) = reg[s];
+      else if (q < xchunks + ychunks)
+        *reinterpret_cast<u32x4 *>(yimg + yr * SX + 4 * yg) = mask_row_chunk(reg[s], (c >= 0) & (c < M));
+    }
+  }
+  __syncthreads();
+
+  float *Cb = C + (int64_t)b * csb + (int64_t)i0 * W;
+  for (int item = tid; item < rows * W; item += kThreads) {
+    const int r = item / W, j = item - r * W;
+    const int c = i0 + r + j - w;
+    const float *xp = ximg + r * SX, *yp = yimg + (r + j) * SX;
+    float acc[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int g = 0; g < NCG; ++g) {
+      const f32x4v x = *reinterpret_cast<const f32x4v *>(xp + 4 * g), y = *reinterpret_cast<const f32x4v *>(yp + 4 * g);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) acc[e] = __builtin_fmaf(x[e], y[e], acc[e]);
+    }
+    const float sum = (acc[0] + acc[1]) + (acc[2] + acc[3]);
+    Cb[item] = (c >= 0 && c < M) ? sum : 0.f;  // +0.0 outside the sequence, whatever X holds
+  }
 }
+
+// Output rows per workgroup: as many as keep the LDS images of the widest supported window small.
+int vector_rows(int64_t N, int dtype) { return dtype == WM_DTYPE_F32 && N > 64 ? 64 : 128; }
+int vector_out_rows(int64_t N) { return N > 64 ? 32 : 64; }
+size_t vector_lds(int64_t w, int64_t N, int dtype) {
+  const int64_t W = 2 * w + 1, vec = dtype == WM_DTYPE_F32 ? 4 : 8, rows = vector_rows(N, dtype);
+  return (size_t)((((rows + 2 * w) * W + 3 * vec - 1) & ~(vec - 1)) + (rows + 2 * w) * (N + vec)) * (16 / vec);
+}
+size_t vector_out_lds(int64_t w, int64_t N) { return (size_t)((2 * vector_out_rows(N) + 2 * w) * (N + 4)) * 4; }
+
+unsigned vector_grid(int64_t B, int64_t nblk) { return (unsigned)(((B + 7) / 8) * 8 * nblk); }
 
 template <typename T, bool TRANSPOSED>
 hipError_t launch_vector(const Problem &p, const View &a, const View &y, const View &c) {
-  const int nblk = (int)((p.M + VROWS - 1) / VROWS);
-  const dim3 grid((unsigned)(((p.B + 7) / 8) * 8 * nblk)), block(kThreads);
-  const size_t lds = vector_lds(p.w, p.N);
+  typedef typename Elem<T>::type E;
+  const int vrows = vector_rows(p.N, p.dtype);
+  const int nblk = (int)((p.M + vrows - 1) / vrows);
+  const dim3 grid(vector_grid(p.B, nblk)), block(kThreads);
+  const size_t lds = vector_lds(p.w, p.N, p.dtype);
+  const int pieces = (int)(p.N * sizeof(E) / 16);
 #define WM_VEC(NK)                                                                                              \
   case NK:                                                                                                      \
-    hipLaunchKernelGGL((vector_band_in_kernel<T, NK, TRANSPOSED>), grid, block, lds, p.stream,                  \
-                       (const uint16_t *)a.data, (const uint16_t *)y.data, (uint16_t *)c.data, (int)p.B,        \
-                       (int)p.M, (int)p.w, nblk, a.sb, y.sb, y.sr, c.sb, c.sr);                                 \
+    hipLaunchKernelGGL((vector_band_in_kernel<T, NK, TRANSPOSED>), grid, block, lds, p.stream, (const E *)a.data, \
+                       (const E *)y.data, (E *)c.data, (int)p.B, (int)p.M, (int)p.w, nblk, vrows, a.sb, y.sb, y.sr, \
+                       c.sb, c.sr);                                                                                   \
     break;
-  switch (p.N / 16) {
+  switch (pieces / 2) {
     WM_VEC(1) WM_VEC(2) WM_VEC(3) WM_VEC(4) WM_VEC(5) WM_VEC(6) WM_VEC(7) WM_VEC(8)
+    WM_VEC(9) WM_VEC(10) WM_VEC(11) WM_VEC(12) WM_VEC(13) WM_VEC(14) WM_VEC(15) WM_VEC(16)
     default: return hipErrorInvalidValue;
   }
 #undef WM_VEC
+  return hipGetLastError();
+}
+
+hipError_t launch_vector_out_f32(const Problem &p, const View &x, const View &y, const View &c) {
+  const int vrows = vector_out_rows(p.N);
+  const int nblk = (int)((p.M + vrows - 1) / vrows);
+  const dim3 grid(vector_grid(p.B, nblk)), block(kThreads);
+  const size_t lds = vector_out_lds(p.w, p.N);
+#define WM_VOUT(NK)                                                                                             \
+  case NK:                                                                                                      \
+    hipLaunchKernelGGL((vector_band_out_f32_kernel<NK>), grid, block, lds, p.stream, (const float *)x.data,     \
+                       (const float *)y.data, (float *)c.data, (int)p.B, (int)p.M, (int)p.w, nblk, vrows, x.sb,  \
+                       x.sr, y.sb, y.sr, c.sb);                                                                       \
+    break;
+  switch (p.N / 8) {
+    WM_VOUT(1) WM_VOUT(2) WM_VOUT(3) WM_VOUT(4) WM_VOUT(5) WM_VOUT(6) WM_VOUT(7) WM_VOUT(8)
+    WM_VOUT(9) WM_VOUT(10) WM_VOUT(11) WM_VOUT(12) WM_VOUT(13) WM_VOUT(14) WM_VOUT(15) WM_VOUT(16)
+    default: return hipErrorInvalidValue;
+  }
+#undef WM_VOUT
   return hipGetLastError();
 }
 
@@ -154,27 +282,41 @@ bool band_contiguous(const View &v, int64_t W) { return v.sc == 1 && v.sr == W &
 
 }  // namespace
 
-// Windows the narrow-band MFMA kernels do not take (w % 4 != 0) and the wide-band kernels either do
-// not take (w < 8) or serve poorly.
+// 16-bit: the windows the narrow-band MFMA kernels do not take (w % 4 != 0) below the wide-band
+// family's range (band-in products only; the narrow-band band-out kernel takes every w).
+// float32: every window up to VECTOR_F32_MAX_W, all three products.
 bool vector_supports(int op, int64_t M, int64_t N, int64_t w, int dtype) {
-  if (op != 2 && op != 3) return false;
-  if (dtype != WM_DTYPE_BF16 && dtype != WM_DTYPE_F16) return false;
+  if (op < 1 || op > 3 || M < 1 || M > (1 << 30) || w < 1) return false;
+  if (dtype == WM_DTYPE_F32) {
+    if (N < 8 || N > 128 || N % 8 != 0 || w > VECTOR_F32_MAX_W) return false;
+    return (op == 1 ? vector_out_lds(w, N) : vector_lds(w, N, dtype)) <= 65536;
+  }
+  if (op == 1 || (dtype != WM_DTYPE_BF16 && dtype != WM_DTYPE_F16)) return false;
   if (N < 16 || N > 128 || N % 16 != 0) return false;
-  return M >= 1 && M <= (1 << 30) && w >= 1 && w <= VECTOR_MAX_W && w % 4 != 0 && vector_lds(w, N) <= 65536;
+  return w <= VECTOR_MAX_W && w % 4 != 0 && vector_lds(w, N, dtype) <= 65536;
 }
 
+bool try_launch_vector_p1(const Problem &p, const View &x, const View &y, const View &c, hipError_t *err) {
+  if (!vector_supports(1, p.M, p.N, p.w, p.dtype)) return false;
+  if (!fast_layout(x, p.dtype) || !fast_layout(y, p.dtype) || c.sc != 1 || c.sr != 2 * p.w + 1) return false;
+  *err = launch_vector_out_f32(p, x, y, c);
+  return true;
+}
+
+template <bool TRANSPOSED>
+bool try_launch_vector_in(const Problem &p, const View &a, const View &y, const View &c, hipError_t *err) {
+  if (!vector_supports(TRANSPOSED ? 3 : 2, p.M, p.N, p.w, p.dtype)) return false;
+  if (!band_contiguous(a, 2 * p.w + 1) || !fast_layout(y, p.dtype) || !fast_layout(c, p.dtype)) return false;
+  *err = p.dtype == WM_DTYPE_BF16  ? launch_vector<bf16_t, TRANSPOSED>(p, a, y, c)
+         : p.dtype == WM_DTYPE_F16 ? launch_vector<f16_t, TRANSPOSED>(p, a, y, c)
+                                   : launch_vector<f32_t, TRANSPOSED>(p, a, y, c);
+  return true;
+}
 bool try_launch_vector_p2(const Problem &p, const View &a, const View &y, const View &c, hipError_t *err) {
-  if (!vector_supports(2, p.M, p.N, p.w, p.dtype)) return false;
-  if (!band_contiguous(a, 2 * p.w + 1) || !fast_layout(y, p.dtype) || !fast_layout(c, p.dtype)) return false;
-  *err = p.dtype == WM_DTYPE_BF16 ? launch_vector<bf16_t, false>(p, a, y, c) : launch_vector<f16_t, false>(p, a, y, c);
-  return true;
+  return try_launch_vector_in<false>(p, a, y, c, err);
 }
-
 bool try_launch_vector_p3(const Problem &p, const View &a, const View &y, const View &c, hipError_t *err) {
-  if (!vector_supports(3, p.M, p.N, p.w, p.dtype)) return false;
-  if (!band_contiguous(a, 2 * p.w + 1) || !fast_layout(y, p.dtype) || !fast_layout(c, p.dtype)) return false;
-  *err = p.dtype == WM_DTYPE_BF16 ? launch_vector<bf16_t, true>(p, a, y, c) : launch_vector<f16_t, true>(p, a, y, c);
-  return true;
+  return try_launch_vector_in<true>(p, a, y, c, err);
 }
 
 }  // namespace wm

@@ -67,7 +67,12 @@ def test_kernel_choice_names():
     assert L.wm_kernel_choice(3, 96, 16384, 64, 7, 1, 1, 0) == b"vector_p3"
     assert L.wm_kernel_choice(1, 96, 16384, 64, 7, 1, 1, 0) == b"narrow_p1"
     assert L.wm_kernel_choice(2, 96, 16384, 64, 7, 2, 1, abi.NO_NARROW_BAND) == b"strided_p2"
-    assert L.wm_kernel_choice(2, 96, 16384, 64, 3, 0, 1, 0) == b"strided_p2"  # float32 below w = 4
+    # float32: all three products on the vector ALU up to w = 10, the float32 MFMA kernels beyond
+    assert L.wm_kernel_choice(2, 96, 16384, 64, 3, 0, 1, 0) == b"vector_p2"
+    assert L.wm_kernel_choice(1, 2, 128, 64, 4, 0, 1, 0) == b"vector_p1"
+    assert L.wm_kernel_choice(3, 96, 16384, 64, 10, 0, 1, 0) == b"vector_p3"
+    assert L.wm_kernel_choice(3, 96, 16384, 64, 11, 0, 1, 0) == b"f32_mfma_p3"
+    assert L.wm_kernel_choice(1, 96, 16384, 64, 8, 0, 1, abi.NO_NARROW_BAND) == b"f32_mfma_p1"
     assert L.wm_kernel_choice(1, 2, 128, 3, 4, 0, 1, 0) == b"strided_p1"  # N not a multiple of 8
     assert L.wm_kernel_choice(1, 2, 128, 64, 4, 2, 0, 0) == b"strided_p1"  # layout not vector friendly
 
