@@ -8,9 +8,10 @@
 // are 2w+1 multiply-adds per output element on operands that are streamed once: far too little
 // arithmetic for the matrix pipe to matter, so each thread simply owns 16 bytes of one output row
 // (8 or 4 consecutive columns) and walks the 2w+1 terms: one LDS read of the band entry (the same
-// address for the threads of a row), one 16-byte LDS read of the Y row piece, 8 packed dot products
-// that each pair the entry with one of the 8 values and a zero with its neighbour (16-bit), or 4
-// FMAs (float32).  The workgroup first copies what it needs into LDS with coalesced 16-byte loads
+// address for the threads of a row), one 16-byte LDS read of the Y row piece, 8 FMAs on the unpacked
+// values (16-bit) or 4 FMAs (float32).  (Packed dot products that pair the entry with one value and
+// a zero with its neighbour need no unpacking but are no faster, LDS reads sharing the bound, and
+// would let an Inf in one column of Y turn the neighbouring output column into NaN.)  The workgroup first copies what it needs into LDS with coalesced 16-byte loads
 // (its band rows as one flat image, the Y rows they reach row-major, zero outside the sequence);
 // the result leaves as 16-byte non-temporal stores, consecutive threads on consecutive pieces of a row.
 // The float32 band-out product  P1  band[i,j] = sum_h X[i,h] Y[i+j-w,h]  gets the same treatment:
@@ -31,18 +32,28 @@ constexpr int VECTOR_MAX_W = WM_VECTOR_MAX_W;
 constexpr int VECTOR_F32_MAX_W = WM_VECTOR_F32_MAX_W;
 typedef float f32x4v __attribute__((ext_vector_type(4)));
 
-// acc + a.lo * y.lo + a.hi * y.hi on packed pairs (v_dot2_f32_bf16 / v_dot2_f32_f16): with the band
-// entry in one half of `a` and zero in the other, one instruction per multiply-add and no unpacking.
+// A 16-bit storage value, and the two values of a dword, as floats.
 template <typename T>
-__device__ __forceinline__ float dot2(uint32_t a, uint32_t y, float acc);
+__device__ __forceinline__ float to_float(uint16_t x);
 template <>
-__device__ __forceinline__ float dot2<bf16_t>(uint32_t a, uint32_t y, float acc) {
-  return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, a), __builtin_bit_cast(bf16x2, y), acc, false);
+__device__ __forceinline__ float to_float<bf16_t>(uint16_t x) {
+  return __builtin_bit_cast(float, (uint32_t)x << 16);
 }
 template <>
-__device__ __forceinline__ float dot2<f16_t>(uint32_t a, uint32_t y, float acc) {
-  typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
-  return __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2, a), __builtin_bit_cast(f16x2, y), acc, false);
+__device__ __forceinline__ float to_float<f16_t>(uint16_t x) {
+  return (float)__builtin_bit_cast(_Float16, x);
+}
+template <typename T>
+__device__ __forceinline__ void unpack2(uint32_t x, float &lo, float &hi);
+template <>
+__device__ __forceinline__ void unpack2<bf16_t>(uint32_t x, float &lo, float &hi) {
+  lo = __builtin_bit_cast(float, x << 16);
+  hi = __builtin_bit_cast(float, x & 0xffff0000u);
+}
+template <>
+__device__ __forceinline__ void unpack2<f16_t>(uint32_t x, float &lo, float &hi) {
+  lo = (float)__builtin_bit_cast(_Float16, (uint16_t)x);
+  hi = (float)__builtin_bit_cast(_Float16, (uint16_t)(x >> 16));
 }
 
 // Storage element of a type tag, and the float32 "tag".
@@ -133,11 +144,13 @@ __global__ __launch_bounds__(kThreads) void vector_band_in_kernel(const typename
     for (int t = t_lo; t <= t_hi; ++t) {
       const u32x4 y = *reinterpret_cast<const u32x4 *>(yp);
       if constexpr (sizeof(E) == 2) {
-        const uint32_t a_lo = *ap, a_hi = a_lo << 16;  // (a, 0) and (0, a)
+        const float a = to_float<T>(*ap);
 #pragma unroll
         for (int d = 0; d < 4; ++d) {
-          acc[2 * d] = dot2<T>(a_lo, y[d], acc[2 * d]);
-          acc[2 * d + 1] = dot2<T>(a_hi, y[d], acc[2 * d + 1]);
+          float lo, hi;
+          unpack2<T>(y[d], lo, hi);
+          acc[2 * d] = __builtin_fmaf(a, lo, acc[2 * d]);
+          acc[2 * d + 1] = __builtin_fmaf(a, hi, acc[2 * d + 1]);
         }
       } else {
         const float a = *ap;
