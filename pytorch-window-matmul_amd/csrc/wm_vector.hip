@@ -8,12 +8,13 @@
 // are 2w+1 multiply-adds per output element on operands that are streamed once: far too little
 // arithmetic for the matrix pipe to matter, so each thread simply owns 16 bytes of one output row
 // (8 or 4 consecutive columns) and walks the 2w+1 terms: one LDS read of the band entry (the same
-// address for the threads of a row), one 16-byte LDS read of the Y row piece, 8 FMAs on the unpacked
-// values (16-bit) or 4 FMAs (float32).  (Packed dot products that pair the entry with one value and
-// a zero with its neighbour need no unpacking but are no faster, LDS reads sharing the bound, and
-// would let an Inf in one column of Y turn the neighbouring output column into NaN.)  The workgroup first copies what it needs into LDS with coalesced 16-byte loads
-// (its band rows as one flat image, the Y rows they reach row-major, zero outside the sequence);
-// the result leaves as 16-byte non-temporal stores, consecutive threads on consecutive pieces of a row.
+// address for the threads of a row), one 16-byte LDS read of the Y row piece, 8 FMAs on the
+// unpacked values (16-bit) or 4 FMAs (float32).  (Packed dot products that pair the entry with one
+// value and a zero with its neighbour need no unpacking but are no faster, LDS reads sharing the
+// bound, and would let an Inf in one column of Y turn the neighbouring output column into NaN.)
+// The workgroup first copies what it needs into LDS with coalesced 16-byte loads (its band rows
+// as one flat image, the Y rows they reach row-major, zero outside the sequence); the result
+// leaves as 16-byte non-temporal stores, consecutive threads on consecutive pieces of a row.
 // The float32 band-out product  P1  band[i,j] = sum_h X[i,h] Y[i+j-w,h]  gets the same treatment:
 // X and Y rows in LDS, one thread per band entry, consecutive threads on consecutive entries of
 // the flat band.  One barrier per workgroup; no atomics.
