@@ -26,15 +26,15 @@ int to_status(hipError_t err) {
 typedef bool (*mfma_fn)(const Problem &, const View &, const View &, const View &, hipError_t *);
 typedef hipError_t (*strided_fn)(const Problem &, const View &, const View &, const View &);
 
-// Kernel choice per primitive: narrow-band family (MFMA, or vector ALU for the windows that
-// leaves out), else wide-band MFMA family (all 16-bit storage), else the float32 MFMA family,
-// else strided.
+// Kernel choice per primitive: vector-ALU kernels (the narrowest windows), else narrow-band MFMA
+// family, else wide-band MFMA family (all 16-bit storage except the float32 vector kernels), else
+// the float32 MFMA family, else strided.
 int run_primitive(mfma_fn narrow, mfma_fn vector, mfma_fn fast, mfma_fn f32, strided_fn slow, const Problem &p,
                   const View &a, const View &y, const View &c) {
   hipError_t err = hipSuccess;
   if (!(p.flags & WM_FLAG_FORCE_STRIDED)) {
-    if (narrow && !(p.flags & WM_FLAG_NO_NARROW_BAND) && narrow(p, a, y, c, &err)) return to_status(err);
     if (vector && !(p.flags & WM_FLAG_NO_NARROW_BAND) && vector(p, a, y, c, &err)) return to_status(err);
+    if (narrow && !(p.flags & WM_FLAG_NO_NARROW_BAND) && narrow(p, a, y, c, &err)) return to_status(err);
     if (fast(p, a, y, c, &err)) return to_status(err);
     if (f32(p, a, y, c, &err)) return to_status(err);
   }
@@ -188,12 +188,12 @@ const char *wm_kernel_choice(int op, int64_t B, int64_t M, int64_t N, int64_t w,
                              unsigned flags) {
   if (op < 1 || op > 3) return "invalid";
   if (!(flags & WM_FLAG_FORCE_STRIDED) && fast) {
-    if (!(flags & WM_FLAG_NO_NARROW_BAND) && small_supports(op, M, N, w, dtype)) {
-      static const char *names[] = {"narrow_p1", "narrow_p2", "narrow_p3"};
-      return names[op - 1];
-    }
     if (!(flags & WM_FLAG_NO_NARROW_BAND) && vector_supports(op, M, N, w, dtype)) {
       static const char *names[] = {"vector_p1", "vector_p2", "vector_p3"};
+      return names[op - 1];
+    }
+    if (!(flags & WM_FLAG_NO_NARROW_BAND) && small_supports(op, M, N, w, dtype)) {
+      static const char *names[] = {"narrow_p1", "narrow_p2", "narrow_p3"};
       return names[op - 1];
     }
     if (mfma_supports(op, B, M, N, w, dtype)) {

@@ -15,9 +15,9 @@
 // The workgroup first copies what it needs into LDS with coalesced 16-byte loads (its band rows
 // as one flat image, the Y rows they reach row-major, zero outside the sequence); the result
 // leaves as 16-byte non-temporal stores, consecutive threads on consecutive pieces of a row.
-// The float32 band-out product  P1  band[i,j] = sum_h X[i,h] Y[i+j-w,h]  gets the same treatment:
-// X and Y rows in LDS, one thread per band entry, consecutive threads on consecutive entries of
-// the flat band.  One barrier per workgroup; no atomics.
+// The band-out product  P1  band[i,j] = sum_h X[i,h] Y[i+j-w,h]  gets the same treatment (float32 up
+// to w = 10; 16-bit only for w <= 2, beyond that the narrow-band MFMA kernel is faster): X and Y rows
+// in LDS, one thread per band entry, consecutive threads on consecutive entries of the flat band.  One barrier per workgroup; no atomics.
 #include "wm_mfma_common.hpp"
 
 namespace wm {
@@ -31,6 +31,10 @@ constexpr int VECTOR_MAX_W = WM_VECTOR_MAX_W;
 #define WM_VECTOR_F32_MAX_W 10
 #endif
 constexpr int VECTOR_F32_MAX_W = WM_VECTOR_F32_MAX_W;
+#ifndef WM_VECTOR_OUT_MAX_W
+#define WM_VECTOR_OUT_MAX_W 2
+#endif
+constexpr int VECTOR_OUT_MAX_W = WM_VECTOR_OUT_MAX_W;  // 16-bit band-out product
 typedef float f32x4v __attribute__((ext_vector_type(4)));
 
 // A 16-bit storage value, and the two values of a dword, as floats.
@@ -174,19 +178,34 @@ __global__ __launch_bounds__(kThreads) void vector_band_in_kernel(const typename
   }
 }
 
-// float32 P1: band[b,i,j] = sum_h X[b,i,h] Y[b,i+j-w,h]  (+0.0 where i+j-w is outside the sequence).
+// x.lo * y.lo + x.hi * y.hi + acc on packed pairs of 16-bit values (v_dot2_f32_bf16 / v_dot2_f32_f16).
+template <typename T>
+__device__ __forceinline__ float dot2(uint32_t x, uint32_t y, float acc);
+template <>
+__device__ __forceinline__ float dot2<bf16_t>(uint32_t x, uint32_t y, float acc) {
+  return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, x), __builtin_bit_cast(bf16x2, y), acc, false);
+}
+template <>
+__device__ __forceinline__ float dot2<f16_t>(uint32_t x, uint32_t y, float acc) {
+  typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+  return __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2, x), __builtin_bit_cast(f16x2, y), acc, false);
+}
+
+// P1: band[b,i,j] = sum_h X[b,i,h] Y[b,i+j-w,h]  (+0.0 where i+j-w is outside the sequence).
 // One thread per band entry, consecutive threads on consecutive entries of the flat band.
-template <int NK>  // N = 8 NK
-__global__ __launch_bounds__(kThreads) void vector_band_out_f32_kernel(const float *__restrict__ X,
-                                                                       const float *__restrict__ Y,
-                                                                       float *__restrict__ C, int B, int M, int w,
-                                                                       int nblk, int vrows, int64_t xsb, int64_t xsr,
-                                                                       int64_t ysb, int64_t ysr, int64_t csb) {
-  constexpr int N = 8 * NK, NCG = N / 4;
-  constexpr int SX = N + 4;  // rows 16 bytes apart mod 128
+template <typename T, int NK>  // 2 NK 16-byte pieces per row: N = 16 NK (16-bit) or 8 NK (float32)
+__global__ __launch_bounds__(kThreads) void vector_band_out_kernel(const typename Elem<T>::type *__restrict__ X,
+                                                                   const typename Elem<T>::type *__restrict__ Y,
+                                                                   typename Elem<T>::type *__restrict__ C, int B,
+                                                                   int M, int w, int nblk, int vrows, int64_t xsb,
+                                                                   int64_t xsr, int64_t ysb, int64_t ysr, int64_t csb) {
+  typedef typename Elem<T>::type E;
+  constexpr int VEC = 16 / sizeof(E);
+  constexpr int NCG = 2 * NK, N = NCG * VEC;
+  constexpr int SX = N + VEC;  // rows 16 bytes apart mod 128
   extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
-  float *ximg = reinterpret_cast<float *>(lds_raw);  // rows i0 .. i0 + rows
-  float *yimg = ximg + vrows * SX;                   // rows i0 - w .. i0 + rows + w, zero outside the sequence
+  E *ximg = reinterpret_cast<E *>(lds_raw);  // rows i0 .. i0 + rows
+  E *yimg = ximg + vrows * SX;               // rows i0 - w .. i0 + rows + w, zero outside the sequence
 
   int b, blk;
   if (!decode_block(nblk, B, &b, &blk)) return;
@@ -194,7 +213,7 @@ __global__ __launch_bounds__(kThreads) void vector_band_out_f32_kernel(const flo
   const int W = 2 * w + 1;
   const int i0 = blk * vrows;
   const int rows = min(vrows, M - i0);
-  const float *Xb = X + (int64_t)b * xsb, *Yb = Y + (int64_t)b * ysb;
+  const E *Xb = X + (int64_t)b * xsb, *Yb = Y + (int64_t)b * ysb;
   const int xchunks = rows * NCG, ychunks = (rows + 2 * w) * NCG;
   constexpr int BATCH = 8;
   for (int base = 0; base < xchunks + ychunks; base += BATCH * kThreads) {
@@ -204,7 +223,7 @@ __global__ __launch_bounds__(kThreads) void vector_band_out_f32_kernel(const flo
       const int q = base + s * kThreads + tid;
       const int qy = q - xchunks;
       const int xr = q / NCG, xg = q - xr * NCG, yr = qy / NCG, yg = qy - yr * NCG, c = i0 - w + yr;
-      const float *src = q < xchunks ? Xb + (int64_t)(i0 + xr) * xsr + 4 * xg : Yb + (int64_t)c * ysr + 4 * yg;
+      const E *src = q < xchunks ? Xb + (int64_t)(i0 + xr) * xsr + VEC * xg : Yb + (int64_t)c * ysr + VEC * yg;
       const bool ok = q < xchunks || (q < xchunks + ychunks && c >= 0 && c < M);
       reg[s] = *reinterpret_cast<const u32x4 *>(ok ? src : X);
     }
@@ -214,38 +233,50 @@ __global__ __launch_bounds__(kThreads) void vector_band_out_f32_kernel(const flo
       const int qy = q - xchunks;
       const int xr = q / NCG, xg = q - xr * NCG, yr = qy / NCG, yg = qy - yr * NCG, c = i0 - w + yr;
       if (q < xchunks)
-        *reinterpret_cast<u32x4 *>(ximg + xr * SX + 4 * xg) = reg[s];
+        *reinterpret_cast<u32x4 *>(ximg + xr * SX + VEC * xg) = reg[s];
       else if (q < xchunks + ychunks)
-        *reinterpret_cast<u32x4 *>(yimg + yr * SX + 4 * yg) = mask_row_chunk(reg[s], (c >= 0) & (c < M));
+        *reinterpret_cast<u32x4 *>(yimg + yr * SX + VEC * yg) = mask_row_chunk(reg[s], (c >= 0) & (c < M));
     }
   }
   __syncthreads();
 
-  float *Cb = C + (int64_t)b * csb + (int64_t)i0 * W;
+  E *Cb = C + (int64_t)b * csb + (int64_t)i0 * W;
   for (int item = tid; item < rows * W; item += kThreads) {
     const int r = item / W, j = item - r * W;
     const int c = i0 + r + j - w;
-    const float *xp = ximg + r * SX, *yp = yimg + (r + j) * SX;
+    const E *xp = ximg + r * SX, *yp = yimg + (r + j) * SX;
     float acc[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int g = 0; g < NCG; ++g) {
-      const f32x4v x = *reinterpret_cast<const f32x4v *>(xp + 4 * g), y = *reinterpret_cast<const f32x4v *>(yp + 4 * g);
+      const u32x4 x = *reinterpret_cast<const u32x4 *>(xp + VEC * g), y = *reinterpret_cast<const u32x4 *>(yp + VEC * g);
+      if constexpr (sizeof(E) == 2) {
 #pragma unroll
-      for (int e = 0; e < 4; ++e) acc[e] = __builtin_fmaf(x[e], y[e], acc[e]);
+        for (int e = 0; e < 4; ++e) acc[e] = dot2<T>(x[e], y[e], acc[e]);
+      } else {
+        const f32x4v xf = __builtin_bit_cast(f32x4v, x), yf = __builtin_bit_cast(f32x4v, y);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) acc[e] = __builtin_fmaf(xf[e], yf[e], acc[e]);
+      }
     }
-    const float sum = (acc[0] + acc[1]) + (acc[2] + acc[3]);
-    Cb[item] = (c >= 0 && c < M) ? sum : 0.f;  // +0.0 outside the sequence, whatever X holds
+    const float sum = (c >= 0 && c < M) ? (acc[0] + acc[1]) + (acc[2] + acc[3]) : 0.f;  // +0.0 outside the sequence
+    if constexpr (sizeof(E) == 2)
+      Cb[item] = (uint16_t)Mma<T>::pack2(sum, 0.f);
+    else
+      Cb[item] = sum;
   }
 }
 
 // Output rows per workgroup: as many as keep the LDS images of the widest supported window small.
 int vector_rows(int64_t N, int dtype) { return dtype == WM_DTYPE_F32 && N > 64 ? 64 : 128; }
-int vector_out_rows(int64_t N) { return N > 64 ? 32 : 64; }
+int vector_out_rows(int64_t N, int dtype) { return dtype == WM_DTYPE_F32 ? (N > 64 ? 32 : 64) : 128; }
 size_t vector_lds(int64_t w, int64_t N, int dtype) {
   const int64_t W = 2 * w + 1, vec = dtype == WM_DTYPE_F32 ? 4 : 8, rows = vector_rows(N, dtype);
   return (size_t)((((rows + 2 * w) * W + 3 * vec - 1) & ~(vec - 1)) + (rows + 2 * w) * (N + vec)) * (16 / vec);
 }
-size_t vector_out_lds(int64_t w, int64_t N) { return (size_t)((2 * vector_out_rows(N) + 2 * w) * (N + 4)) * 4; }
+size_t vector_out_lds(int64_t w, int64_t N, int dtype) {
+  const int64_t vec = dtype == WM_DTYPE_F32 ? 4 : 8;
+  return (size_t)((2 * vector_out_rows(N, dtype) + 2 * w) * (N + vec)) * (16 / vec);
+}
 
 unsigned vector_grid(int64_t B, int64_t nblk) { return (unsigned)(((B + 7) / 8) * 8 * nblk); }
 
@@ -272,18 +303,21 @@ hipError_t launch_vector(const Problem &p, const View &a, const View &y, const V
   return hipGetLastError();
 }
 
-hipError_t launch_vector_out_f32(const Problem &p, const View &x, const View &y, const View &c) {
-  const int vrows = vector_out_rows(p.N);
+template <typename T>
+hipError_t launch_vector_out(const Problem &p, const View &x, const View &y, const View &c) {
+  typedef typename Elem<T>::type E;
+  const int vrows = vector_out_rows(p.N, p.dtype);
   const int nblk = (int)((p.M + vrows - 1) / vrows);
   const dim3 grid(vector_grid(p.B, nblk)), block(kThreads);
-  const size_t lds = vector_out_lds(p.w, p.N);
+  const size_t lds = vector_out_lds(p.w, p.N, p.dtype);
+  const int pieces = (int)(p.N * sizeof(E) / 16);
 #define WM_VOUT(NK)                                                                                             \
   case NK:                                                                                                      \
-    hipLaunchKernelGGL((vector_band_out_f32_kernel<NK>), grid, block, lds, p.stream, (const float *)x.data,     \
-                       (const float *)y.data, (float *)c.data, (int)p.B, (int)p.M, (int)p.w, nblk, vrows, x.sb,  \
-                       x.sr, y.sb, y.sr, c.sb);                                                                       \
+    hipLaunchKernelGGL((vector_band_out_kernel<T, NK>), grid, block, lds, p.stream, (const E *)x.data,          \
+                       (const E *)y.data, (E *)c.data, (int)p.B, (int)p.M, (int)p.w, nblk, vrows, x.sb, x.sr,   \
+                       y.sb, y.sr, c.sb);                                                                       \
     break;
-  switch (p.N / 8) {
+  switch (pieces / 2) {
     WM_VOUT(1) WM_VOUT(2) WM_VOUT(3) WM_VOUT(4) WM_VOUT(5) WM_VOUT(6) WM_VOUT(7) WM_VOUT(8)
     WM_VOUT(9) WM_VOUT(10) WM_VOUT(11) WM_VOUT(12) WM_VOUT(13) WM_VOUT(14) WM_VOUT(15) WM_VOUT(16)
     default: return hipErrorInvalidValue;
@@ -296,24 +330,28 @@ bool band_contiguous(const View &v, int64_t W) { return v.sc == 1 && v.sr == W &
 
 }  // namespace
 
-// 16-bit: the windows the narrow-band MFMA kernels do not take (w % 4 != 0) below the wide-band
-// family's range (band-in products only; the narrow-band band-out kernel takes every w).
+// 16-bit: band-in products at the windows the narrow-band MFMA kernels do not take (w % 4 != 0) below
+// the wide-band family's range; the band-out product at w <= 2 (measured faster than the narrow-band
+// MFMA kernel there: 79-94 us against 96-98 us at B96 M16384 N64).
 // float32: every window up to VECTOR_F32_MAX_W, all three products.
 bool vector_supports(int op, int64_t M, int64_t N, int64_t w, int dtype) {
   if (op < 1 || op > 3 || M < 1 || M > (1 << 30) || w < 1) return false;
   if (dtype == WM_DTYPE_F32) {
     if (N < 8 || N > 128 || N % 8 != 0 || w > VECTOR_F32_MAX_W) return false;
-    return (op == 1 ? vector_out_lds(w, N) : vector_lds(w, N, dtype)) <= 65536;
+    return (op == 1 ? vector_out_lds(w, N, dtype) : vector_lds(w, N, dtype)) <= 65536;
   }
-  if (op == 1 || (dtype != WM_DTYPE_BF16 && dtype != WM_DTYPE_F16)) return false;
+  if (dtype != WM_DTYPE_BF16 && dtype != WM_DTYPE_F16) return false;
   if (N < 16 || N > 128 || N % 16 != 0) return false;
+  if (op == 1) return w <= VECTOR_OUT_MAX_W && vector_out_lds(w, N, dtype) <= 65536;
   return w <= VECTOR_MAX_W && w % 4 != 0 && vector_lds(w, N, dtype) <= 65536;
 }
 
 bool try_launch_vector_p1(const Problem &p, const View &x, const View &y, const View &c, hipError_t *err) {
   if (!vector_supports(1, p.M, p.N, p.w, p.dtype)) return false;
   if (!fast_layout(x, p.dtype) || !fast_layout(y, p.dtype) || c.sc != 1 || c.sr != 2 * p.w + 1) return false;
-  *err = launch_vector_out_f32(p, x, y, c);
+  *err = p.dtype == WM_DTYPE_BF16  ? launch_vector_out<bf16_t>(p, x, y, c)
+         : p.dtype == WM_DTYPE_F16 ? launch_vector_out<f16_t>(p, x, y, c)
+                                   : launch_vector_out<f32_t>(p, x, y, c);
   return true;
 }
 
