@@ -133,39 +133,31 @@ __global__ __launch_bounds__(kThreads) void vector_band_in_kernel(const typename
   }
   __syncthreads();
 
-  for (int item = tid; item < orows * NCG; item += kThreads) {
-    const int r = item / NCG, hg = item - r * NCG;
-    const int o = o0 + r;  // output row
-    float acc[VEC];
+  // A thread owns one 16-byte piece of two consecutive output rows o, o + 1: they share all but one of
+  // their Y rows, so every Y piece is read (and unpacked) once for both.  Pair term u = 0 .. 2w+1 is the
+  // Y row o - w + u (image row r + u); it is term u of row o (u <= 2w) and term u - 1 of row o + 1 (u >= 1).
+  auto entry = [&](const E *p) -> float {
+    if constexpr (sizeof(E) == 2)
+      return to_float<T>(*p);
+    else
+      return *p;
+  };
+  auto add_piece = [&](float a, const u32x4 &y, float(&acc)[VEC]) {
+    if constexpr (sizeof(E) == 2) {
 #pragma unroll
-    for (int e = 0; e < VEC; ++e) acc[e] = 0.f;
-    // term t = 0 .. 2w: the Y row is o - w + t (image row r + t) in both products
-    const int t_lo = max(0, w - o), t_hi = min(2 * w, M - 1 - o + w);  // Y rows inside the sequence
-    const E *yp = yimg + (r + t_lo) * SY + VEC * hg;
-    // P2: band entry (o, t) -> image index (o - a0) W + t, next term +1.
-    // P3: band entry (o - w + t, 2w - t) -> image index (o - w + t - a0) W + 2w - t, next term +W - 1.
-    const E *ap = aimg + delta + (TRANSPOSED ? (o - w + t_lo - a0) * W + 2 * w - t_lo : (o - a0) * W + t_lo);
-    const int a_step = TRANSPOSED ? W - 1 : 1;
-    for (int t = t_lo; t <= t_hi; ++t) {
-      const u32x4 y = *reinterpret_cast<const u32x4 *>(yp);
-      if constexpr (sizeof(E) == 2) {
-        const float a = to_float<T>(*ap);
-#pragma unroll
-        for (int d = 0; d < 4; ++d) {
-          float lo, hi;
-          unpack2<T>(y[d], lo, hi);
-          acc[2 * d] = __builtin_fmaf(a, lo, acc[2 * d]);
-          acc[2 * d + 1] = __builtin_fmaf(a, hi, acc[2 * d + 1]);
-        }
-      } else {
-        const float a = *ap;
-        const f32x4v yf = __builtin_bit_cast(f32x4v, y);  // (a bit cast of one element y[d] reads element 0)
-#pragma unroll
-        for (int d = 0; d < 4; ++d) acc[d] = __builtin_fmaf(a, yf[d], acc[d]);
+      for (int d = 0; d < 4; ++d) {
+        float lo, hi;
+        unpack2<T>(y[d], lo, hi);
+        acc[2 * d] = __builtin_fmaf(a, lo, acc[2 * d]);
+        acc[2 * d + 1] = __builtin_fmaf(a, hi, acc[2 * d + 1]);
       }
-      ap += a_step;
-      yp += SY;
+    } else {
+      const f32x4v yf = __builtin_bit_cast(f32x4v, y);  // (a bit cast of one element y[d] reads element 0)
+#pragma unroll
+      for (int d = 0; d < 4; ++d) acc[d] = __builtin_fmaf(a, yf[d], acc[d]);
     }
+  };
+  auto store_piece = [&](const float(&acc)[VEC], int o, int hg) {
     u32x4 out;
     if constexpr (sizeof(E) == 2) {
       out = u32x4{Mma<T>::pack2(acc[0], acc[1]), Mma<T>::pack2(acc[2], acc[3]), Mma<T>::pack2(acc[4], acc[5]),
@@ -175,6 +167,36 @@ __global__ __launch_bounds__(kThreads) void vector_band_in_kernel(const typename
                   __builtin_bit_cast(uint32_t, acc[2]), __builtin_bit_cast(uint32_t, acc[3])};
     }
     __builtin_nontemporal_store(out, reinterpret_cast<u32x4 *>(C + (int64_t)b * csb + (int64_t)o * csr + VEC * hg));
+  };
+  const int npairs = (orows + 1) >> 1;
+  for (int item = tid; item < npairs * NCG; item += kThreads) {
+    const int pr = item / NCG, hg = item - pr * NCG;
+    const int r = 2 * pr, o = o0 + r;  // first row of the pair
+    const bool has_b = r + 1 < orows;
+    float acc_a[VEC], acc_b[VEC];
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) acc_a[e] = 0.f, acc_b[e] = 0.f;
+    const int u_lo = max(0, w - o), u_hi = min(2 * w + 1, M - 1 - o + w);  // Y rows inside the sequence
+    // band entries of pair term u, as image indices:
+    //   P2: row o: (o - a0) W + u;                 row o + 1: (o + 1 - a0) W + u - 1;   next term +1
+    //   P3: row o: (o - w + u - a0) W + 2w - u;    row o + 1: the entry right of it;    next term +W - 1
+    const int a_step = TRANSPOSED ? W - 1 : 1;
+    const int u1 = max(u_lo, 1), u2 = min(u_hi, 2 * w);  // terms that belong to both rows
+    const E *pa = aimg + delta + (TRANSPOSED ? (o - w + u1 - a0) * W + 2 * w - u1 : (o - a0) * W + u1);
+    const E *pb = !has_b ? pa : TRANSPOSED ? pa + 1 : pa + W - 1;
+    const E *yp = yimg + (r + u1) * SY + VEC * hg;
+    if (u_lo == 0)  // Y row o - w: first term of row o only
+      add_piece(entry(pa - a_step), *reinterpret_cast<const u32x4 *>(yp - SY), acc_a);
+    for (int u = u1; u <= u2; ++u) {
+      const u32x4 y = *reinterpret_cast<const u32x4 *>(yp);
+      add_piece(entry(pa), y, acc_a);
+      add_piece(entry(pb), y, acc_b);
+      pa += a_step, pb += a_step, yp += SY;
+    }
+    if (u_hi == 2 * w + 1 && has_b)  // Y row o + 1 + w: last term of row o + 1 only
+      add_piece(entry(pb), *reinterpret_cast<const u32x4 *>(yp), acc_b);
+    store_piece(acc_a, o, hg);
+    if (has_b) store_piece(acc_b, o + 1, hg);
   }
 }
 
