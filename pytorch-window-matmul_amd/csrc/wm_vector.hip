@@ -16,7 +16,7 @@
 // as one flat image, the Y rows they reach row-major, zero outside the sequence); the result
 // leaves as 16-byte non-temporal stores, consecutive threads on consecutive pieces of a row.
 // The band-out product  P1  band[i,j] = sum_h X[i,h] Y[i+j-w,h]  gets the same treatment (float32 up
-// to w = 10; 16-bit only for w <= 2, beyond that the narrow-band MFMA kernel is faster): X and Y rows
+// to w = 14; 16-bit only for w <= 2, beyond that the narrow-band MFMA kernel is faster): X and Y rows
 // in LDS, one thread per band entry, consecutive threads on consecutive entries of the flat band.  One barrier per workgroup; no atomics.
 #include "wm_mfma_common.hpp"
 
@@ -24,11 +24,11 @@ namespace wm {
 namespace {
 
 #ifndef WM_VECTOR_MAX_W
-#define WM_VECTOR_MAX_W 7
+#define WM_VECTOR_MAX_W 11
 #endif
 constexpr int VECTOR_MAX_W = WM_VECTOR_MAX_W;
 #ifndef WM_VECTOR_F32_MAX_W
-#define WM_VECTOR_F32_MAX_W 10
+#define WM_VECTOR_F32_MAX_W 14
 #endif
 constexpr int VECTOR_F32_MAX_W = WM_VECTOR_F32_MAX_W;
 #ifndef WM_VECTOR_OUT_MAX_W
@@ -352,8 +352,8 @@ bool band_contiguous(const View &v, int64_t W) { return v.sc == 1 && v.sr == W &
 
 }  // namespace
 
-// 16-bit: band-in products at the windows the narrow-band MFMA kernels do not take (w % 4 != 0) below
-// the wide-band family's range; the band-out product at w <= 2 (measured faster than the narrow-band
+// 16-bit: band-in products at the windows the narrow-band MFMA kernels do not take (w % 4 != 0) up to
+// w = 11, where the wide-band MFMA kernels catch up; the band-out product at w <= 2 (measured faster than the narrow-band
 // MFMA kernel there: 79-94 us against 96-98 us at B96 M16384 N64).
 // float32: every window up to VECTOR_F32_MAX_W, all three products.
 bool vector_supports(int op, int64_t M, int64_t N, int64_t w, int dtype) {

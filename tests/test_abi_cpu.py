@@ -56,24 +56,26 @@ def test_kernel_choice_names():
     assert L.wm_kernel_choice(2, 96, 4096, 64, 256, 2, 1, 0) == b"mfma_p2"
     assert L.wm_kernel_choice(1, 96, 16384, 64, 8, 2, 1, 0) == b"narrow_p1"
     assert L.wm_kernel_choice(2, 96, 16384, 64, 8, 1, 1, 0) == b"narrow_p2"
-    assert L.wm_kernel_choice(2, 96, 16384, 64, 9, 2, 1, 0) == b"mfma_p2"
+    assert L.wm_kernel_choice(2, 96, 16384, 64, 9, 2, 1, 0) == b"vector_p2"
+    assert L.wm_kernel_choice(2, 96, 16384, 64, 13, 2, 1, 0) == b"mfma_p2"
     assert L.wm_kernel_choice(3, 96, 16384, 64, 8, 2, 1, 0) == b"narrow_p3"
-    assert L.wm_kernel_choice(3, 96, 16384, 64, 10, 2, 1, 0) == b"mfma_p3"
+    assert L.wm_kernel_choice(3, 96, 16384, 64, 10, 2, 1, 0) == b"vector_p3"
+    assert L.wm_kernel_choice(3, 96, 16384, 64, 14, 2, 1, 0) == b"mfma_p3"
     assert L.wm_kernel_choice(2, 96, 16384, 64, 32, 2, 1, 0) == b"narrow_p2"  # 32 rows per wave still fit LDS
     assert L.wm_kernel_choice(3, 96, 16384, 128, 32, 2, 1, 0) == b"mfma_p3"   # images beyond 64 KB of LDS
     assert L.wm_kernel_choice(1, 96, 16384, 64, 8, 2, 1, abi.NO_NARROW_BAND) == b"mfma_p1"
-    # very narrow windows the MFMA families leave out (w % 4 != 0, w < 8): vector-ALU band-in kernels
+    # narrow windows the narrow-band MFMA kernels leave out (w % 4 != 0, w <= 11): vector-ALU band-in kernels
     assert L.wm_kernel_choice(2, 96, 16384, 64, 1, 2, 1, 0) == b"vector_p2"
     assert L.wm_kernel_choice(3, 96, 16384, 64, 7, 1, 1, 0) == b"vector_p3"
     assert L.wm_kernel_choice(1, 96, 16384, 64, 7, 1, 1, 0) == b"narrow_p1"
     assert L.wm_kernel_choice(1, 96, 16384, 64, 2, 2, 1, 0) == b"vector_p1"
     assert L.wm_kernel_choice(1, 96, 16384, 64, 3, 2, 1, 0) == b"narrow_p1"
     assert L.wm_kernel_choice(2, 96, 16384, 64, 7, 2, 1, abi.NO_NARROW_BAND) == b"strided_p2"
-    # float32: all three products on the vector ALU up to w = 10, the float32 MFMA kernels beyond
+    # float32: all three products on the vector ALU up to w = 14, the float32 MFMA kernels beyond
     assert L.wm_kernel_choice(2, 96, 16384, 64, 3, 0, 1, 0) == b"vector_p2"
     assert L.wm_kernel_choice(1, 2, 128, 64, 4, 0, 1, 0) == b"vector_p1"
-    assert L.wm_kernel_choice(3, 96, 16384, 64, 10, 0, 1, 0) == b"vector_p3"
-    assert L.wm_kernel_choice(3, 96, 16384, 64, 11, 0, 1, 0) == b"f32_mfma_p3"
+    assert L.wm_kernel_choice(3, 96, 16384, 64, 14, 0, 1, 0) == b"vector_p3"
+    assert L.wm_kernel_choice(3, 96, 16384, 64, 15, 0, 1, 0) == b"f32_mfma_p3"
     assert L.wm_kernel_choice(1, 96, 16384, 64, 8, 0, 1, abi.NO_NARROW_BAND) == b"f32_mfma_p1"
     assert L.wm_kernel_choice(1, 2, 128, 3, 4, 0, 1, 0) == b"strided_p1"  # N not a multiple of 8
     assert L.wm_kernel_choice(1, 2, 128, 64, 4, 2, 0, 0) == b"strided_p1"  # layout not vector friendly
