@@ -201,3 +201,28 @@ def test_gradient_of_one_input_only(device, which):
     assert (v.grad if first else a.grad) is None
     one = native.unwindow_matmul_backward(a0, v0, w, 2 * out, need_src=first, need_other=not first)
     assert one[1 if first else 0] is None and one[0 if first else 1] is not None
+
+
+def test_ops_follow_the_current_stream(device):
+    """Launches go to torch's current stream: the same chain on two side streams at once, each ordered
+    only by its own stream, gives the result of the default stream (no hidden use of stream 0)."""
+    from window_matmul import unwindow_matmul, window_matmul
+
+    B, M, N, w = 4, 1024, 64, 24
+    q, k, v = (seeded((B, M, N), s, torch.bfloat16).to(device) for s in (41, 42, 43))
+
+    def chain(x):
+        att = window_matmul(x, k.transpose(-1, -2), w)
+        return unwindow_matmul(torch.softmax(att.float() * 0.125, -1).to(att.dtype), v, w)
+
+    want = chain(q)
+    want2 = chain(q + 1)
+    torch.cuda.synchronize()
+    s1, s2 = torch.cuda.Stream(), torch.cuda.Stream()
+    with torch.cuda.stream(s1):
+        got = chain(q)
+    with torch.cuda.stream(s2):
+        got2 = chain(q + 1)
+    s1.synchronize()
+    s2.synchronize()
+    assert torch.equal(got, want) and torch.equal(got2, want2)
