@@ -19,7 +19,11 @@ from .band_softmax import band_softmax
 from .window_matmul import unwindow_matmul, window_matmul
 
 
-_CHAIN_MAX_W = 12  # widest window for which a training step is faster through the separate ops
+def _chain_is_faster(window_size: int) -> bool:
+    """Windows at which a training step is faster through the separate ops than through the fused
+    kernels (measured at B96 M16384 N64 bf16: 0.49-0.60 ms against 0.67-0.75 ms at w <= 8 and at
+    w = 12; the fused kernels win at w = 9, 10, 11 and from 13 on, 0.67 ms against 0.69-1.0 ms)."""
+    return window_size <= 8 or window_size == 12
 
 
 class WindowAttentionFunc(torch.autograd.Function):
@@ -62,10 +66,9 @@ def window_attention(query: torch.Tensor, key: torch.Tensor, value: torch.Tensor
         return torch.softmax(score, -1) * value
     q, k, v = (t.reshape(-1, t.shape[-2], t.shape[-1]) for t in (query, key, value))
     # With a very narrow band the recomputing backward of the fused kernels costs more than the
-    # band it avoids writing (measured at N = 64: 0.80 ms fused against 0.57 ms for the separate ops
-    # at w = 8, break-even near w = 16), so training there goes through the separate ops.
+    # band it avoids writing, so training there goes through the separate ops.
     training = torch.is_grad_enabled() and any(t.requires_grad for t in (q, k, v))
-    if _native.window_attention_supported(q, window_size, scale) and not (training and window_size <= _CHAIN_MAX_W):
+    if _native.window_attention_supported(q, window_size, scale) and not (training and _chain_is_faster(window_size)):
         out = WindowAttentionFunc.apply(q, k, v, window_size, scale, bool(mask_out_of_range))
     else:
         att = window_matmul(q, k.transpose(-1, -2), window_size)
