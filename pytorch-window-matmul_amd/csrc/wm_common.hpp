@@ -44,13 +44,13 @@ hipError_t launch_strided_p3(const Problem &p, const View &a, const View &y, con
 bool try_launch_mfma_p1(const Problem &p, const View &x, const View &y, const View &c, hipError_t *err);
 bool try_launch_mfma_p2(const Problem &p, const View &a, const View &y, const View &c, hipError_t *err);
 bool try_launch_mfma_p3(const Problem &p, const View &a, const View &y, const View &c, hipError_t *err);
-// Narrow-band family (w <= 32): P1 for any such w, P2 and P3 for w % 4 == 0.
+// Narrow-band family (w <= 32; P2 and P3 while their LDS images fit 64 KB).
 bool try_launch_small_p1(const Problem &p, const View &x, const View &y, const View &c, hipError_t *err);
 bool try_launch_small_p2(const Problem &p, const View &a, const View &y, const View &c, hipError_t *err);
 bool try_launch_small_p3(const Problem &p, const View &a, const View &y, const View &c, hipError_t *err);
 bool small_supports(int op, int64_t M, int64_t N, int64_t w, int dtype);
-// Vector-ALU kernels for the very narrow windows the MFMA families leave out: 16-bit band-in products
-// at w % 4 != 0 below 8, float32 (all three products) below the float32 family's range.
+// Vector-ALU kernels for the narrowest windows: 16-bit up to w = 3 (band-in) and w = 2 (band-out),
+// float32 (all three products) up to w = 14.
 bool try_launch_vector_p1(const Problem &p, const View &x, const View &y, const View &c, hipError_t *err);
 bool try_launch_vector_p2(const Problem &p, const View &a, const View &y, const View &c, hipError_t *err);
 bool try_launch_vector_p3(const Problem &p, const View &a, const View &y, const View &c, hipError_t *err);

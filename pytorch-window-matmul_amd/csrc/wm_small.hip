@@ -14,8 +14,8 @@
 //   P2  the workgroup copies its band rows flat into LDS (aligned 16-byte loads) and the
 //       rows [i0-w, i0+rows+w) of Y row-major into LDS; each wave then multiplies its rows:
 //       the skewed tile is read back with ds_read_b128 (the flat image keeps 8-column groups
-//       16-byte aligned when w % 4 == 0) and masked on bits, Y is read transposed with
-//       ds_read_b64_tr_b16.
+//       16-byte aligned when w % 4 == 0; for other windows the rows are re-pitched on their way
+//       into LDS) and masked on bits, Y is read transposed with ds_read_b64_tr_b16.
 //
 // One workgroup barrier per kernel; results are written exactly once; out-of-sequence band
 // entries are stored as +0.0.
@@ -137,9 +137,56 @@ __global__ __launch_bounds__(kThreads) void small_p1_kernel(const uint16_t *__re
 }
 
 // ------------------------------------------------------------------------------------------
-// P2 narrow: C[b,i,h] = sum_j A[b,i,j] * Y[b,i+j-w,h]      (w % 4 == 0)
+// Band rows for windows that are not a multiple of 4.  The MFMA reads of the band-in kernels
+// need an image whose 8-column groups are 16-byte aligned in every row, i.e. a row pitch of
+// 1 (mod 8) elements, which the flat band has only when w % 4 == 0.  For the other windows the
+// rows are re-pitched on their way into LDS: entry (r, j) goes to img[r * pitch + j], with the
+// pitch of the next window wp that is a multiple of 4 and the row centred in it, so that the
+// image is the band of window wp with the outer wp - w entries on either side missing (they are
+// masked like every other invalid entry).  The rows are fetched as aligned 16-byte chunks, all
+// issued together, and scattered element by element.
 // ------------------------------------------------------------------------------------------
-template <typename T, int NT, int RW>  // N <= 32 NT; RW rows per wave (64 or 32)
+template <int MAXC>
+__device__ __forceinline__ void fetch_band_rows(u32x4 (&reg)[MAXC], const uint16_t *rows, int n_el,
+                                                const uint16_t *safe, int tid) {
+  const int dg = (int)((reinterpret_cast<uintptr_t>(rows) >> 1) & 7);
+  const int n = n_el > 0 ? (dg + n_el + 7) >> 3 : 0;  // <= MAXC * kThreads (checked on the host)
+#pragma unroll
+  for (int u = 0; u < MAXC; ++u) {
+    const int q = tid + kThreads * u;
+    reg[u] = *reinterpret_cast<const u32x4 *>(q < n ? rows - dg + 8 * q : safe);
+  }
+}
+template <int MAXC>
+__device__ __forceinline__ void scatter_band_rows(const u32x4 (&reg)[MAXC], const uint16_t *rows, int n_el, int W,
+                                                  uint16_t *img, int pitch, int tid) {
+  const int dg = (int)((reinterpret_cast<uintptr_t>(rows) >> 1) & 7);
+  const int n = n_el > 0 ? (dg + n_el + 7) >> 3 : 0;
+  // (Lanes 16 apart meet in one LDS bank here; an element order rotated per 16-lane group avoids
+  // that and was measured 15-30 % slower: the address arithmetic, not the bank, is what costs.)
+#pragma unroll
+  for (int u = 0; u < MAXC; ++u) {
+    const int q = tid + kThreads * u;
+    if (q >= n) continue;
+    const int first = 8 * q - dg;  // flat index (r W + j) of the chunk's element 0
+    const int s = max(first, 0);
+    int r = s / W, j = s - r * W;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const int id = first + e;
+      if (id >= 0 && id < n_el) {
+        img[r * pitch + j] = (uint16_t)(reg[u][e >> 1] >> (16 * (e & 1)));
+        if (++j == W) j = 0, ++r;
+      }
+    }
+  }
+}
+constexpr int kRepitchChunksP2 = 4, kRepitchChunksP3 = 6;  // per thread: 128 and 192 rows of up to 63 entries
+
+// ------------------------------------------------------------------------------------------
+// P2 narrow: C[b,i,h] = sum_j A[b,i,j] * Y[b,i+j-w,h]
+// ------------------------------------------------------------------------------------------
+template <typename T, int NT, int RW, bool RP>  // N <= 32 NT; RW rows per wave; RP: w % 4 != 0, re-pitched image
 __global__ __launch_bounds__(kThreads) void small_p2_kernel(const uint16_t *__restrict__ A,
                                                             const uint16_t *__restrict__ Y,
                                                             uint16_t *__restrict__ C, int B, int M, int N, int w,
@@ -149,7 +196,8 @@ __global__ __launch_bounds__(kThreads) void small_p2_kernel(const uint16_t *__re
   constexpr int SY = lds_stride_tr(32 * NT);
   extern __shared__ __attribute__((aligned(16))) uint16_t lds[];
   const int W = 2 * w + 1;
-  const int a_elems = ((ROWS * W + 16 + 7) >> 3) << 3;  // flat band image, whole 16-byte chunks
+  const int wp = RP ? (w + 3) & ~3 : w, pad = wp - w;    // the image is laid out for window wp
+  const int a_elems = ((ROWS * (2 * wp + 1) + 16 + 7) >> 3) << 3;  // band image, whole 16-byte chunks
   uint16_t *aimg = lds;
   uint16_t *yimg = lds + a_elems;  // rows c = cv0 .. cv0 + ROWS + 2w + 32, stride SY; all initialised
 
@@ -160,15 +208,17 @@ __global__ __launch_bounds__(kThreads) void small_p2_kernel(const uint16_t *__re
   const int nrows = min(ROWS, M - i0);
   const uint16_t *Ab = A + (int64_t)b * asb + (int64_t)i0 * W;
   const uint16_t *Yb = Y + (int64_t)b * ysb;
-  const int delta = (int)((reinterpret_cast<uintptr_t>(Ab) >> 1) & 7);
+  const int delta = RP ? 0 : (int)((reinterpret_cast<uintptr_t>(Ab) >> 1) & 7);
 
   // band rows, flat: aligned chunks; the first and last chunk may hold neighbours' entries
   // (inside the tensor's pages: aligned 16-byte chunks never straddle a page)
   const int n_el = nrows * W;
-  const int chunks = (delta + n_el + 7) >> 3;
+  const int chunks = RP ? 0 : (delta + n_el + 7) >> 3;
+  u32x4 band[RP ? kRepitchChunksP2 : 1];
+  if constexpr (RP) fetch_band_rows(band, Ab, n_el, A, tid);
   // Y rows, row-major, zero outside the sequence
-  const int cv0 = i0 - w - 8;
-  const int yrows = ROWS + 2 * w + 32, ncg = N >> 3;  // every row a 16-column step can reach
+  const int cv0 = i0 - wp - 8;
+  const int yrows = ROWS + 2 * wp + 32, ncg = N >> 3;  // every row a 16-column step can reach
   const int ychunks = yrows * ncg;
   // loads go out in batches of 8 per thread before any of them is used
   constexpr int BATCH = 8;
@@ -192,9 +242,10 @@ __global__ __launch_bounds__(kThreads) void small_p2_kernel(const uint16_t *__re
         *reinterpret_cast<u32x4 *>(yimg + yr * SY + 8 * hg) = mask_row_chunk(reg[s], (c >= 0) & (c < M));
     }
   }
+  if constexpr (RP) scatter_band_rows(band, Ab, n_el, W, aimg + pad, 2 * wp + 1, tid);
   __syncthreads();
 
-  const int nks = (32 + 2 * w + delta + 15) >> 4;  // 16-column steps covering one 32-row tile's band
+  const int nks = (32 + 2 * wp + delta + 15) >> 4;  // 16-column steps covering one 32-row tile's band
   u32x2 outp[RW / 32][NT][4];
 #pragma unroll
   for (int nt = 0; nt < RW / 32; ++nt) {
@@ -205,16 +256,17 @@ __global__ __launch_bounds__(kThreads) void small_p2_kernel(const uint16_t *__re
     for (int t = 0; t < NT; ++t)
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[t][v] = 0.f;
-    // dense columns start at c_al = i0 + r0 - w - delta, which makes every 8-column group of every
-    // row an aligned chunk of the flat image: element index (r0 + r) 2w + r0 + 16 ks + 8 kg
-    const uint16_t *trow = aimg + (r0 + r) * 2 * w + r0 + 8 * (lane >> 5);
+    // dense columns start at c_al = i0 + r0 - wp - delta, which makes every 8-column group of every
+    // row an aligned chunk of the image: element index (r0 + r) 2wp + r0 + 16 ks + 8 kg
+    const uint16_t *trow = aimg + (r0 + r) * 2 * wp + r0 + 8 * (lane >> 5);
     for (int ks = 0; ks < nks; ++ks) {
       const int off = 16 * ks + 8 * (lane >> 5);    // column offset of this lane's group from c_al
-      const int c_g = i0 + r0 - w - delta + off;     // sequence position of its first element
+      const int c_g = i0 + r0 - wp - delta + off;    // sequence position of its first element
       u32x4 bop = *reinterpret_cast<const u32x4 *>(trow + 16 * ks);
-      // element e is band column j = off + e - delta - r of row i: valid iff 0 <= j <= 2w and 0 <= c < M
-      const int e_lo = max(delta + r - off, -c_g);
-      const int e_hi = i < M ? min(2 * w + delta + r - off, M - 1 - c_g) : -1;
+      // element e is image column off + e - delta - r of row i, band column j = that - pad:
+      // valid iff 0 <= j <= 2w and 0 <= c < M
+      const int e_lo = max(pad + delta + r - off, -c_g);
+      const int e_hi = i < M ? min(pad + 2 * w + delta + r - off, M - 1 - c_g) : -1;
       bop = mask_band_chunk(bop, e_lo, e_hi);
       const int k0 = r0 - delta + 8 + 16 * ks;  // row of yimg holding sequence position c_al + 16 ks
 #pragma unroll
@@ -257,7 +309,7 @@ __global__ __launch_bounds__(kThreads) void small_p2_kernel(const uint16_t *__re
 }
 
 // ------------------------------------------------------------------------------------------
-// P3 narrow: C[b,c,h] = sum_r A[b,r,c-r+w] * Y[b,r,h]      (w % 4 == 0)
+// P3 narrow: C[b,c,h] = sum_r A[b,r,c-r+w] * Y[b,r,h]
 // ------------------------------------------------------------------------------------------
 // Output-stationary like the wide kernel, staged like the narrow P2: a workgroup owns ROWS
 // output rows c and copies the band rows r in [c_first - w, c_last + w] flat into LDS, plus
@@ -266,7 +318,9 @@ __global__ __launch_bounds__(kThreads) void small_p2_kernel(const uint16_t *__re
 // chunk grid along c is the same in every row: output tiles are laid on that grid (shifted by
 // `shift` = (base + w) mod 8 against c = 0, the same for all workgroups of a batch element) and
 // ds_read_b64_tr_b16 then delivers, per lane c, the entries of 8 consecutive r: the B operand.
-template <typename T, int NT, int RW>  // N <= 32 NT; RW output rows per wave (64 or 32)
+// For w % 4 != 0 (RP) the image is re-pitched to the next multiple of 4, wp, and its grid is free:
+// Mat has row stride 2wp, starts on a chunk boundary and the tiles start at c = 0.
+template <typename T, int NT, int RW, bool RP>  // N <= 32 NT; RW output rows per wave
 __global__ __launch_bounds__(kThreads) void small_p3_kernel(const uint16_t *__restrict__ A,
                                                             const uint16_t *__restrict__ Y,
                                                             uint16_t *__restrict__ C, int B, int M, int N, int w,
@@ -276,8 +330,9 @@ __global__ __launch_bounds__(kThreads) void small_p3_kernel(const uint16_t *__re
   constexpr int SY = lds_stride_tr(32 * NT);
   extern __shared__ __attribute__((aligned(16))) uint16_t lds[];
   const int W = 2 * w + 1;
-  const int span = ROWS + 2 * w;                         // band / Y rows a workgroup can touch
-  const int a_elems = ((span * W + 16 + 7) >> 3) << 3;   // flat band image, whole 16-byte chunks
+  const int wp = RP ? (w + 3) & ~3 : w, pad = wp - w;    // the image is laid out for window wp
+  const int span = ROWS + 2 * wp;                        // band / Y rows a workgroup can touch
+  const int a_elems = ((span * (2 * wp + 1) + 16 + 7) >> 3) << 3;  // band image, whole 16-byte chunks
   uint16_t *aimg = lds;
   // Y rows r_org .. r_org + span + 15 (the last 16-row step may run past the span), stride SY, zero
   // outside the sequence and all initialised: they meet masked zeros of the band inside the MFMA
@@ -287,21 +342,25 @@ __global__ __launch_bounds__(kThreads) void small_p3_kernel(const uint16_t *__re
   if (!decode_block(nblk, B, &b, &blk)) return;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int64_t base_el = (int64_t)(reinterpret_cast<uintptr_t>(A) >> 1) + (int64_t)b * asb;
-  const int shift = (int)((base_el + w) & 7);
+  const int shift = RP ? 0 : (int)((base_el + w) & 7);
   const int c_first = blk * ROWS - shift;  // first output row of this workgroup (may be < 0)
   if (c_first >= M) return;
-  const int r_org = c_first - w;           // band row that image row 0 stands for (may be < 0)
+  const int r_org = c_first - wp;          // band row that image row 0 stands for (may be < 0)
   const int r_s = max(r_org, 0), r_e = min(r_org + span - 1, M - 1);  // rows that exist
   const uint16_t *Yb = Y + (int64_t)b * ysb;
   // global element index of image element 0, rounded down to a chunk: g0 = base + r_org * W - delta
   const int64_t g_org = base_el + (int64_t)r_org * W;
-  const int delta = (int)(g_org & 7);
+  const int delta = RP ? 0 : (int)(g_org & 7);
   const uint16_t *img_src = A + ((g_org - delta) - (int64_t)(reinterpret_cast<uintptr_t>(A) >> 1));
 
   // flat band rows r_s..r_e: whole aligned chunks (neighbours' entries at both ends are masked later)
   const int q_lo = (delta + (r_s - r_org) * W) >> 3;
   const int q_hi = (delta + (r_e + 1 - r_org) * W + 7) >> 3;  // exclusive
-  const int chunks = max(q_hi - q_lo, 0);
+  const int chunks = RP ? 0 : max(q_hi - q_lo, 0);
+  const uint16_t *band_rows = A + (int64_t)b * asb + (int64_t)r_s * W;  // RP: rows r_s..r_e, re-pitched
+  const int band_el = (r_e - r_s + 1) * W;
+  u32x4 band[RP ? kRepitchChunksP3 : 1];
+  if constexpr (RP) fetch_band_rows(band, band_rows, band_el, A, tid);
   const int ncg = N >> 3;
   const int ychunks = (span + 16) * ncg;
   constexpr int BATCH = 8;
@@ -325,9 +384,11 @@ __global__ __launch_bounds__(kThreads) void small_p3_kernel(const uint16_t *__re
         *reinterpret_cast<u32x4 *>(yimg + yr * SY + 8 * hg) = mask_row_chunk(reg[s], (r >= 0) & (r < M));
     }
   }
+  if constexpr (RP)
+    scatter_band_rows(band, band_rows, band_el, W, aimg + (r_s - r_org) * (2 * wp + 1) + pad, 2 * wp + 1, tid);
   __syncthreads();
 
-  const int nks = (32 + 2 * w + 15) >> 4;  // 16-row steps covering the band rows of one 32-row output tile
+  const int nks = (32 + 2 * wp + 15) >> 4;  // 16-row steps covering the band rows of one 32-row output tile
   u32x2 outp[RW / 32][NT][4];
 #pragma unroll
   for (int nt = 0; nt < RW / 32; ++nt) {
@@ -338,11 +399,11 @@ __global__ __launch_bounds__(kThreads) void small_p3_kernel(const uint16_t *__re
     for (int t = 0; t < NT; ++t)
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[t][v] = 0.f;
-    // Mat[k][x]: k = r - r_org, x = c - r_org + w = t0 + (lane & 31) + 2w; element delta + k*2w + x
+    // Mat[k][x]: k = r - r_org, x = c - r_org + wp = t0 + (lane & 31) + 2wp; element delta + k*2wp + x
     for (int ks = 0; ks < nks; ++ks) {
-      const int k0 = t0 + 16 * ks;                       // image row of band row c_tile - w + 16 ks
+      const int k0 = t0 + 16 * ks;                       // image row of band row c_tile - wp + 16 ks
       const int r_g = r_org + k0 + 8 * (lane >> 5);      // band row of this lane's element 0
-      u32x4 bop = lds_read_transposed(aimg + delta, 2 * w, k0, t0 + 2 * w, lane);
+      u32x4 bop = lds_read_transposed(aimg + delta, 2 * wp, k0, t0 + 2 * wp, lane);
       // element e is band row r_g + e: valid iff |r - c| <= w and 0 <= r < M
       const int e_lo = max(c - w - r_g, -r_g);
       const int e_hi = min(c + w - r_g, M - 1 - r_g);
@@ -425,7 +486,10 @@ hipError_t launch_small_p1(const Problem &p, const View &x, const View &y, const
   return hipGetLastError();
 }
 
-// LDS bytes of the P2 kernel: flat band image of `rows` rows plus the Y rows they reach.
+// Window the LDS images of the band-in kernels are laid out for: w itself or the next multiple of 4.
+int64_t image_window(int64_t w) { return (w + 3) & ~(int64_t)3; }
+
+// LDS bytes of the P2 kernel: band image of `rows` rows plus the Y rows they reach.
 size_t small_p2_lds(int64_t rows, int64_t w, int64_t NT) {
   const int64_t W = 2 * w + 1;
   const size_t a_elems = (size_t)(((rows * W + 16 + 7) >> 3) << 3);
@@ -444,17 +508,24 @@ hipError_t launch_small_p2(const Problem &p, const View &a, const View &y, const
   const int rows = 4 * RW;
   const int nblk = (int)((p.M + rows - 1) / rows);
   const dim3 grid(small_grid(p.B, nblk)), block(kThreads);
-  const size_t lds = small_p2_lds(rows, p.w, NT);
-#define WM_SP2(NT_, RW_)                                                                                       \
-  hipLaunchKernelGGL((small_p2_kernel<T, NT_, RW_>), grid, block, lds, p.stream, (const uint16_t *)a.data,     \
+  const size_t lds = small_p2_lds(rows, image_window(p.w), NT);
+#define WM_SP2(NT_, RW_, RP_)                                                                                  \
+  hipLaunchKernelGGL((small_p2_kernel<T, NT_, RW_, RP_>), grid, block, lds, p.stream, (const uint16_t *)a.data, \
                      (const uint16_t *)y.data, (uint16_t *)c.data, (int)p.B, (int)p.M, (int)p.N, (int)p.w, nblk, \
                      a.sb, y.sb, y.sr, c.sb, c.sr)
-  switch (NT) {
-    case 1: WM_SP2(1, 32); break;
-    case 2: WM_SP2(2, 32); break;
-    case 3: WM_SP2(3, 32); break;
-    default: WM_SP2(4, 32); break;
+#define WM_SP2_N(RP_)                   \
+  switch (NT) {                         \
+    case 1: WM_SP2(1, 32, RP_); break;  \
+    case 2: WM_SP2(2, 32, RP_); break;  \
+    case 3: WM_SP2(3, 32, RP_); break;  \
+    default: WM_SP2(4, 32, RP_); break; \
   }
+  if (p.w % 4 == 0) {
+    WM_SP2_N(false)
+  } else {
+    WM_SP2_N(true)
+  }
+#undef WM_SP2_N
 #undef WM_SP2
   return hipGetLastError();
 }
@@ -474,17 +545,24 @@ hipError_t launch_small_p3(const Problem &p, const View &a, const View &y, const
   const int rows = 4 * RW;
   const int nblk = (int)((p.M + 7 + rows - 1) / rows);  // output tiles start up to 7 rows before row 0
   const dim3 grid(small_grid(p.B, nblk)), block(kThreads);
-  const size_t lds = small_p3_lds(rows, p.w, NT);
-#define WM_SP3(NT_, RW_)                                                                                       \
-  hipLaunchKernelGGL((small_p3_kernel<T, NT_, RW_>), grid, block, lds, p.stream, (const uint16_t *)a.data,     \
+  const size_t lds = small_p3_lds(rows, image_window(p.w), NT);
+#define WM_SP3(NT_, RW_, RP_)                                                                                  \
+  hipLaunchKernelGGL((small_p3_kernel<T, NT_, RW_, RP_>), grid, block, lds, p.stream, (const uint16_t *)a.data, \
                      (const uint16_t *)y.data, (uint16_t *)c.data, (int)p.B, (int)p.M, (int)p.N, (int)p.w, nblk, \
                      a.sb, y.sb, y.sr, c.sb, c.sr)
-  switch (NT) {
-    case 1: WM_SP3(1, 32); break;
-    case 2: WM_SP3(2, 32); break;
-    case 3: WM_SP3(3, 32); break;
-    default: WM_SP3(4, 32); break;
+#define WM_SP3_N(RP_)                   \
+  switch (NT) {                         \
+    case 1: WM_SP3(1, 32, RP_); break;  \
+    case 2: WM_SP3(2, 32, RP_); break;  \
+    case 3: WM_SP3(3, 32, RP_); break;  \
+    default: WM_SP3(4, 32, RP_); break; \
   }
+  if (p.w % 4 == 0) {
+    WM_SP3_N(false)
+  } else {
+    WM_SP3_N(true)
+  }
+#undef WM_SP3_N
 #undef WM_SP3
   return hipGetLastError();
 }
@@ -499,11 +577,14 @@ bool small_supports(int op, int64_t M, int64_t N, int64_t w, int dtype) {
   if (op == 2) {
     // the two LDS images must fit the default 64 KB dynamic limit; wider cases go to the wide-band family
     const int64_t NT = (N + 31) / 32;
-    return w % 4 == 0 && small_p2_lds(4 * small_p2_rows_per_wave(w, NT), w, NT) <= kSmallLdsLimit;
+    return small_p2_lds(4 * small_p2_rows_per_wave(w, NT), image_window(w), NT) <= kSmallLdsLimit;
   }
   if (op == 3) {
     const int64_t NT = (N + 31) / 32;
-    return w % 4 == 0 && small_p3_lds(4 * small_p3_rows_per_wave(w, NT), w, NT) <= kSmallLdsLimit;
+    // re-pitched images of w = 29..31 (two workgroups per CU) were measured slower than the wide-band
+    // kernel: 198-202 us against 156-161 us at B96 M16384 N64
+    if (w % 4 != 0 && w > 28) return false;
+    return small_p3_lds(4 * small_p3_rows_per_wave(w, NT), image_window(w), NT) <= kSmallLdsLimit;
   }
   return false;
 }

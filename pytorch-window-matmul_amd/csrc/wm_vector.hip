@@ -1,9 +1,8 @@
 // Vector-ALU kernels for very narrow bands on gfx950 (16-bit storage and float32, float32 accumulate).
 //
-// The narrow-band MFMA kernels read their skewed tile with 16-byte LDS reads, which needs the flat
-// band image to keep 8-column groups aligned in every row, i.e. w % 4 == 0, and the float32 MFMA
-// kernels walk 128-row tiles in chunks of 32 columns, mostly empty when the band is a few entries
-// wide.  For these windows the band-in products
+// The narrow-band MFMA kernels multiply 32-row tiles against at least 48 dense columns and the
+// float32 MFMA kernels walk 128-row tiles in chunks of 32 columns: mostly empty work when the band
+// is a few entries wide.  For these windows the band-in products
 //     P2  C[i,h] = sum_j A[i,j] Y[i+j-w,h]          P3  C[c,h] = sum_r A[r,c-r+w] Y[r,h]
 // are 2w+1 multiply-adds per output element on operands that are streamed once: far too little
 // arithmetic for the matrix pipe to matter, so each thread simply owns 16 bytes of one output row
@@ -24,7 +23,7 @@ namespace wm {
 namespace {
 
 #ifndef WM_VECTOR_MAX_W
-#define WM_VECTOR_MAX_W 11
+#define WM_VECTOR_MAX_W 3
 #endif
 constexpr int VECTOR_MAX_W = WM_VECTOR_MAX_W;
 #ifndef WM_VECTOR_F32_MAX_W
@@ -352,9 +351,8 @@ bool band_contiguous(const View &v, int64_t W) { return v.sc == 1 && v.sr == W &
 
 }  // namespace
 
-// 16-bit: band-in products at the windows the narrow-band MFMA kernels do not take (w % 4 != 0) up to
-// w = 11, where the wide-band MFMA kernels catch up; the band-out product at w <= 2 (measured faster than the narrow-band
-// MFMA kernel there: 79-94 us against 96-98 us at B96 M16384 N64).
+// 16-bit: band-in products up to w = 3 (61-71 us against 73-86 us for the narrow-band MFMA kernels at
+// B96 M16384 N64; those win from w = 4 on); the band-out product at w <= 2 (79-94 us against 96-98 us).
 // float32: every window up to VECTOR_F32_MAX_W, all three products.
 bool vector_supports(int op, int64_t M, int64_t N, int64_t w, int dtype) {
   if (op < 1 || op > 3 || M < 1 || M > (1 << 30) || w < 1) return false;
@@ -365,7 +363,7 @@ bool vector_supports(int op, int64_t M, int64_t N, int64_t w, int dtype) {
   if (dtype != WM_DTYPE_BF16 && dtype != WM_DTYPE_F16) return false;
   if (N < 16 || N > 128 || N % 16 != 0) return false;
   if (op == 1) return w <= VECTOR_OUT_MAX_W && vector_out_lds(w, N, dtype) <= 65536;
-  return w <= VECTOR_MAX_W && w % 4 != 0 && vector_lds(w, N, dtype) <= 65536;
+  return w <= VECTOR_MAX_W && vector_lds(w, N, dtype) <= 65536;
 }
 
 bool try_launch_vector_p1(const Problem &p, const View &x, const View &y, const View &c, hipError_t *err) {

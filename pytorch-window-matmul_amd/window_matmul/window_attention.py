@@ -21,9 +21,9 @@ from .window_matmul import unwindow_matmul, window_matmul
 
 def _chain_is_faster(window_size: int) -> bool:
     """Windows at which a training step is faster through the separate ops than through the fused
-    kernels (measured at B96 M16384 N64 bf16: 0.49-0.60 ms against 0.67-0.75 ms at w <= 8 and at
-    w = 12; the fused kernels win at w = 9, 10, 11 and from 13 on, 0.67 ms against 0.69-1.0 ms)."""
-    return window_size <= 8 or window_size == 12
+    kernels (measured at B96 M16384 N64 bf16: 0.48-0.64 ms against 0.67-0.75 ms up to w = 12, equal
+    at w = 13, 0.68-1.08 ms against 0.67-0.69 ms from w = 14 to 32)."""
+    return window_size <= 12
 
 
 class WindowAttentionFunc(torch.autograd.Function):

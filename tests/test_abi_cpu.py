@@ -56,17 +56,19 @@ def test_kernel_choice_names():
     assert L.wm_kernel_choice(2, 96, 4096, 64, 256, 2, 1, 0) == b"mfma_p2"
     assert L.wm_kernel_choice(1, 96, 16384, 64, 8, 2, 1, 0) == b"narrow_p1"
     assert L.wm_kernel_choice(2, 96, 16384, 64, 8, 1, 1, 0) == b"narrow_p2"
-    assert L.wm_kernel_choice(2, 96, 16384, 64, 9, 2, 1, 0) == b"vector_p2"
-    assert L.wm_kernel_choice(2, 96, 16384, 64, 13, 2, 1, 0) == b"mfma_p2"
+    assert L.wm_kernel_choice(2, 96, 16384, 64, 9, 2, 1, 0) == b"narrow_p2"   # re-pitched LDS image
+    assert L.wm_kernel_choice(2, 96, 16384, 64, 13, 2, 1, 0) == b"narrow_p2"
     assert L.wm_kernel_choice(3, 96, 16384, 64, 8, 2, 1, 0) == b"narrow_p3"
-    assert L.wm_kernel_choice(3, 96, 16384, 64, 10, 2, 1, 0) == b"vector_p3"
-    assert L.wm_kernel_choice(3, 96, 16384, 64, 14, 2, 1, 0) == b"mfma_p3"
+    assert L.wm_kernel_choice(3, 96, 16384, 64, 10, 2, 1, 0) == b"narrow_p3"
+    assert L.wm_kernel_choice(3, 96, 16384, 64, 27, 2, 1, 0) == b"narrow_p3"
+    assert L.wm_kernel_choice(3, 96, 16384, 64, 30, 2, 1, 0) == b"mfma_p3"     # two workgroups per CU: slower
+    assert L.wm_kernel_choice(2, 96, 16384, 64, 30, 2, 1, 0) == b"narrow_p2"
     assert L.wm_kernel_choice(2, 96, 16384, 64, 32, 2, 1, 0) == b"narrow_p2"  # 32 rows per wave still fit LDS
     assert L.wm_kernel_choice(3, 96, 16384, 128, 32, 2, 1, 0) == b"mfma_p3"   # images beyond 64 KB of LDS
     assert L.wm_kernel_choice(1, 96, 16384, 64, 8, 2, 1, abi.NO_NARROW_BAND) == b"mfma_p1"
-    # narrow windows the narrow-band MFMA kernels leave out (w % 4 != 0, w <= 11): vector-ALU band-in kernels
+    # the narrowest windows (w <= 3, not enough terms for a matrix pipe): vector-ALU band-in kernels
     assert L.wm_kernel_choice(2, 96, 16384, 64, 1, 2, 1, 0) == b"vector_p2"
-    assert L.wm_kernel_choice(3, 96, 16384, 64, 7, 1, 1, 0) == b"vector_p3"
+    assert L.wm_kernel_choice(3, 96, 16384, 64, 3, 1, 1, 0) == b"vector_p3"
     assert L.wm_kernel_choice(1, 96, 16384, 64, 7, 1, 1, 0) == b"narrow_p1"
     assert L.wm_kernel_choice(1, 96, 16384, 64, 2, 2, 1, 0) == b"vector_p1"
     assert L.wm_kernel_choice(1, 96, 16384, 64, 3, 2, 1, 0) == b"narrow_p1"

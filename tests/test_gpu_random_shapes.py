@@ -63,6 +63,25 @@ def test_kernel_choice_agrees_with_strided_family(device, dtype, B, M, N, w):
         _assert_close(results[0][name], results[1][name], tol, name)
 
 
+@pytest.mark.parametrize("w", range(1, 33))
+@pytest.mark.parametrize("dtype,B,M,N", [(torch.bfloat16, 3, 300, 64), (torch.float16, 2, 129, 16),
+                                         (torch.bfloat16, 5, 1000, 128), (torch.float16, 2, 31, 96)])
+def test_every_narrow_window(device, dtype, B, M, N, w):
+    """The band-in kernels lay their LDS image out differently for w % 4 == 0 and for the other
+    windows, and the batch stride M (2w + 1) moves the band rows through every alignment."""
+    g = torch.Generator().manual_seed(w * 131 + M)
+    q, k, v, go = (_randn((B, M, N), g, dtype, device) for _ in range(4))
+    a = _randn((B, M, 2 * w + 1), g, dtype, device, 0.2)
+    results = []
+    for flags in (0, abi.FORCE_STRIDED):
+        out = abi.unwindow_forward(a, v, w, flags)
+        ga, gv = abi.unwindow_backward(a, v, w, go, flags)
+        gq, gk = abi.window_backward(q, k.transpose(1, 2), w, a, flags)
+        results.append(dict(unwindow_fwd=out, grad_a=ga, grad_v=gv, grad_q=gq, grad_k=gk))
+    for name in results[0]:
+        _assert_close(results[0][name], results[1][name], 2e-2, name)
+
+
 ATTENTION_CASES = _draw(2, 40, [16, 32, 48, 64, 80, 96, 112, 128], [torch.bfloat16, torch.float16])
 
 
