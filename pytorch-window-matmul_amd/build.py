@@ -30,7 +30,7 @@ HIPCC_FLAGS = [
     "-fPIC",
     "-Wall",
     "-Wno-unused-function",
-    # extra hipcc flags for experiments, e.g. WM_EXTRA_FLAGS=-DWM_P2_KC=32
+    # extra hipcc flags for experiments, e.g. WM_EXTRA_FLAGS=-DWM_VECTOR_MAX_W=0
     *os.environ.get("WM_EXTRA_FLAGS", "").split(),
     # keep the compiler from forming packed-fp32 VALU ops
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",

@@ -560,6 +560,8 @@ int band_group(const View &v, int64_t w) { return (w % 32 == 0 && ((uintptr_t)v.
 
 unsigned grid_size(int64_t B, int64_t nblk) { return (unsigned)(((B + 7) / 8) * 8 * nblk); }
 
+// Chunk length of P2 (64: the result rows are staged in the band tile buffers, which 32 would make
+// too small; 32 and 128 were measured slower before that).
 #ifndef WM_P2_KC
 #define WM_P2_KC 64
 #endif
