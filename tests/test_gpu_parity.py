@@ -31,6 +31,8 @@ EDGE = [
     (1, 300, 64, 150), (2, 65, 16, 100), (1, 513, 72, 256), (2, 96, 64, 8), (1, 200, 40, 12), (3, 64, 64, 1),
     (1, 1000, 64, 32), (2, 333, 24, 7), (3, 700, 64, 32), (1, 1100, 32, 256), (2, 900, 128, 64), (9, 260, 16, 96),
     (2, 600, 128, 16), (2, 515, 80, 20), (1, 300, 64, 7), (2, 260, 48, 28), (1, 257, 64, 8), (2, 1030, 64, 12),
+    # windows that are not a multiple of 4 (band rows re-pitched on their way into LDS), odd batch strides
+    (3, 201, 64, 13), (2, 150, 32, 22), (3, 141, 128, 27), (2, 90, 16, 5), (3, 171, 96, 30), (2, 400, 64, 9),
 ]
 CASES = REF_GRID + EDGE
 DTYPES = [torch.float32, torch.bfloat16, torch.float16, torch.float64]
