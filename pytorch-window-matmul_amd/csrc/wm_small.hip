@@ -6,7 +6,7 @@
 // wave owns 64 (P1) or 32 (P2, P3) consecutive rows and everything it needs:
 //
 //   P1  the wave loads its rows of X and the rows [r0-w, r0+64+w) of Y straight from HBM
-//       into MFMA operand registers (no LDS, no barrier), forms the 32x32 tiles that touch
+//       into MFMA operand registers (no LDS, no barrier), forms the 16x16 tiles that touch
 //       the band, and scatters the band entries into a flat LDS image of the workgroup's
 //       band rows, which then leaves as aligned 16-byte stores.
 //       (Staging the operands in LDS with coalesced loads, 32 rows per wave, and replacing the
@@ -29,13 +29,19 @@ constexpr int SMALL_MAX_W = 32;
 // ------------------------------------------------------------------------------------------
 // P1 narrow: band[b,i,j] = sum_h X[b,i,h] * Y[b,i+j-w,h]
 // ------------------------------------------------------------------------------------------
-template <typename T, int NK, int NMT>  // N = 16 NK; NMT 32-column tiles cover 64 + 2w columns
+// 16x16x32 tiles: a 16-row block of the band meets 2 + w / 8 Y tiles of 16 rows, and a wave fetches
+// 64 + 2w (+ up to 15) rows of Y.  (The same kernel on 32x32x16 tiles formed and scattered twice
+// as many products per band entry and fetched 96 or 128 rows of Y: 98 us against 85 us at
+// B96 M16384 N64 w8, 10-20 % slower at every N and w.)  When N is an odd multiple of 16 the upper
+// half of the last 32-column step is fed zeros.
+template <typename T, int NK, int NYT>  // N = 16 NK; NYT 16-row tiles of Y cover 64 + 2w rows
 __global__ __launch_bounds__(kThreads) void small_p1_kernel(const uint16_t *__restrict__ X,
-                                                            const uint16_t *__restrict__ Y,
-                                                            uint16_t *__restrict__ C, int B, int M, int w, int nblk,
-                                                            int64_t xsb, int64_t xsr, int64_t ysb, int64_t ysr,
-                                                            int64_t csb) {
+                                                              const uint16_t *__restrict__ Y,
+                                                              uint16_t *__restrict__ C, int B, int M, int w, int nblk,
+                                                              int64_t xsb, int64_t xsr, int64_t ysb, int64_t ysr,
+                                                              int64_t csb) {
   constexpr int ROWS = 256;  // band rows per workgroup, 64 per wave
+  constexpr int NK2 = (NK + 1) / 2;  // 32-column steps
   extern __shared__ __attribute__((aligned(16))) uint16_t flat[];  // 8 + ROWS * W (+ slack) elements
 
   int b, blk;
@@ -44,38 +50,38 @@ __global__ __launch_bounds__(kThreads) void small_p1_kernel(const uint16_t *__re
   const int W = 2 * w + 1;
   const int i0 = blk * ROWS, iw0 = i0 + 64 * wave;
   const int nrows = min(ROWS, M - i0);
-  uint16_t *Cb = C + (int64_t)b * csb + (int64_t)i0 * W;  // first band entry of this workgroup
-  const int delta = (int)((reinterpret_cast<uintptr_t>(Cb) >> 1) & 7);  // elements past a 16-byte boundary
+  uint16_t *Cb = C + (int64_t)b * csb + (int64_t)i0 * W;
+  const int delta = (int)((reinterpret_cast<uintptr_t>(Cb) >> 1) & 7);
 
   if (iw0 < M) {
-    // operands straight into registers: all loads are issued before the first use
-    u32x4 xop[2][NK], yop[NMT][NK];
+    const int l16 = lane & 15, kq = lane >> 4;  // row of a tile; 8-column group of a 32-column step
+    auto has_columns = [&](int ks) { return 32 * ks + 8 * kq < 16 * NK; };  // false only in half a last step
+    u32x4 xop[4][NK2], yop[NYT][NK2];
     const uint16_t *Xb = X + (int64_t)b * xsb, *Yb = Y + (int64_t)b * ysb;
 #pragma unroll
-    for (int nt = 0; nt < 2; ++nt) {
-      const int i = iw0 + 32 * nt + (lane & 31);
+    for (int rb = 0; rb < 4; ++rb) {
+      const int i = iw0 + 16 * rb + l16;
 #pragma unroll
-      for (int ks = 0; ks < NK; ++ks)
-        xop[nt][ks] = fetch_row_chunk(Xb + (int64_t)i * xsr + 16 * ks + 8 * (lane >> 5), X, i < M);
+      for (int ks = 0; ks < NK2; ++ks) xop[rb][ks] = fetch_row_chunk(Xb + (int64_t)i * xsr + 32 * ks + 8 * kq, X, (i < M) & has_columns(ks));
     }
 #pragma unroll
-    for (int mt = 0; mt < NMT; ++mt) {
-      const int c = iw0 - w + 32 * mt + (lane & 31);
+    for (int t = 0; t < NYT; ++t) {
+      const int c = iw0 - w + 16 * t + l16;
 #pragma unroll
-      for (int ks = 0; ks < NK; ++ks)
-        yop[mt][ks] = fetch_row_chunk(Yb + (int64_t)c * ysr + 16 * ks + 8 * (lane >> 5), Y, (c >= 0) & (c < M));
+      for (int ks = 0; ks < NK2; ++ks)
+        yop[t][ks] = fetch_row_chunk(Yb + (int64_t)c * ysr + 32 * ks + 8 * kq, Y, (c >= 0) & (c < M) & has_columns(ks));
     }
 #pragma unroll
-    for (int nt = 0; nt < 2; ++nt) {
-      const int i = iw0 + 32 * nt + (lane & 31);
+    for (int rb = 0; rb < 4; ++rb) {
+      const int i = iw0 + 16 * rb + l16;
 #pragma unroll
-      for (int ks = 0; ks < NK; ++ks) xop[nt][ks] = mask_row_chunk(xop[nt][ks], i < M);
+      for (int ks = 0; ks < NK2; ++ks) xop[rb][ks] = mask_row_chunk(xop[rb][ks], (i < M) & has_columns(ks));
     }
 #pragma unroll
-    for (int mt = 0; mt < NMT; ++mt) {
-      const int c = iw0 - w + 32 * mt + (lane & 31);
+    for (int t = 0; t < NYT; ++t) {
+      const int c = iw0 - w + 16 * t + l16;
 #pragma unroll
-      for (int ks = 0; ks < NK; ++ks) yop[mt][ks] = mask_row_chunk(yop[mt][ks], (c >= 0) & (c < M));
+      for (int ks = 0; ks < NK2; ++ks) yop[t][ks] = mask_row_chunk(yop[t][ks], (c >= 0) & (c < M) & has_columns(ks));
     }
 
     uint16_t *img = flat + delta + (64 * wave) * W;  // this wave's 64 rows of the flat band image
@@ -83,39 +89,32 @@ __global__ __launch_bounds__(kThreads) void small_p1_kernel(const uint16_t *__re
     // even, c_rel being a multiple of 4): then every quad of 4 consecutive entries is 8-byte aligned
     const bool quad_aligned = (w % 2 == 0) && (delta % 4 == 0);
 #pragma unroll
-    for (int nt = 0; nt < 2; ++nt) {
+    for (int rb = 0; rb < 4; ++rb) {
 #pragma unroll
-      for (int mt = 0; mt < NMT; ++mt) {
-        // tile columns c_rel in [32 mt, 32 mt + 32), rows r_rel in [32 nt, 32 nt + 32); j = c_rel - r_rel
-        if (32 * (mt - nt) + 31 < 0 || 32 * (mt - nt) - 31 > 2 * w) continue;
-        f32x16 acc;
+      for (int t = 0; t < NYT; ++t) {
+        // tile columns c_rel in [16 t, 16 t + 16), rows r_rel in [16 rb, 16 rb + 16); j = c_rel - r_rel
+        if (16 * (t - rb) + 15 < 0 || 16 * (t - rb) - 15 > 2 * w) continue;
+        f32x4 acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int v = 0; v < 16; ++v) acc[v] = 0.f;
-#pragma unroll
-        for (int ks = 0; ks < NK; ++ks) acc = Mma<T>::run(yop[mt][ks], xop[nt][ks], acc);
-        // acc[v]: c_rel = 32 mt + 8 (v / 4) + 4 (lane / 32) + v % 4, r_rel = 32 nt + lane % 32
-        const int r_rel = 32 * nt + (lane & 31);
+        for (int ks = 0; ks < NK2; ++ks) acc = Mma<T>::run16(yop[t][ks], xop[rb][ks], acc);
+        // acc[v]: c_rel = 16 t + 4 (lane / 16) + v, r_rel = 16 rb + lane % 16
+        const int r_rel = 16 * rb + l16, c_rel = 16 * t + 4 * kq;
         uint16_t *row = img + r_rel * W;
-#pragma unroll
-        for (int q4 = 0; q4 < 4; ++q4) {
-          const int c_rel = 32 * mt + 8 * q4 + 4 * (lane >> 5);
-          const int j = c_rel - r_rel;     // band column of the first of 4 consecutive entries
-          const int c = iw0 - w + c_rel;   // their sequence positions c .. c + 3
-          const uint32_t lo = Mma<T>::pack2(acc[4 * q4], acc[4 * q4 + 1]);
-          const uint32_t hi = Mma<T>::pack2(acc[4 * q4 + 2], acc[4 * q4 + 3]);
-          // entries outside the sequence are +0.0 by definition, whatever X holds
-          const bool seq_all = c >= 0 && c + 3 < M;
-          if (quad_aligned && j >= 0 && j + 3 <= 2 * w && seq_all) {
-            u32x2 o = {lo, hi};  // whole quad inside band and sequence: one 8-byte LDS write
-            *reinterpret_cast<u32x2 *>(row + j) = o;
-          } else if (j + 3 >= 0 && j <= 2 * w) {
-            if (j >= 0 && j <= 2 * w) row[j] = (c >= 0 && c < M) ? (uint16_t)lo : (uint16_t)0;
-            if (j + 1 >= 0 && j + 1 <= 2 * w)
-              row[j + 1] = (c + 1 >= 0 && c + 1 < M) ? (uint16_t)(lo >> 16) : (uint16_t)0;
-            if (j + 2 >= 0 && j + 2 <= 2 * w) row[j + 2] = (c + 2 >= 0 && c + 2 < M) ? (uint16_t)hi : (uint16_t)0;
-            if (j + 3 >= 0 && j + 3 <= 2 * w)
-              row[j + 3] = (c + 3 >= 0 && c + 3 < M) ? (uint16_t)(hi >> 16) : (uint16_t)0;
-          }
+        const int j = c_rel - r_rel;     // band column of the first of 4 consecutive entries
+        const int c = iw0 - w + c_rel;   // their sequence positions c .. c + 3
+        const uint32_t lo = Mma<T>::pack2(acc[0], acc[1]);
+        const uint32_t hi = Mma<T>::pack2(acc[2], acc[3]);
+        const bool seq_all = c >= 0 && c + 3 < M;  // entries outside the sequence are +0.0 by definition
+        if (quad_aligned && j >= 0 && j + 3 <= 2 * w && seq_all) {
+          u32x2 o = {lo, hi};  // whole quad inside band and sequence: one 8-byte LDS write
+          *reinterpret_cast<u32x2 *>(row + j) = o;
+        } else if (j + 3 >= 0 && j <= 2 * w) {
+          if (j >= 0 && j <= 2 * w) row[j] = (c >= 0 && c < M) ? (uint16_t)lo : (uint16_t)0;
+          if (j + 1 >= 0 && j + 1 <= 2 * w)
+            row[j + 1] = (c + 1 >= 0 && c + 1 < M) ? (uint16_t)(lo >> 16) : (uint16_t)0;
+          if (j + 2 >= 0 && j + 2 <= 2 * w) row[j + 2] = (c + 2 >= 0 && c + 2 < M) ? (uint16_t)hi : (uint16_t)0;
+          if (j + 3 >= 0 && j + 3 <= 2 * w)
+            row[j + 3] = (c + 3 >= 0 && c + 3 < M) ? (uint16_t)(hi >> 16) : (uint16_t)0;
         }
       }
     }
@@ -461,25 +460,29 @@ hipError_t launch_small_p1(const Problem &p, const View &x, const View &y, const
   const int nblk = (int)((p.M + 255) / 256);
   const dim3 grid(small_grid(p.B, nblk)), block(kThreads);
   const size_t lds = (size_t)(256 * (2 * p.w + 1) + 24) * 2;
-#define WM_SP1(NK, NMT)                                                                                        \
-  hipLaunchKernelGGL((small_p1_kernel<T, NK, NMT>), grid, block, lds, p.stream, (const uint16_t *)x.data,      \
+#define WM_SP1(NK, NYT)                                                                                      \
+  hipLaunchKernelGGL((small_p1_kernel<T, NK, NYT>), grid, block, lds, p.stream, (const uint16_t *)x.data,      \
                      (const uint16_t *)y.data, (uint16_t *)c.data, (int)p.B, (int)p.M, (int)p.w, nblk, x.sb,   \
                      x.sr, y.sb, y.sr, c.sb)
-#define WM_SP1_N(NMT)                    \
+#define WM_SP1_N(NYT)                    \
   switch (p.N / 16) {                    \
-    case 1: WM_SP1(1, NMT); break;       \
-    case 2: WM_SP1(2, NMT); break;       \
-    case 3: WM_SP1(3, NMT); break;       \
-    case 4: WM_SP1(4, NMT); break;       \
-    case 5: WM_SP1(5, NMT); break;       \
-    case 6: WM_SP1(6, NMT); break;       \
-    case 7: WM_SP1(7, NMT); break;       \
-    default: WM_SP1(8, NMT); break;      \
+    case 1: WM_SP1(1, NYT); break;       \
+    case 2: WM_SP1(2, NYT); break;       \
+    case 3: WM_SP1(3, NYT); break;       \
+    case 4: WM_SP1(4, NYT); break;       \
+    case 5: WM_SP1(5, NYT); break;       \
+    case 6: WM_SP1(6, NYT); break;       \
+    case 7: WM_SP1(7, NYT); break;       \
+    default: WM_SP1(8, NYT); break;      \
   }
-  if (p.w <= 16) {
-    WM_SP1_N(3)
+  if (p.w <= 8) {  // 16-row tiles of Y that cover 64 + 2w rows
+    WM_SP1_N(5)
+  } else if (p.w <= 16) {
+    WM_SP1_N(6)
+  } else if (p.w <= 24) {
+    WM_SP1_N(7)
   } else {
-    WM_SP1_N(4)
+    WM_SP1_N(8)
   }
 #undef WM_SP1_N
 #undef WM_SP1

@@ -15,7 +15,7 @@
 // as one flat image, the Y rows they reach row-major, zero outside the sequence); the result
 // leaves as 16-byte non-temporal stores, consecutive threads on consecutive pieces of a row.
 // The band-out product  P1  band[i,j] = sum_h X[i,h] Y[i+j-w,h]  gets the same treatment (float32 up
-// to w = 14; 16-bit only for w <= 2, beyond that the narrow-band MFMA kernel is faster): X and Y rows
+// to w = 14; for 16-bit storage the narrow-band MFMA kernel is faster at every w): X and Y rows
 // in LDS, one thread per band entry, consecutive threads on consecutive entries of the flat band.  One barrier per workgroup; no atomics.
 #include "wm_mfma_common.hpp"
 
@@ -30,10 +30,6 @@ constexpr int VECTOR_MAX_W = WM_VECTOR_MAX_W;
 #define WM_VECTOR_F32_MAX_W 14
 #endif
 constexpr int VECTOR_F32_MAX_W = WM_VECTOR_F32_MAX_W;
-#ifndef WM_VECTOR_OUT_MAX_W
-#define WM_VECTOR_OUT_MAX_W 2
-#endif
-constexpr int VECTOR_OUT_MAX_W = WM_VECTOR_OUT_MAX_W;  // 16-bit band-out product
 typedef float f32x4v __attribute__((ext_vector_type(4)));
 
 // A 16-bit storage value, and the two values of a dword, as floats.
@@ -352,7 +348,7 @@ bool band_contiguous(const View &v, int64_t W) { return v.sc == 1 && v.sr == W &
 }  // namespace
 
 // 16-bit: band-in products up to w = 3 (61-71 us against 73-86 us for the narrow-band MFMA kernels at
-// B96 M16384 N64; those win from w = 4 on); the band-out product at w <= 2 (79-94 us against 96-98 us).
+// B96 M16384 N64; those win from w = 4 on); the band-out product never (86-92 us against 80 us at w = 1, 2).
 // float32: every window up to VECTOR_F32_MAX_W, all three products.
 bool vector_supports(int op, int64_t M, int64_t N, int64_t w, int dtype) {
   if (op < 1 || op > 3 || M < 1 || M > (1 << 30) || w < 1) return false;
@@ -362,16 +358,14 @@ bool vector_supports(int op, int64_t M, int64_t N, int64_t w, int dtype) {
   }
   if (dtype != WM_DTYPE_BF16 && dtype != WM_DTYPE_F16) return false;
   if (N < 16 || N > 128 || N % 16 != 0) return false;
-  if (op == 1) return w <= VECTOR_OUT_MAX_W && vector_out_lds(w, N, dtype) <= 65536;
+  if (op == 1) return false;  // 16-bit band-out: the narrow-band MFMA kernel is faster at every w
   return w <= VECTOR_MAX_W && vector_lds(w, N, dtype) <= 65536;
 }
 
 bool try_launch_vector_p1(const Problem &p, const View &x, const View &y, const View &c, hipError_t *err) {
   if (!vector_supports(1, p.M, p.N, p.w, p.dtype)) return false;
   if (!fast_layout(x, p.dtype) || !fast_layout(y, p.dtype) || c.sc != 1 || c.sr != 2 * p.w + 1) return false;
-  *err = p.dtype == WM_DTYPE_BF16  ? launch_vector_out<bf16_t>(p, x, y, c)
-         : p.dtype == WM_DTYPE_F16 ? launch_vector_out<f16_t>(p, x, y, c)
-                                   : launch_vector_out<f32_t>(p, x, y, c);
+  *err = launch_vector_out<f32_t>(p, x, y, c);
   return true;
 }
 

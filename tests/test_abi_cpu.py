@@ -70,7 +70,7 @@ def test_kernel_choice_names():
     assert L.wm_kernel_choice(2, 96, 16384, 64, 1, 2, 1, 0) == b"vector_p2"
     assert L.wm_kernel_choice(3, 96, 16384, 64, 3, 1, 1, 0) == b"vector_p3"
     assert L.wm_kernel_choice(1, 96, 16384, 64, 7, 1, 1, 0) == b"narrow_p1"
-    assert L.wm_kernel_choice(1, 96, 16384, 64, 2, 2, 1, 0) == b"vector_p1"
+    assert L.wm_kernel_choice(1, 96, 16384, 64, 2, 2, 1, 0) == b"narrow_p1"
     assert L.wm_kernel_choice(1, 96, 16384, 64, 3, 2, 1, 0) == b"narrow_p1"
     assert L.wm_kernel_choice(2, 96, 16384, 64, 7, 2, 1, abi.NO_NARROW_BAND) == b"strided_p2"
     # float32: all three products on the vector ALU up to w = 14, the float32 MFMA kernels beyond
