@@ -21,9 +21,9 @@ from .window_matmul import unwindow_matmul, window_matmul
 
 def _chain_is_faster(window_size: int) -> bool:
     """Windows at which a training step is faster through the separate ops than through the fused
-    kernels (measured at B96 M16384 N64 bf16: 0.48-0.64 ms against 0.67-0.75 ms up to w = 12, equal
-    at w = 13, 0.68-1.08 ms against 0.67-0.69 ms from w = 14 to 32)."""
-    return window_size <= 12
+    kernels (measured at B96 M16384 N64 bf16: 0.48-0.66 ms against 0.67-0.75 ms up to w = 14, equal
+    at w = 15, 0.71-1.08 ms against 0.67-0.69 ms from w = 16 to 32)."""
+    return window_size <= 14
 
 
 class WindowAttentionFunc(torch.autograd.Function):

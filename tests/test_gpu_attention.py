@@ -267,7 +267,7 @@ def test_narrow_window_training_goes_through_the_separate_ops(device):
     with torch.no_grad():
         want = window_attention(q, k, v, 8)          # fused one-pass forward
     qq, kk, vv = (t.clone().requires_grad_(True) for t in (q, k, v))
-    out = window_attention(qq, kk, vv, 8)             # separate ops (w <= 12 and gradients wanted)
+    out = window_attention(qq, kk, vv, 8)             # separate ops (w <= 14 and gradients wanted)
     assert "UnwindowMatmulFuncBackward" in _graph_nodes(out)
     torch.testing.assert_close(out.float(), want.float(), **TOL)
     out.backward(go)
@@ -275,5 +275,5 @@ def test_narrow_window_training_goes_through_the_separate_ops(device):
     for x, y in zip((qq.grad, kk.grad, vv.grad), want_g):
         close(x, y)
     assert "UnwindowMatmulFuncBackward" in _graph_nodes(window_attention(qq, kk, vv, 12))
-    for w in (13, 16):  # the fused kernels win there
+    for w in (16, 20):  # the fused kernels win there
         assert "WindowAttentionFuncBackward" in _graph_nodes(window_attention(qq, kk, vv, w))
