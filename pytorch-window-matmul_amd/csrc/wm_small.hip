@@ -136,6 +136,110 @@ __global__ __launch_bounds__(kThreads) void small_p1_kernel(const uint16_t *__re
 }
 
 // ------------------------------------------------------------------------------------------
+// P1 narrow, float32: the same kernel on v_mfma_f32_16x16x4_f32.  A lane fetches 16 bytes of its row
+// (columns 16 ks + 4 (lane / 16) ..+3) and element e of that piece feeds MFMA (ks, e): the contraction
+// is split into groups of four columns {16 ks + 4 q + e : q = 0..3}, the same for both operands, so
+// no value ever changes lanes.  The band image holds floats; quads are 16 bytes.
+// ------------------------------------------------------------------------------------------
+template <int NK, int NYT>  // N = 16 NK; NYT 16-row tiles of Y cover 64 + 2w rows
+__global__ __launch_bounds__(kThreads) void small_p1_f32_kernel(const float *__restrict__ X,
+                                                                const float *__restrict__ Y,
+                                                                float *__restrict__ C, int B, int M, int w, int nblk,
+                                                                int64_t xsb, int64_t xsr, int64_t ysb, int64_t ysr,
+                                                                int64_t csb) {
+  constexpr int ROWS = 256;  // band rows per workgroup, 64 per wave
+  extern __shared__ __attribute__((aligned(16))) float flat_f32[];  // 4 + ROWS * W (+ slack) elements
+
+  int b, blk;
+  if (!decode_block(nblk, B, &b, &blk)) return;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int W = 2 * w + 1;
+  const int i0 = blk * ROWS, iw0 = i0 + 64 * wave;
+  const int nrows = min(ROWS, M - i0);
+  float *Cb = C + (int64_t)b * csb + (int64_t)i0 * W;
+  const int delta = (int)((reinterpret_cast<uintptr_t>(Cb) >> 2) & 3);  // elements past a 16-byte boundary
+  const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
+
+  if (iw0 < M) {
+    const int l16 = lane & 15, kq = lane >> 4;
+    f32x4 xop[4][NK], yop[NYT][NK];
+    const float *Xb = X + (int64_t)b * xsb, *Yb = Y + (int64_t)b * ysb;
+#pragma unroll
+    for (int rb = 0; rb < 4; ++rb) {
+      const int i = iw0 + 16 * rb + l16;
+#pragma unroll
+      for (int ks = 0; ks < NK; ++ks)
+        xop[rb][ks] = *reinterpret_cast<const f32x4 *>(i < M ? Xb + (int64_t)i * xsr + 16 * ks + 4 * kq : X);
+    }
+#pragma unroll
+    for (int t = 0; t < NYT; ++t) {
+      const int c = iw0 - w + 16 * t + l16;
+#pragma unroll
+      for (int ks = 0; ks < NK; ++ks)
+        yop[t][ks] = *reinterpret_cast<const f32x4 *>((c >= 0) & (c < M) ? Yb + (int64_t)c * ysr + 16 * ks + 4 * kq : Y);
+    }
+#pragma unroll
+    for (int rb = 0; rb < 4; ++rb) {
+      const int i = iw0 + 16 * rb + l16;
+#pragma unroll
+      for (int ks = 0; ks < NK; ++ks) xop[rb][ks] = i < M ? xop[rb][ks] : zero;
+    }
+#pragma unroll
+    for (int t = 0; t < NYT; ++t) {
+      const int c = iw0 - w + 16 * t + l16;
+#pragma unroll
+      for (int ks = 0; ks < NK; ++ks) yop[t][ks] = (c >= 0) & (c < M) ? yop[t][ks] : zero;
+    }
+
+    float *img = flat_f32 + delta + (64 * wave) * W;
+    // image index of entry (r, j) is delta + 2w r + c_rel, c_rel a multiple of 4: 16-byte aligned quads
+    const bool quad_aligned = (w % 2 == 0) && delta == 0;
+#pragma unroll
+    for (int rb = 0; rb < 4; ++rb) {
+#pragma unroll
+      for (int t = 0; t < NYT; ++t) {
+        if (16 * (t - rb) + 15 < 0 || 16 * (t - rb) - 15 > 2 * w) continue;
+        f32x4 acc = zero;
+#pragma unroll
+        for (int ks = 0; ks < NK; ++ks)
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            acc = __builtin_amdgcn_mfma_f32_16x16x4f32(yop[t][ks][e], xop[rb][ks][e], acc, 0, 0, 0);
+        // acc[v]: c_rel = 16 t + 4 (lane / 16) + v, r_rel = 16 rb + lane % 16
+        const int r_rel = 16 * rb + l16, c_rel = 16 * t + 4 * kq;
+        float *row = img + r_rel * W;
+        const int j = c_rel - r_rel;
+        const int c = iw0 - w + c_rel;
+        if (quad_aligned && j >= 0 && j + 3 <= 2 * w && c >= 0 && c + 3 < M) {
+          *reinterpret_cast<f32x4 *>(row + j) = acc;
+        } else if (j + 3 >= 0 && j <= 2 * w) {
+#pragma unroll
+          for (int v = 0; v < 4; ++v)  // entries outside the sequence are +0.0 by definition
+            if (j + v >= 0 && j + v <= 2 * w) row[j + v] = (c + v >= 0 && c + v < M) ? acc[v] : 0.f;
+        }
+      }
+    }
+  }
+  __syncthreads();
+
+  // flat image -> HBM: chunk q holds image elements [4q, 4q+4), i.e. band elements [4q - delta, ...)
+  const int n_el = nrows * W;
+  const int chunks = (delta + n_el + 3) >> 2;
+  for (int q = tid; q < chunks; q += kThreads) {
+    const f32x4 v = *reinterpret_cast<const f32x4 *>(flat_f32 + 4 * q);
+    const int first = 4 * q - delta;
+    float *dst = Cb + first;
+    if (first >= 0 && first + 4 <= n_el) {
+      __builtin_nontemporal_store(v, reinterpret_cast<f32x4 *>(dst));
+    } else {
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        if (first + e >= 0 && first + e < n_el) dst[e] = v[e];
+    }
+  }
+}
+
+// ------------------------------------------------------------------------------------------
 // Band rows for windows that are not a multiple of 4.  The MFMA reads of the band-in kernels
 // need an image whose 8-column groups are 16-byte aligned in every row, i.e. a row pitch of
 // 1 (mod 8) elements, which the flat band has only when w % 4 == 0.  For the other windows the
@@ -489,6 +593,40 @@ hipError_t launch_small_p1(const Problem &p, const View &x, const View &y, const
   return hipGetLastError();
 }
 
+// float32 band-out kernel: N a multiple of 16 up to 64 (the operands live in registers), w up to
+// SMALL_F32_MAX_W (the float image of 256 band rows must fit 64 KB of LDS).
+#ifndef WM_SMALL_F32_MAX_W
+#define WM_SMALL_F32_MAX_W 31
+#endif
+hipError_t launch_small_p1_f32(const Problem &p, const View &x, const View &y, const View &c) {
+  const int nblk = (int)((p.M + 255) / 256);
+  const dim3 grid(small_grid(p.B, nblk)), block(kThreads);
+  const size_t lds = (size_t)(256 * (2 * p.w + 1) + 12) * 4;
+#define WM_SPF(NK, NYT)                                                                                      \
+  hipLaunchKernelGGL((small_p1_f32_kernel<NK, NYT>), grid, block, lds, p.stream, (const float *)x.data,      \
+                     (const float *)y.data, (float *)c.data, (int)p.B, (int)p.M, (int)p.w, nblk, x.sb, x.sr, \
+                     y.sb, y.sr, c.sb)
+#define WM_SPF_N(NYT)                    \
+  switch (p.N / 16) {                    \
+    case 1: WM_SPF(1, NYT); break;       \
+    case 2: WM_SPF(2, NYT); break;       \
+    case 3: WM_SPF(3, NYT); break;       \
+    default: WM_SPF(4, NYT); break;      \
+  }
+  if (p.w <= 8) {
+    WM_SPF_N(5)
+  } else if (p.w <= 16) {
+    WM_SPF_N(6)
+  } else if (p.w <= 24) {
+    WM_SPF_N(7)
+  } else {
+    WM_SPF_N(8)
+  }
+#undef WM_SPF_N
+#undef WM_SPF
+  return hipGetLastError();
+}
+
 // Window the LDS images of the band-in kernels are laid out for: w itself or the next multiple of 4.
 int64_t image_window(int64_t w) { return (w + 3) & ~(int64_t)3; }
 
@@ -574,7 +712,12 @@ bool band_contiguous(const View &v, int64_t W) { return v.sc == 1 && v.sr == W &
 
 }  // namespace
 
+bool small_f32_p1_supports(int64_t M, int64_t N, int64_t w) {
+  return M >= 1 && M <= (1 << 30) && N >= 16 && N <= 64 && N % 16 == 0 && w >= 1 && w <= WM_SMALL_F32_MAX_W;
+}
+
 bool small_supports(int op, int64_t M, int64_t N, int64_t w, int dtype) {
+  if (dtype == WM_DTYPE_F32) return op == 1 && small_f32_p1_supports(M, N, w);
   if (!small_shape_ok(M, N, w, dtype)) return false;
   if (op == 1) return true;
   if (op == 2) {
@@ -595,6 +738,10 @@ bool small_supports(int op, int64_t M, int64_t N, int64_t w, int dtype) {
 bool try_launch_small_p1(const Problem &p, const View &x, const View &y, const View &c, hipError_t *err) {
   if (!small_supports(1, p.M, p.N, p.w, p.dtype)) return false;
   if (!fast_layout(x, p.dtype) || !fast_layout(y, p.dtype) || !band_contiguous(c, 2 * p.w + 1)) return false;
+  if (p.dtype == WM_DTYPE_F32) {
+    *err = launch_small_p1_f32(p, x, y, c);
+    return true;
+  }
   *err = p.dtype == WM_DTYPE_BF16 ? launch_small_p1<bf16_t>(p, x, y, c) : launch_small_p1<f16_t>(p, x, y, c);
   return true;
 }

@@ -73,9 +73,14 @@ def test_kernel_choice_names():
     assert L.wm_kernel_choice(1, 96, 16384, 64, 2, 2, 1, 0) == b"narrow_p1"
     assert L.wm_kernel_choice(1, 96, 16384, 64, 3, 2, 1, 0) == b"narrow_p1"
     assert L.wm_kernel_choice(2, 96, 16384, 64, 7, 2, 1, abi.NO_NARROW_BAND) == b"strided_p2"
-    # float32: all three products on the vector ALU up to w = 14, the float32 MFMA kernels beyond
+    # float32: band-in products on the vector ALU up to w = 14, the float32 MFMA kernels beyond; the
+    # band-out product on the narrow-band MFMA kernel up to w = 31 when N is a multiple of 16 up to 64
     assert L.wm_kernel_choice(2, 96, 16384, 64, 3, 0, 1, 0) == b"vector_p2"
-    assert L.wm_kernel_choice(1, 2, 128, 64, 4, 0, 1, 0) == b"vector_p1"
+    assert L.wm_kernel_choice(1, 2, 128, 64, 4, 0, 1, 0) == b"narrow_p1"
+    assert L.wm_kernel_choice(1, 2, 128, 48, 31, 0, 1, 0) == b"narrow_p1"
+    assert L.wm_kernel_choice(1, 2, 128, 64, 32, 0, 1, 0) == b"f32_mfma_p1"
+    assert L.wm_kernel_choice(1, 2, 128, 128, 4, 0, 1, 0) == b"vector_p1"
+    assert L.wm_kernel_choice(1, 2, 128, 24, 4, 0, 1, 0) == b"vector_p1"
     assert L.wm_kernel_choice(3, 96, 16384, 64, 14, 0, 1, 0) == b"vector_p3"
     assert L.wm_kernel_choice(3, 96, 16384, 64, 15, 0, 1, 0) == b"f32_mfma_p3"
     assert L.wm_kernel_choice(1, 96, 16384, 64, 8, 0, 1, abi.NO_NARROW_BAND) == b"f32_mfma_p1"

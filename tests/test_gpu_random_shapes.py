@@ -65,21 +65,24 @@ def test_kernel_choice_agrees_with_strided_family(device, dtype, B, M, N, w):
 
 @pytest.mark.parametrize("w", range(1, 33))
 @pytest.mark.parametrize("dtype,B,M,N", [(torch.bfloat16, 3, 300, 64), (torch.float16, 2, 129, 16),
-                                         (torch.bfloat16, 5, 1000, 128), (torch.float16, 2, 31, 96)])
+                                         (torch.bfloat16, 5, 1000, 128), (torch.float16, 2, 31, 96),
+                                         (torch.float32, 3, 300, 64), (torch.float32, 2, 129, 48)])
 def test_every_narrow_window(device, dtype, B, M, N, w):
     """The band-in kernels lay their LDS image out differently for w % 4 == 0 and for the other
-    windows, and the batch stride M (2w + 1) moves the band rows through every alignment."""
+    windows, and the batch stride M (2w + 1) moves the band rows through every alignment; the
+    float32 shapes are the ones the narrow band-out kernel takes (N a multiple of 16 up to 64)."""
     g = torch.Generator().manual_seed(w * 131 + M)
     q, k, v, go = (_randn((B, M, N), g, dtype, device) for _ in range(4))
     a = _randn((B, M, 2 * w + 1), g, dtype, device, 0.2)
     results = []
     for flags in (0, abi.FORCE_STRIDED):
+        att = abi.window_forward(q, k.transpose(1, 2), w, flags)
         out = abi.unwindow_forward(a, v, w, flags)
         ga, gv = abi.unwindow_backward(a, v, w, go, flags)
         gq, gk = abi.window_backward(q, k.transpose(1, 2), w, a, flags)
-        results.append(dict(unwindow_fwd=out, grad_a=ga, grad_v=gv, grad_q=gq, grad_k=gk))
+        results.append(dict(window_fwd=att, unwindow_fwd=out, grad_a=ga, grad_v=gv, grad_q=gq, grad_k=gk))
     for name in results[0]:
-        _assert_close(results[0][name], results[1][name], 2e-2, name)
+        _assert_close(results[0][name], results[1][name], 1e-3 if dtype == torch.float32 else 2e-2, name)
 
 
 ATTENTION_CASES = _draw(2, 40, [16, 32, 48, 64, 80, 96, 112, 128], [torch.bfloat16, torch.float16])
