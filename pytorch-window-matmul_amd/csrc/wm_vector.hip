@@ -15,7 +15,8 @@
 // as one flat image, the Y rows they reach row-major, zero outside the sequence); the result
 // leaves as 16-byte non-temporal stores, consecutive threads on consecutive pieces of a row.
 // The band-out product  P1  band[i,j] = sum_h X[i,h] Y[i+j-w,h]  gets the same treatment (float32 up
-// to w = 14; for 16-bit storage the narrow-band MFMA kernel is faster at every w): X and Y rows
+// to w = 14 where the narrow-band MFMA kernel does not apply, i.e. N not a multiple of 16 or above
+// 64; for 16-bit storage that kernel is faster at every w): X and Y rows
 // in LDS, one thread per band entry, consecutive threads on consecutive entries of the flat band.  One barrier per workgroup; no atomics.
 #include "wm_mfma_common.hpp"
 
