@@ -556,6 +556,16 @@ bool small_shape_ok(int64_t M, int64_t N, int64_t w, int dtype) {
   if (N < 16 || N > 128 || N % 16 != 0) return false;
   return M >= 1 && M <= (1 << 30) && w >= 1 && w <= SMALL_MAX_W;
 }
+// The band-out kernel reaches further when its operands are small enough for the registers: the
+// image of 256 band rows fits 64 KB of LDS up to w = 63.
+#ifndef WM_SMALL_P1_MAX_W
+#define WM_SMALL_P1_MAX_W 63
+#endif
+bool small_p1_shape_ok(int64_t M, int64_t N, int64_t w, int dtype) {
+  if (dtype != WM_DTYPE_BF16 && dtype != WM_DTYPE_F16) return false;
+  if (N < 16 || N > 128 || N % 16 != 0) return false;
+  return M >= 1 && M <= (1 << 30) && w >= 1 && w <= (N <= 64 ? WM_SMALL_P1_MAX_W : SMALL_MAX_W);
+}
 
 unsigned small_grid(int64_t B, int64_t nblk) { return (unsigned)(((B + 7) / 8) * 8 * nblk); }
 
@@ -585,8 +595,22 @@ hipError_t launch_small_p1(const Problem &p, const View &x, const View &y, const
     WM_SP1_N(6)
   } else if (p.w <= 24) {
     WM_SP1_N(7)
-  } else {
+  } else if (p.w <= 32) {
     WM_SP1_N(8)
+  } else {  // N <= 64 only
+#define WM_SP1_W(NYT)                    \
+  switch (p.N / 16) {                    \
+    case 1: WM_SP1(1, NYT); break;       \
+    case 2: WM_SP1(2, NYT); break;       \
+    case 3: WM_SP1(3, NYT); break;       \
+    default: WM_SP1(4, NYT); break;      \
+  }
+    if (p.w <= 48) {
+      WM_SP1_W(10)
+    } else {
+      WM_SP1_W(12)
+    }
+#undef WM_SP1_W
   }
 #undef WM_SP1_N
 #undef WM_SP1
@@ -718,8 +742,8 @@ bool small_f32_p1_supports(int64_t M, int64_t N, int64_t w) {
 
 bool small_supports(int op, int64_t M, int64_t N, int64_t w, int dtype) {
   if (dtype == WM_DTYPE_F32) return op == 1 && small_f32_p1_supports(M, N, w);
+  if (op == 1) return small_p1_shape_ok(M, N, w, dtype);
   if (!small_shape_ok(M, N, w, dtype)) return false;
-  if (op == 1) return true;
   if (op == 2) {
     // the two LDS images must fit the default 64 KB dynamic limit; wider cases go to the wide-band family
     const int64_t NT = (N + 31) / 32;

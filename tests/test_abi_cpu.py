@@ -66,6 +66,12 @@ def test_kernel_choice_names():
     assert L.wm_kernel_choice(2, 96, 16384, 64, 32, 2, 1, 0) == b"narrow_p2"  # 32 rows per wave still fit LDS
     assert L.wm_kernel_choice(3, 96, 16384, 128, 32, 2, 1, 0) == b"mfma_p3"   # images beyond 64 KB of LDS
     assert L.wm_kernel_choice(1, 96, 16384, 64, 8, 2, 1, abi.NO_NARROW_BAND) == b"mfma_p1"
+    # the band-out kernel of the narrow family reaches w = 63 while the operands fit the registers (N <= 64)
+    assert L.wm_kernel_choice(1, 96, 16384, 64, 48, 2, 1, 0) == b"narrow_p1"
+    assert L.wm_kernel_choice(1, 96, 16384, 48, 63, 1, 1, 0) == b"narrow_p1"
+    assert L.wm_kernel_choice(1, 96, 16384, 64, 64, 2, 1, 0) == b"mfma_p1"
+    assert L.wm_kernel_choice(1, 96, 16384, 128, 48, 2, 1, 0) == b"mfma_p1"
+    assert L.wm_kernel_choice(2, 96, 16384, 64, 48, 2, 1, 0) == b"mfma_p2"
     # the narrowest windows (w <= 3, not enough terms for a matrix pipe): vector-ALU band-in kernels
     assert L.wm_kernel_choice(2, 96, 16384, 64, 1, 2, 1, 0) == b"vector_p2"
     assert L.wm_kernel_choice(3, 96, 16384, 64, 3, 1, 1, 0) == b"vector_p3"

@@ -33,6 +33,8 @@ EDGE = [
     (2, 600, 128, 16), (2, 515, 80, 20), (1, 300, 64, 7), (2, 260, 48, 28), (1, 257, 64, 8), (2, 1030, 64, 12),
     # windows that are not a multiple of 4 (band rows re-pitched on their way into LDS), odd batch strides
     (3, 201, 64, 13), (2, 150, 32, 22), (3, 141, 128, 27), (2, 90, 16, 5), (3, 171, 96, 30), (2, 400, 64, 9),
+    # windows between 33 and 63 at N <= 64: band-out product on the narrow-band kernel, band-in on the wide-band ones
+    (2, 300, 64, 40), (3, 201, 32, 63), (2, 150, 48, 57), (1, 700, 16, 33),
 ]
 CASES = REF_GRID + EDGE
 DTYPES = [torch.float32, torch.bfloat16, torch.float16, torch.float64]
