@@ -44,11 +44,12 @@ hipError_t launch_strided_p3(const Problem &p, const View &a, const View &y, con
 bool try_launch_mfma_p1(const Problem &p, const View &x, const View &y, const View &c, hipError_t *err);
 bool try_launch_mfma_p2(const Problem &p, const View &a, const View &y, const View &c, hipError_t *err);
 bool try_launch_mfma_p3(const Problem &p, const View &a, const View &y, const View &c, hipError_t *err);
-// Narrow-band family (w <= 32; P2 and P3 while their LDS images fit 64 KB; P1 also in float32).
+// Narrow-band family (w <= 32; P2 and P3 while their LDS images fit 64 KB; float32 at N <= 64).
 bool try_launch_small_p1(const Problem &p, const View &x, const View &y, const View &c, hipError_t *err);
 bool try_launch_small_p2(const Problem &p, const View &a, const View &y, const View &c, hipError_t *err);
 bool try_launch_small_p3(const Problem &p, const View &a, const View &y, const View &c, hipError_t *err);
 bool small_supports(int op, int64_t M, int64_t N, int64_t w, int dtype);
+bool small_f32_in_supports(int64_t M, int64_t N, int64_t w);  // float32 band-in kernels of the narrow-band family
 bool small_f32_p1_supports(int64_t M, int64_t N, int64_t w);  // float32 band-out kernel of the narrow-band family
 // Vector-ALU kernels for the narrowest windows: 16-bit up to w = 3 (band-in) and w = 2 (band-out),
 // float32 up to w = 14 (the band-out product only where the narrow-band float32 kernel does not apply).

@@ -1,4 +1,5 @@
-// Narrow-band kernels (w <= 32) for 16-bit storage on gfx950.
+// Narrow-band kernels (w <= 32) for 16-bit storage on gfx950, and their float32 counterparts on
+// v_mfma_f32_16x16x4_f32 for N <= 64 further down.
 //
 // With a narrow band the whole band of a block of rows is small (256 rows x 17 entries =
 // 8.7 KB at w = 8), the op is a pure stream over Q/K (P1) or V/O (P2), and the dense tiles of
@@ -236,6 +237,138 @@ __global__ __launch_bounds__(kThreads) void small_p1_f32_kernel(const float *__r
       for (int e = 0; e < 4; ++e)
         if (first + e >= 0 && first + e < n_el) dst[e] = v[e];
     }
+  }
+}
+
+// ------------------------------------------------------------------------------------------
+// P2 / P3 narrow, float32:  C[i,h] = sum_j A[i,j] Y[i+j-w,h]   and   C[c,h] = sum_r A[r,c-r+w] Y[r,h]
+// on v_mfma_f32_16x16x4_f32, one template.  A workgroup owns 64 output rows, a wave 16 of them.
+// LDS holds two images, both written element by element on the way in:
+//   * the band rows, re-pitched to an even window wp (row pitch 2wp + 1, entry j at j + wp - w), so
+//     that the four consecutive entries a lane needs are one aligned 16-byte read.  For P3 the
+//     image is that of the transposed band: entry (r, j) goes to row c = r + j - w, column 2w - j,
+//     and everything after the barrier is the same code;
+//   * the Y rows the block reaches, transposed (Yt[h][c]), so that four consecutive sequence
+//     positions of one column are one 16-byte read as well.
+// As in the band-out kernel the contraction is split into groups {16 ks + 4 q + e : q = 0..3}:
+// element e of a lane's two 16-byte reads feeds MFMA (ks, e).
+// ------------------------------------------------------------------------------------------
+template <int NT, bool TRANSPOSED>  // N = 16 NT <= 64
+__global__ __launch_bounds__(kThreads) void small_in_f32_kernel(const float *__restrict__ A,
+                                                                const float *__restrict__ Y,
+                                                                float *__restrict__ C, int B, int M, int w, int nblk,
+                                                                int64_t asb, int64_t ysb, int64_t ysr, int64_t csb,
+                                                                int64_t csr) {
+  constexpr int ROWS = 64, N = 16 * NT;
+  constexpr int MAXC = TRANSPOSED ? 8 : 4;  // aligned 4-float chunks of band rows per thread (checked on the host)
+  extern __shared__ __attribute__((aligned(16))) float lds_f32[];
+  const int W = 2 * w + 1;
+  const int wp = (w + 1) & ~1, pad = wp - w, P = 2 * wp + 1;
+  const int yc = ROWS + 2 * wp + 16;             // sequence positions cv0 .. cv0 + yc - 1 in the Y image
+  const int SYT = (((yc + 3) >> 2) | 1) << 2;    // pitch of a Yt row: SYT / 4 odd keeps 16 rows in 16 bank groups
+  float *aimg = lds_f32;
+  float *yimg = lds_f32 + ROWS * P + 32;
+
+  int b, blk;
+  if (!decode_block(nblk, B, &b, &blk)) return;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int i0 = blk * ROWS;
+  const float *Ab = A + (int64_t)b * asb, *Yb = Y + (int64_t)b * ysb;
+  const int cv0 = i0 - wp;
+
+  // band rows r_s .. r_e, flat: aligned chunks of four floats, all requested before any is used
+  const int r_s = TRANSPOSED ? max(i0 - w, 0) : i0;
+  const int r_e = min(TRANSPOSED ? i0 + ROWS - 1 + w : i0 + ROWS - 1, M - 1);
+  const float *rows = Ab + (int64_t)r_s * W;
+  const int n_el = (r_e - r_s + 1) * W;
+  const int dg = (int)((reinterpret_cast<uintptr_t>(rows) >> 2) & 3);
+  const int n_chunks = (dg + n_el + 3) >> 2;
+  f32x4 band[MAXC];
+#pragma unroll
+  for (int u = 0; u < MAXC; ++u) {
+    const int q = tid + kThreads * u;
+    band[u] = *reinterpret_cast<const f32x4 *>(q < n_chunks ? rows - dg + 4 * q : A);
+  }
+  // Y rows: an instruction takes 16 consecutive positions x 4 consecutive pieces, so that its four
+  // scalar LDS writes are free of bank conflicts (positions run along a Yt row)
+  const int y_items = ((yc + 15) >> 4) * 16 * (N / 4);  // whole blocks of 16 positions; positions >= yc are skipped
+  for (int base = 0; base < y_items; base += 4 * kThreads) {
+    f32x4 yv[4];
+    int yrow[4], ycol[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int q = base + kThreads * u + tid;
+      const int grp = q >> 6, l = q & 63;
+      const int cc = 16 * (grp / NT) + (l & 15), piece = 4 * (grp % NT) + (l >> 4);
+      const int c = cv0 + cc;
+      const bool ok = (q < y_items) & (cc < yc) & (c >= 0) & (c < M);
+      yv[u] = *reinterpret_cast<const f32x4 *>(ok ? Yb + (int64_t)c * ysr + 4 * piece : Y);
+      yrow[u] = (q < y_items) & (cc < yc) ? 4 * piece : -1;
+      ycol[u] = ok ? cc : -1 - cc;  // negative: position outside the sequence, stored as zeros
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      if (yrow[u] < 0) continue;
+      const bool ok = ycol[u] >= 0;
+      const int cc = ok ? ycol[u] : -1 - ycol[u];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) yimg[(yrow[u] + e) * SYT + cc] = ok ? yv[u][e] : 0.f;
+    }
+  }
+  // band chunks -> image
+#pragma unroll
+  for (int u = 0; u < MAXC; ++u) {
+    const int q = tid + kThreads * u;
+    if (q >= n_chunks) continue;
+    const int first = 4 * q - dg;  // flat index (r W + j, r from r_s) of the chunk's element 0
+    const int s0 = max(first, 0);
+    int r = s0 / W, j = s0 - r * W;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const int id = first + e;
+      if (id >= 0 && id < n_el) {
+        if (TRANSPOSED) {
+          const int c = r_s + r + j - w - i0;  // output row, relative to the block
+          if (c >= 0 && c < ROWS) aimg[c * P + 2 * w - j + pad] = band[u][e];
+        } else {
+          aimg[r * P + j + pad] = band[u][e];
+        }
+        if (++j == W) j = 0, ++r;
+      }
+    }
+  }
+  __syncthreads();
+
+  const int r0 = 16 * wave, r = lane & 15, kq = lane >> 4;
+  const int R = r0 + r, i = i0 + R;
+  const int nks = (16 + 2 * wp + 15) >> 4;
+  f32x4 acc[NT];
+#pragma unroll
+  for (int t = 0; t < NT; ++t) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+  // image column off + e of row R is band column j' = off + e - r (j' - pad in the band), contraction
+  // position cv0 + r0 + off + e; element index R P + j' = R 2wp + r0 + off + e
+  const float *trow = aimg + R * 2 * wp + r0 + 4 * kq;
+  const float *yrow0 = yimg + r * SYT + r0 + 4 * kq;
+  for (int ks = 0; ks < nks; ++ks) {
+    const int off = 16 * ks + 4 * kq;
+    f32x4 bop = *reinterpret_cast<const f32x4 *>(trow + 16 * ks);
+    const int pos = cv0 + r0 + off;  // contraction position of element 0
+    const int e_lo = max(pad + r - off, -pos);
+    const int e_hi = i < M ? min(pad + 2 * w + r - off, M - 1 - pos) : -1;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) bop[e] = (e >= e_lo) & (e <= e_hi) ? bop[e] : 0.f;
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+      const f32x4 aop = *reinterpret_cast<const f32x4 *>(yrow0 + 16 * t * SYT + 16 * ks);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(aop[e], bop[e], acc[t], 0, 0, 0);
+    }
+  }
+  // acc[t][v]: column 16 t + 4 (lane / 16) + v of row i
+  if (i < M) {
+    float *crow = C + (int64_t)b * csb + (int64_t)i * csr + 4 * kq;
+#pragma unroll
+    for (int t = 0; t < NT; ++t) __builtin_nontemporal_store(acc[t], reinterpret_cast<f32x4 *>(crow + 16 * t));
   }
 }
 
@@ -651,6 +784,39 @@ hipError_t launch_small_p1_f32(const Problem &p, const View &x, const View &y, c
   return hipGetLastError();
 }
 
+// float32 band-in kernels: N a multiple of 16 up to 64; w limited by the two LDS images.
+// Range (B96 M16384, alternating builds, P2 / P3 in us): against the vector-ALU kernels, which stop at
+// w = 14: N = 64, w = 12: 225 / 245 against 280 / 293, w = 8: 197 / 221 against 204 / 217, w = 4: 203 / 229
+// against 182 / 183; N = 32, w = 12: 111 / 141 against 98 / 128.  Against the float32 MFMA family: N = 64,
+// w = 16: 226 / 247 against 366 / 344, w = 28: 338 / 373 against 441 / 408, w = 31: 413 / 487 against
+// 441 / 410; N = 16, w = 16: 88 / 116 against 208 / 229.
+#ifndef WM_SMALL_F32_IN_MAX_W
+#define WM_SMALL_F32_IN_MAX_W 28
+#endif
+int64_t small_in_f32_min_w(int64_t N) { return N >= 48 ? 12 : 15; }
+size_t small_in_f32_lds(int64_t w, int64_t N) {
+  const int64_t wp = (w + 1) & ~(int64_t)1, yc = 64 + 2 * wp + 16, syt = (((yc + 3) >> 2) | 1) << 2;
+  return (size_t)(64 * (2 * wp + 1) + 32 + N * syt) * 4;
+}
+template <bool TRANSPOSED>
+hipError_t launch_small_in_f32(const Problem &p, const View &a, const View &y, const View &c) {
+  const int nblk = (int)((p.M + 63) / 64);
+  const dim3 grid(small_grid(p.B, nblk)), block(kThreads);
+  const size_t lds = small_in_f32_lds(p.w, p.N);
+#define WM_SIF(NT)                                                                                              \
+  hipLaunchKernelGGL((small_in_f32_kernel<NT, TRANSPOSED>), grid, block, lds, p.stream, (const float *)a.data,  \
+                     (const float *)y.data, (float *)c.data, (int)p.B, (int)p.M, (int)p.w, nblk, a.sb, y.sb,    \
+                     y.sr, c.sb, c.sr)
+  switch (p.N / 16) {
+    case 1: WM_SIF(1); break;
+    case 2: WM_SIF(2); break;
+    case 3: WM_SIF(3); break;
+    default: WM_SIF(4); break;
+  }
+#undef WM_SIF
+  return hipGetLastError();
+}
+
 // Window the LDS images of the band-in kernels are laid out for: w itself or the next multiple of 4.
 int64_t image_window(int64_t w) { return (w + 3) & ~(int64_t)3; }
 
@@ -740,8 +906,14 @@ bool small_f32_p1_supports(int64_t M, int64_t N, int64_t w) {
   return M >= 1 && M <= (1 << 30) && N >= 16 && N <= 64 && N % 16 == 0 && w >= 1 && w <= WM_SMALL_F32_MAX_W;
 }
 
+bool small_f32_in_supports(int64_t M, int64_t N, int64_t w) {
+  // band chunks per thread: 64 rows (P2) or 64 + 2w rows (P3) of 2w + 1 floats, 4 / 8 chunks of 4 floats x 256 threads
+  return M >= 1 && M <= (1 << 30) && N >= 16 && N <= 64 && N % 16 == 0 && w >= small_in_f32_min_w(N) && w <= WM_SMALL_F32_IN_MAX_W &&
+         (64 + 2 * w) * (2 * w + 1) + 6 <= 8 * 4 * 256 && small_in_f32_lds(w, N) <= kSmallLdsLimit;
+}
+
 bool small_supports(int op, int64_t M, int64_t N, int64_t w, int dtype) {
-  if (dtype == WM_DTYPE_F32) return op == 1 && small_f32_p1_supports(M, N, w);
+  if (dtype == WM_DTYPE_F32) return op == 1 ? small_f32_p1_supports(M, N, w) : small_f32_in_supports(M, N, w);
   if (op == 1) return small_p1_shape_ok(M, N, w, dtype);
   if (!small_shape_ok(M, N, w, dtype)) return false;
   if (op == 2) {
@@ -773,6 +945,10 @@ bool try_launch_small_p1(const Problem &p, const View &x, const View &y, const V
 bool try_launch_small_p2(const Problem &p, const View &a, const View &y, const View &c, hipError_t *err) {
   if (!small_supports(2, p.M, p.N, p.w, p.dtype)) return false;
   if (!band_contiguous(a, 2 * p.w + 1) || !fast_layout(y, p.dtype) || !fast_layout(c, p.dtype)) return false;
+  if (p.dtype == WM_DTYPE_F32) {
+    *err = launch_small_in_f32<false>(p, a, y, c);
+    return true;
+  }
   *err = p.dtype == WM_DTYPE_BF16 ? launch_small_p2<bf16_t>(p, a, y, c) : launch_small_p2<f16_t>(p, a, y, c);
   return true;
 }
@@ -780,6 +956,10 @@ bool try_launch_small_p2(const Problem &p, const View &a, const View &y, const V
 bool try_launch_small_p3(const Problem &p, const View &a, const View &y, const View &c, hipError_t *err) {
   if (!small_supports(3, p.M, p.N, p.w, p.dtype)) return false;
   if (!band_contiguous(a, 2 * p.w + 1) || !fast_layout(y, p.dtype) || !fast_layout(c, p.dtype)) return false;
+  if (p.dtype == WM_DTYPE_F32) {
+    *err = launch_small_in_f32<true>(p, a, y, c);
+    return true;
+  }
   *err = p.dtype == WM_DTYPE_BF16 ? launch_small_p3<bf16_t>(p, a, y, c) : launch_small_p3<f16_t>(p, a, y, c);
   return true;
 }

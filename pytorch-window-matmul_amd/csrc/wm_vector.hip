@@ -356,6 +356,7 @@ bool vector_supports(int op, int64_t M, int64_t N, int64_t w, int dtype) {
   if (dtype == WM_DTYPE_F32) {
     if (N < 8 || N > 128 || N % 8 != 0 || w > VECTOR_F32_MAX_W) return false;
     if (op == 1 && small_f32_p1_supports(M, N, w)) return false;  // the MFMA band-out kernel is faster there
+    if (op != 1 && small_f32_in_supports(M, N, w)) return false;  // likewise the MFMA band-in kernels
     return (op == 1 ? vector_out_lds(w, N, dtype) : vector_lds(w, N, dtype)) <= 65536;
   }
   if (dtype != WM_DTYPE_BF16 && dtype != WM_DTYPE_F16) return false;

@@ -87,8 +87,14 @@ def test_kernel_choice_names():
     assert L.wm_kernel_choice(1, 2, 128, 64, 32, 0, 1, 0) == b"f32_mfma_p1"
     assert L.wm_kernel_choice(1, 2, 128, 128, 4, 0, 1, 0) == b"vector_p1"
     assert L.wm_kernel_choice(1, 2, 128, 24, 4, 0, 1, 0) == b"vector_p1"
-    assert L.wm_kernel_choice(3, 96, 16384, 64, 14, 0, 1, 0) == b"vector_p3"
-    assert L.wm_kernel_choice(3, 96, 16384, 64, 15, 0, 1, 0) == b"f32_mfma_p3"
+    assert L.wm_kernel_choice(3, 96, 16384, 64, 11, 0, 1, 0) == b"vector_p3"
+    assert L.wm_kernel_choice(3, 96, 16384, 32, 14, 0, 1, 0) == b"vector_p3"
+    assert L.wm_kernel_choice(3, 96, 16384, 128, 15, 0, 1, 0) == b"f32_mfma_p3"
+    # float32 band-in products on the narrow-band MFMA kernels: N a multiple of 16 up to 64, w = 12 (15) .. 28
+    assert L.wm_kernel_choice(3, 96, 16384, 64, 12, 0, 1, 0) == b"narrow_p3"
+    assert L.wm_kernel_choice(2, 96, 16384, 32, 15, 0, 1, 0) == b"narrow_p2"
+    assert L.wm_kernel_choice(2, 96, 16384, 16, 28, 0, 1, 0) == b"narrow_p2"
+    assert L.wm_kernel_choice(2, 96, 16384, 64, 29, 0, 1, 0) == b"f32_mfma_p2"
     assert L.wm_kernel_choice(1, 96, 16384, 64, 8, 0, 1, abi.NO_NARROW_BAND) == b"f32_mfma_p1"
     assert L.wm_kernel_choice(1, 2, 128, 3, 4, 0, 1, 0) == b"strided_p1"  # N not a multiple of 8
     assert L.wm_kernel_choice(1, 2, 128, 64, 4, 2, 0, 0) == b"strided_p1"  # layout not vector friendly

@@ -35,6 +35,8 @@ EDGE = [
     (3, 201, 64, 13), (2, 150, 32, 22), (3, 141, 128, 27), (2, 90, 16, 5), (3, 171, 96, 30), (2, 400, 64, 9),
     # windows between 33 and 63 at N <= 64: band-out product on the narrow-band kernel, band-in on the wide-band ones
     (2, 300, 64, 40), (3, 201, 32, 63), (2, 150, 48, 57), (1, 700, 16, 33),
+    # float32 at N <= 64, w = 12..28: narrow-band MFMA kernels for all three products
+    (3, 201, 64, 12), (2, 333, 48, 17), (3, 140, 16, 28), (2, 90, 32, 21),
 ]
 CASES = REF_GRID + EDGE
 DTYPES = [torch.float32, torch.bfloat16, torch.float16, torch.float64]

@@ -66,11 +66,12 @@ def test_kernel_choice_agrees_with_strided_family(device, dtype, B, M, N, w):
 @pytest.mark.parametrize("w", range(1, 33))
 @pytest.mark.parametrize("dtype,B,M,N", [(torch.bfloat16, 3, 300, 64), (torch.float16, 2, 129, 16),
                                          (torch.bfloat16, 5, 1000, 128), (torch.float16, 2, 31, 96),
-                                         (torch.float32, 3, 300, 64), (torch.float32, 2, 129, 48)])
+                                         (torch.float32, 3, 300, 64), (torch.float32, 2, 129, 48),
+                                         (torch.float32, 5, 1000, 16), (torch.float32, 2, 65, 32)])
 def test_every_narrow_window(device, dtype, B, M, N, w):
     """The band-in kernels lay their LDS image out differently for w % 4 == 0 and for the other
     windows, and the batch stride M (2w + 1) moves the band rows through every alignment; the
-    float32 shapes are the ones the narrow band-out kernel takes (N a multiple of 16 up to 64)."""
+    float32 shapes are the ones the narrow-band float32 kernels take (N a multiple of 16 up to 64)."""
     g = torch.Generator().manual_seed(w * 131 + M)
     q, k, v, go = (_randn((B, M, N), g, dtype, device) for _ in range(4))
     a = _randn((B, M, 2 * w + 1), g, dtype, device, 0.2)
