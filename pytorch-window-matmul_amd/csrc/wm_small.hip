@@ -89,6 +89,7 @@ __global__ __launch_bounds__(kThreads) void small_p1_kernel(const uint16_t *__re
     // image index of entry (r, j) is delta + r W + j = delta + 2w r + c_rel (mod 4 it is delta when w is
     // even, c_rel being a multiple of 4): then every quad of 4 consecutive entries is 8-byte aligned
     const bool quad_aligned = (w % 2 == 0) && (delta % 4 == 0);
+    const bool pair_aligned = delta % 2 == 0;  // 2w r + c_rel is even
 #pragma unroll
     for (int rb = 0; rb < 4; ++rb) {
 #pragma unroll
@@ -109,6 +110,9 @@ __global__ __launch_bounds__(kThreads) void small_p1_kernel(const uint16_t *__re
         if (quad_aligned && j >= 0 && j + 3 <= 2 * w && seq_all) {
           u32x2 o = {lo, hi};  // whole quad inside band and sequence: one 8-byte LDS write
           *reinterpret_cast<u32x2 *>(row + j) = o;
+        } else if (pair_aligned && j >= 0 && j + 3 <= 2 * w && seq_all) {
+          *reinterpret_cast<uint32_t *>(row + j) = lo;  // odd w: every other row is 4 bytes off the quad grid
+          *reinterpret_cast<uint32_t *>(row + j + 2) = hi;
         } else if (j + 3 >= 0 && j <= 2 * w) {
           if (j >= 0 && j <= 2 * w) row[j] = (c >= 0 && c < M) ? (uint16_t)lo : (uint16_t)0;
           if (j + 1 >= 0 && j + 1 <= 2 * w)
@@ -195,6 +199,7 @@ __global__ __launch_bounds__(kThreads) void small_p1_f32_kernel(const float *__r
     float *img = flat_f32 + delta + (64 * wave) * W;
     // image index of entry (r, j) is delta + 2w r + c_rel, c_rel a multiple of 4: 16-byte aligned quads
     const bool quad_aligned = (w % 2 == 0) && delta == 0;
+    const bool pair_aligned = delta % 2 == 0;  // 2w r + c_rel is even
 #pragma unroll
     for (int rb = 0; rb < 4; ++rb) {
 #pragma unroll
@@ -213,6 +218,9 @@ __global__ __launch_bounds__(kThreads) void small_p1_f32_kernel(const float *__r
         const int c = iw0 - w + c_rel;
         if (quad_aligned && j >= 0 && j + 3 <= 2 * w && c >= 0 && c + 3 < M) {
           *reinterpret_cast<f32x4 *>(row + j) = acc;
+        } else if (pair_aligned && j >= 0 && j + 3 <= 2 * w && c >= 0 && c + 3 < M) {
+          *reinterpret_cast<f32x2 *>(row + j) = f32x2{acc[0], acc[1]};
+          *reinterpret_cast<f32x2 *>(row + j + 2) = f32x2{acc[2], acc[3]};
         } else if (j + 3 >= 0 && j <= 2 * w) {
 #pragma unroll
           for (int v = 0; v < 4; ++v)  // entries outside the sequence are +0.0 by definition
