@@ -9,7 +9,8 @@
  * Conventions
  *   - All pointers are device pointers on the current HIP device; the caller
  *     owns every buffer.  The library allocates nothing, never synchronises and
- *     keeps no mutable state, so it may be called from several host threads.
+ *     keeps no mutable state, so it may be called from several host threads
+ *     (the one exception, wm_window_attention_backward_static, says so below).
  *   - Work is enqueued on `stream` (a hipStream_t passed as void*; NULL is the
  *     legacy default stream) and the call returns as soon as it is enqueued.
  *   - Every operand is a rank-3 view described by a base pointer and ELEMENT
@@ -33,7 +34,7 @@
 extern "C" {
 #endif
 
-#define WM_ABI_VERSION 2
+#define WM_ABI_VERSION 3
 
 typedef enum wm_dtype {
   WM_DTYPE_F32 = 0,
@@ -50,8 +51,9 @@ typedef enum wm_status {
   WM_ERR_BAD_FLAGS = 4,        /* unknown bit set in flags                          */
   WM_ERR_LAUNCH_FAILED = 5,    /* the HIP runtime rejected a kernel launch          */
   WM_ERR_NO_DEVICE_CODE = 6,   /* the library holds no code object for this GPU     */
-  WM_ERR_UNSUPPORTED = 7       /* a fused entry point has no kernel for this shape, dtype or layout;
+  WM_ERR_UNSUPPORTED = 7,      /* a fused entry point has no kernel for this shape, dtype or layout;
                                   nothing was launched: run the chain of the separate ops instead */
+  WM_ERR_SCRATCH_TOO_SMALL = 8 /* wm_window_attention_backward_static: B * M > WM_STATIC_SCRATCH_ROWS */
 } wm_status;
 
 /* Kernel selection.  0 lets the library choose per (shape, dtype, layout). */
@@ -169,6 +171,25 @@ int wm_window_attention_backward(const wm_operand *q, const wm_operand *k, const
                                  const wm_operand *grad_v, float *delta, int64_t B, int64_t M,
                                  int64_t N, int64_t w, double scale, int dtype, unsigned flags,
                                  void *stream);
+
+/* wm_window_attention_backward for callers that cannot allocate device memory (code under HIP
+ * graph capture, tight serving loops, harnesses that forbid hipMalloc): the same kernels and the
+ * same results, with the delta workspace taken from a static device array inside the library
+ * instead of from the caller.  No counterpart in the reference, whose launchers allocate their
+ * outputs themselves (reference cuda/window_matmul_cuda.cu:239-242).
+ *   - Limit: B * M <= WM_STATIC_SCRATCH_ROWS (8 MiB of float32 per GPU, resident from the first
+ *     call on that GPU until the process ends); beyond it WM_ERR_SCRATCH_TOO_SMALL, nothing launched.
+ *   - The call allocates and frees nothing.  The first call on a GPU looks the array's address
+ *     up (hipGetSymbolAddress) and keeps it; make that call outside any stream capture.
+ *   - All calls on one GPU share the one array: calls that may overlap on a GPU (different
+ *     streams, or several host threads) race on it and must be serialised by the caller.
+ *     Nothing in it has to be cleared between calls: every value read was written by the same call. */
+#define WM_STATIC_SCRATCH_ROWS (1 << 21)
+int wm_window_attention_backward_static(const wm_operand *q, const wm_operand *k, const wm_operand *v,
+                                        const wm_operand *o, const float *lse, const wm_operand *grad_o,
+                                        const wm_operand *grad_q, const wm_operand *grad_k,
+                                        const wm_operand *grad_v, int64_t B, int64_t M, int64_t N, int64_t w,
+                                        double scale, int dtype, unsigned flags, void *stream);
 
 /* 1 if the fused kernels exist for this shape, dtype and scale (layout aside), else 0. */
 int wm_window_attention_supported(int64_t M, int64_t N, int64_t w, int dtype, double scale);

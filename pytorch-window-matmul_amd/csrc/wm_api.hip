@@ -2,8 +2,34 @@
 // the mapping of the four ops onto the three banded primitives.
 #include "wm_common.hpp"
 
+#include <mutex>
+
+// Workspace of wm_window_attention_backward_static: the per-row sums the first backward kernel
+// hands to the second.  One copy per GPU the library runs on, held until the process ends.  In
+// host code this name is only a handle for hipGetSymbolAddress, never a device address.
+static __device__ __align__(256) float scratch[WM_STATIC_SCRATCH_ROWS];
+
 namespace wm {
 namespace {
+
+constexpr int kMaxDevices = 64;
+std::mutex scratch_lock;
+float *scratch_ptr[kMaxDevices];  // device address of `scratch` on each GPU, looked up once per GPU
+
+// Address of `scratch` on the current device.
+int static_scratch(float **out) {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return WM_ERR_LAUNCH_FAILED;
+  std::lock_guard<std::mutex> guard(scratch_lock);
+  if (scratch_ptr[dev] == nullptr) {
+    void *p = nullptr;
+    const hipError_t err = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (err != hipSuccess || p == nullptr) return err == hipErrorNoBinaryForGpu ? WM_ERR_NO_DEVICE_CODE : WM_ERR_LAUNCH_FAILED;
+    scratch_ptr[dev] = static_cast<float *>(p);
+  }
+  *out = scratch_ptr[dev];
+  return WM_OK;
+}
 
 int check_common(int64_t B, int64_t M, int64_t N, int64_t w, int dtype, unsigned flags) {
   if (dtype < WM_DTYPE_F32 || dtype > WM_DTYPE_F64) return WM_ERR_BAD_DTYPE;
@@ -173,6 +199,22 @@ int wm_window_attention_backward(const wm_operand *q, const wm_operand *k, const
   return to_status(err);
 }
 
+int wm_window_attention_backward_static(const wm_operand *q, const wm_operand *k, const wm_operand *v,
+                                        const wm_operand *o, const float *lse, const wm_operand *grad_o,
+                                        const wm_operand *grad_q, const wm_operand *grad_k, const wm_operand *grad_v,
+                                        int64_t B, int64_t M, int64_t N, int64_t w, double scale, int dtype,
+                                        unsigned flags, void *stream) {
+  if (int st = check_common(B, M, N, w, dtype, flags)) return st;
+  if (B * M > (int64_t)WM_STATIC_SCRATCH_ROWS) return WM_ERR_SCRATCH_TOO_SMALL;
+  if (B == 0 || M == 0) return WM_OK;
+  // Every row of the workspace that the second kernel reads is written by the first one in the
+  // same call, so nothing has to be cleared between calls.
+  float *delta = nullptr;
+  if (int st = static_scratch(&delta)) return st;
+  return wm_window_attention_backward(q, k, v, o, lse, grad_o, grad_q, grad_k, grad_v, delta, B, M, N, w, scale, dtype,
+                                      flags, stream);
+}
+
 int wm_window_attention_supported(int64_t M, int64_t N, int64_t w, int dtype, double scale) {
   return attention_supports(M, N, w, dtype, scale) ? 1 : 0;
 }
@@ -218,6 +260,7 @@ const char *wm_status_string(int status) {
     case WM_ERR_BAD_FLAGS: return "unknown flag bit";
     case WM_ERR_LAUNCH_FAILED: return "kernel launch failed";
     case WM_ERR_UNSUPPORTED: return "this entry point has no kernel for the given shape, dtype or layout";
+    case WM_ERR_SCRATCH_TOO_SMALL: return "B * M exceeds WM_STATIC_SCRATCH_ROWS, the rows of the library's static workspace";
     case WM_ERR_NO_DEVICE_CODE: return "no device code for this GPU (library is built for gfx950)";
     default: return "unknown status";
   }

@@ -348,7 +348,7 @@ __global__ __launch_bounds__(kThreads, NK8 <= 8 ? 4 : 2) void f32_band_out_kerne
     for (int s = 0; s < YS; ++s) {
       const int c = cb + y_row[s];
       const f32x4 z = {0.f, 0.f, 0.f, 0.f};
-      if (y_row[s] < KC) *reinterpret_cast<f32x4 *>(&y_lds[buf][y_row[s] * SY + y_col[s]]) = (c >= 0) & (c < M) ? yv[s] : z;
+      if (y_row[s] < KC) *reinterpret_cast<f32x4 *>(&y_lds[buf][y_row[s] * SY + y_col[s]]) = ((c >= 0) & (c < M)) ? yv[s] : z;
     }
   };
 

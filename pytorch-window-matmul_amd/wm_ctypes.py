@@ -64,6 +64,8 @@ def lib():
                                                   ctypes.c_int, u32, vp]
         L.wm_window_attention_backward.argtypes = [P, P, P, P, vp, P, P, P, P, vp, i64, i64, i64, i64, ctypes.c_double,
                                                    ctypes.c_int, u32, vp]
+        L.wm_window_attention_backward_static.argtypes = [P, P, P, P, vp, P, P, P, P, i64, i64, i64, i64,
+                                                          ctypes.c_double, ctypes.c_int, u32, vp]
         L.wm_window_attention_supported.argtypes = [i64, i64, i64, ctypes.c_int, ctypes.c_double]
         _LIB = L
     return _LIB
@@ -151,6 +153,19 @@ def attention_forward(q, k, v, w, scale=1.0, mask=False, flags=0, want_lse=True)
                                             float(scale), int(mask), DTYPES[q.dtype], flags, _stream()),
            "wm_window_attention_forward")
     return o, lse
+
+
+STATIC_SCRATCH_ROWS = 1 << 21
+SCRATCH_TOO_SMALL = 8
+
+
+def attention_backward_static(q, k, v, o, lse, go, gq, gk, gv, w, scale=1.0, flags=0):
+    """wm_window_attention_backward_static: outputs are the caller's (None skips one), the workspace the
+    library's static array; the call itself allocates nothing.  Returns the status code."""
+    B, M, N = q.shape
+    return lib().wm_window_attention_backward_static(op(q), op(k), op(v), op(o), ctypes.c_void_p(lse.data_ptr()),
+                                                     op(go), op(gq), op(gk), op(gv), B, M, N, w, float(scale),
+                                                     DTYPES[q.dtype], flags, _stream())
 
 
 def attention_backward(q, k, v, o, lse, go, w, scale=1.0, flags=0, want=(True, True, True)):
