@@ -60,6 +60,7 @@ typedef enum wm_status {
 #define WM_FLAG_FORCE_STRIDED 0x1u   /* always use the strided fallback kernels (A/B testing) */
 #define WM_FLAG_NO_ALIGNED_BAND 0x2u /* MFMA kernels: never use the 16-byte aligned band variant */
 #define WM_FLAG_NO_NARROW_BAND 0x4u  /* never use the narrow-band kernels (MFMA, w <= 63; vector ALU, w <= 14) */
+#define WM_FLAG_NO_LDS_DIRECT 0x8u   /* fused attention: never use the kernels that load chunks straight into LDS */
 
 /* Rank-3 operand: element (b, r, c) lives at data + b*stride_b + r*stride_r + c*stride_c. */
 typedef struct wm_operand {
@@ -158,8 +159,9 @@ int wm_window_attention_forward(const wm_operand *q, const wm_operand *k, const 
 
 /* Backward of wm_window_attention_forward by recomputation: from q, k, v, the forward's o and
  * lse, and the upstream gradient grad_o, writes grad_q, grad_k, grad_v (all (B, M, N) operands,
- * k and grad_k as key rows).  delta is a caller-owned float32 workspace of B * M values (it
- * receives sum_h grad_o * o per row).  The masking choice of the forward is carried by lse and
+ * k and grad_k as key rows).  delta is a caller-owned float32 workspace of 2 * B * M values (the
+ * first kernel leaves sum_h grad_o * o and the rescaled log-sum-exp of every row there for the
+ * second).  The masking choice of the forward is carried by lse and
  * needs no argument here.  Any of grad_q, grad_k, grad_v may be NULL to skip that gradient
  * (grad_q NULL shortens the first kernel to the delta pass, grad_k and grad_v both NULL drop the
  * second).  Up to two kernels are enqueued on the stream; no atomics, so results are
@@ -177,7 +179,7 @@ int wm_window_attention_backward(const wm_operand *q, const wm_operand *k, const
  * same results, with the delta workspace taken from a static device array inside the library
  * instead of from the caller.  No counterpart in the reference, whose launchers allocate their
  * outputs themselves (reference cuda/window_matmul_cuda.cu:239-242).
- *   - Limit: B * M <= WM_STATIC_SCRATCH_ROWS (8 MiB of float32 per GPU, resident from the first
+ *   - Limit: B * M <= WM_STATIC_SCRATCH_ROWS (two float32 per row: 16 MiB per GPU, resident from the first
  *     call on that GPU until the process ends); beyond it WM_ERR_SCRATCH_TOO_SMALL, nothing launched.
  *   - The call allocates and frees nothing.  The first call on a GPU looks the array's address
  *     up (hipGetSymbolAddress) and keeps it; make that call outside any stream capture.

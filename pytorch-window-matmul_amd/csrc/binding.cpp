@@ -278,7 +278,7 @@ window_attention_backward(torch::Tensor q, torch::Tensor k, torch::Tensor v, tor
   if (need_q) gq = torch::empty({B, M, N}, q.options()), f = operand(*gq);
   if (need_k) gk = torch::empty({B, M, N}, q.options()), g = operand(*gk);
   if (need_v) gv = torch::empty({B, M, N}, q.options()), h = operand(*gv);
-  auto delta = torch::empty({B, M}, lse.options());
+  auto delta = torch::empty({2, B, M}, lse.options());  // row sums and log2-scaled log-sum-exp
   wm_operand a = operand(qq), b = operand(kk), c = operand(vv), d = operand(oo), e = operand(go);
   raise_on_error(wm_window_attention_backward(&a, &b, &c, &d, lse.data_ptr<float>(), &e, need_q ? &f : nullptr,
                                               need_k ? &g : nullptr, need_v ? &h : nullptr, delta.data_ptr<float>(),

@@ -4,10 +4,10 @@
 
 #include <mutex>
 
-// Workspace of wm_window_attention_backward_static: the per-row sums the first backward kernel
-// hands to the second.  One copy per GPU the library runs on, held until the process ends.  In
+// Workspace of wm_window_attention_backward_static: the two per-row values the first backward
+// kernel hands to the second.  One copy per GPU the library runs on, held until the process ends.  In
 // host code this name is only a handle for hipGetSymbolAddress, never a device address.
-static __device__ __align__(256) float scratch[WM_STATIC_SCRATCH_ROWS];
+static __device__ __align__(256) float scratch[2 * WM_STATIC_SCRATCH_ROWS];
 
 namespace wm {
 namespace {
@@ -33,7 +33,7 @@ int static_scratch(float **out) {
 
 int check_common(int64_t B, int64_t M, int64_t N, int64_t w, int dtype, unsigned flags) {
   if (dtype < WM_DTYPE_F32 || dtype > WM_DTYPE_F64) return WM_ERR_BAD_DTYPE;
-  if (flags & ~(WM_FLAG_FORCE_STRIDED | WM_FLAG_NO_ALIGNED_BAND | WM_FLAG_NO_NARROW_BAND)) return WM_ERR_BAD_FLAGS;
+  if (flags & ~(WM_FLAG_FORCE_STRIDED | WM_FLAG_NO_ALIGNED_BAND | WM_FLAG_NO_NARROW_BAND | WM_FLAG_NO_LDS_DIRECT)) return WM_ERR_BAD_FLAGS;
   const int64_t lim = 0x7fffffff;
   if (B < 0 || M < 0 || N < 0 || w < 0) return WM_ERR_BAD_SHAPE;
   if (B > lim || M > lim || N > lim || w > (lim - 1) / 2) return WM_ERR_BAD_SHAPE;

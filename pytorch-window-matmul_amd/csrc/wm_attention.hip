@@ -378,6 +378,238 @@ __global__ __launch_bounds__(kThreads, 2) void attention_forward_narrow_kernel(
   }
 }
 
+
+// ---------------------------------------------------------------------------------------------
+// N = 64 and N = 128: key and value chunks go from memory straight into LDS
+// ---------------------------------------------------------------------------------------------
+// Same tiling and arithmetic as attention_forward_kernel.  What differs is how the wavefronts are
+// kept busy:
+//   * K and V chunks are written into LDS by the memory system itself (buffer loads with the lds
+//     modifier, swizzled tiles, see wm_mfma_common.hpp): no staging registers, no LDS stores, no
+//     address arithmetic per chunk (the chunk position is a scalar offset of the load), rows past
+//     the sequence read as zeros, and chunks are requested DEPTH iterations before their use.
+//   * Everything that decides what a wavefront does with a chunk is scalar (the wavefront's first
+//     query is read with readfirstlane), so skipped blocks cost a scalar branch.
+//   * A chunk whose two 32-key blocks both lie inside the wavefront's band is processed as a pair:
+//     both score tiles are formed by two independent MFMA chains, one row maximum serves both, and
+//     the exponentials of one block run on the vector ALU while the matrix pipe multiplies the
+//     other block's probabilities with V.
+template <typename T, int NK, bool MASK>
+__global__ __launch_bounds__(kThreads, NK <= 4 ? 3 : 2) void attention_forward_dma_kernel(
+    const uint16_t *__restrict__ Q, const uint16_t *__restrict__ K, const uint16_t *__restrict__ V,
+    uint16_t *__restrict__ O, float *__restrict__ L, int B, int M, int w, int nblk, float c, int64_t qsb, int64_t qsr,
+    int64_t ksb, int64_t ksr, int64_t vsb, int64_t vsr, int64_t osb, int64_t osr) {
+  constexpr int N = 16 * NK, NB = NK / 2, PPR = 2 * NK, ROWB = 2 * N;  // pieces and bytes per tile row
+  constexpr int STAGES = NK <= 4 ? 3 : 2, DEPTH = STAGES - 1;
+  constexpr int TILE = AT_KC * N;          // elements per tile
+  constexpr int LOADS = 2 * (PPR / 4);     // loads per wavefront and chunk (K and V)
+  static_assert(NK == 4 || NK == 8, "tile rows of 128 or 256 bytes");
+  __shared__ __attribute__((aligned(1024))) uint16_t k_lds[STAGES][TILE];
+  __shared__ __attribute__((aligned(1024))) uint16_t v_lds[STAGES][TILE];
+
+  int b, blk;
+  if (!decode_block(nblk, B, &b, &blk)) return;
+  const int tid = threadIdx.x, lane = tid & 63, half = lane >> 5;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int i0 = blk * AT_TM;
+  const int qw0 = i0 + 32 * wave;     // first query of this wavefront (scalar)
+  const int qi = qw0 + (lane & 31);   // this lane's query
+
+  const u32x4 k_rsrc = make_rsrc(K + (int64_t)b * ksb, (uint32_t)((M - 1) * ksr * 2 + ROWB));
+  const u32x4 v_rsrc = make_rsrc(V + (int64_t)b * vsb, (uint32_t)((M - 1) * vsr * 2 + ROWB));
+  const uint32_t k_voff = dma_lane_offset<PPR>(wave, lane, ksr), v_voff = dma_lane_offset<PPR>(wave, lane, vsr);
+  const uint32_t k_step = (uint32_t)(256 / PPR * ksr * 2), v_step = (uint32_t)(256 / PPR * vsr * 2);
+  const uint32_t k_chunk = (uint32_t)(AT_KC * ksr * 2), v_chunk = (uint32_t)(AT_KC * vsr * 2);
+  auto request = [&](int kc, int stage) {
+    dma_chunk<PPR>(k_rsrc, k_lds[stage], wave, k_voff, k_chunk * (uint32_t)kc, k_step);
+    dma_chunk<PPR>(v_rsrc, v_lds[stage], wave, v_voff, v_chunk * (uint32_t)kc, v_step);
+  };
+
+  const int kc_lo = max(i0 - w, 0) / AT_KC;
+  const int kc_hi = min(i0 + AT_TM - 1 + w, M - 1) / AT_KC;
+#pragma unroll
+  for (int d = 0; d < DEPTH; ++d) request(kc_lo + d, d);
+
+  // B operand of the first product: the wavefront's 32 queries, all of N, in registers
+  u32x4 qf[NK];
+  {
+    const uint16_t *qr = Q + (int64_t)b * qsb + (int64_t)qi * qsr + 8 * half;
+#pragma unroll
+    for (int ks = 0; ks < NK; ++ks) qf[ks] = load_row_chunk(qr + 16 * ks, Q, qi < M);
+  }
+
+  // LDS byte offsets inside a tile.  Key rows as A operand: row lane % 32 of a block, pieces
+  // 2 ks + half; value columns through the transposing read: rows 4 (grp / 2) + s / 4 (+ 8),
+  // 8 bytes at column 32 hb + 16 (grp % 2) + 4 (s % 4).  The swizzle only touches address bits
+  // that the ks / hb terms do not carry into, so those terms are XORed in at the point of use.
+  const int r32 = lane & 31;
+  const uint32_t k_at = (uint32_t)(r32 * ROWB + ((half ^ swz(r32)) << 4));
+  const int s16 = lane & 15, grp = lane >> 4, rowl = 4 * (grp >> 1) + (s16 >> 2);
+  const uint32_t v_at = (uint32_t)(rowl * ROWB + (((2 * (grp & 1) + ((s16 & 3) >> 1)) ^ swz(rowl)) << 4) + 8 * (s16 & 1));
+  typedef s16x4 __attribute__((address_space(3))) * lds_tr_ptr;
+  auto key_operand = [&](const uint16_t *tile, int kb, int ks) {
+    return *reinterpret_cast<const u32x4 *>(reinterpret_cast<const char *>(tile) + 32 * kb * ROWB + (k_at ^ (32 * ks)));
+  };
+  auto value_operand = [&](const uint16_t *tile, int kb, int t, int hb) {
+    const char *p = reinterpret_cast<const char *>(tile) + (32 * kb + 16 * t) * ROWB + (v_at ^ (64 * hb));
+    const u32x2 lo = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr_ptr)(p)));
+    const u32x2 hi = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr_ptr)(p + 8 * ROWB)));
+    const u32x4 r = {lo[0], lo[1], hi[0], hi[1]};
+    return r;
+  };
+
+  f32x16 o[NB];
+#pragma unroll
+  for (int hb = 0; hb < NB; ++hb)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) o[hb][v] = 0.0f;
+  float m_used = -1.0e30f;  // running maximum in log2 units (finite, so that -inf scores give exp2(-inf) = 0)
+  float l_part = 0.0f;      // this lane's share of the running sum
+  const float ninf = -__builtin_huge_valf();
+
+  // The LDS reads of a product are all issued before its first MFMA: left to itself the compiler
+  // reuses one register set for consecutive operands, one LDS latency in front of every MFMA.
+  auto scores = [&](const uint16_t *kt, int kb) {
+    f32x16 s;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) s[v] = 0.0f;
+    u32x4 ka[NK];
+#pragma unroll
+    for (int ks = 0; ks < NK; ++ks) ka[ks] = key_operand(kt, kb, ks);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int ks = 0; ks < NK; ++ks) s = Mma<T>::run(ka[ks], qf[ks], s);
+    return s;
+  };
+  auto block_max = [&](const f32x16 &s) {
+    float bm = s[0];
+#pragma unroll
+    for (int v = 1; v < 16; ++v) bm = fmaxf(bm, s[v]);
+    return bm;
+  };
+  // raises the running maximum to bm (log2 units, already exchanged between the half-waves) when
+  // some row of the wavefront exceeds it by more than kRaiseStep
+  auto raise_to = [&](float bm) {
+    const bool raise = bm > m_used + kRaiseStep;
+    if (__builtin_amdgcn_ballot_w64(raise) != 0) {
+      const float m_new = raise ? bm : m_used;
+      const float alpha = __builtin_amdgcn_exp2f(m_used - m_new);
+      m_used = m_new;
+      l_part *= alpha;
+#pragma unroll
+      for (int hb = 0; hb < NB; ++hb)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) o[hb][v] *= alpha;
+    }
+  };
+  // P^T = exp2(c S^T - m), rounded; row sums over the rounded values; O^T += V_blk^T P^T
+  auto accumulate = [&](const uint16_t *vt, int kb, const f32x16 &s) {
+    u32x4 va[2][NB];  // in flight while the exponentials run
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int hb = 0; hb < NB; ++hb) va[t][hb] = value_operand(vt, kb, t, hb);
+    __builtin_amdgcn_sched_barrier(0);
+    float p[16];
+#pragma unroll
+    for (int v = 0; v < 16; ++v) p[v] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[v], c, -m_used));
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      const u32x4 pf = {Mma<T>::pack2(p[8 * t + 0], p[8 * t + 1]), Mma<T>::pack2(p[8 * t + 2], p[8 * t + 3]),
+                        Mma<T>::pack2(p[8 * t + 4], p[8 * t + 5]), Mma<T>::pack2(p[8 * t + 6], p[8 * t + 7])};
+#pragma unroll
+      for (int d = 0; d < 4; ++d) l_part = Mma<T>::add_pair(pf[d], l_part);
+#pragma unroll
+      for (int hb = 0; hb < NB; ++hb) o[hb] = Mma<T>::run(va[t][hb], pf, o[hb]);
+    }
+  };
+  // accumulator v of a lane: key c0 + 8 (v / 4) + 4 half + v % 4, query qi; offsets first..last are
+  // inside the band and the sequence
+  auto mask_edge = [&](f32x16 &s, int c0) {
+    const int d0 = c0 + 4 * half - qi;
+    const int first = -w - d0, last = min(w - d0, M - 1 - c0 - 4 * half);
+    const int origin = last < first ? 0x100000 : first;
+    const unsigned span = last < first ? 0u : (unsigned)(last - first);
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+      const int ofs = 8 * (v / 4) + v % 4;
+      s[v] = (unsigned)(ofs - origin) <= span ? s[v] : ninf;
+    }
+  };
+
+  int stage = 0;
+  // Start of an iteration: this wavefront's pieces of chunk kc have landed (the DEPTH - 1 younger
+  // chunks may still be in flight); after the barrier so have everyone's, and nobody reads chunk
+  // kc - 1 any more, whose tile takes chunk kc + DEPTH (beyond the sequence: zeros nobody reads).
+  auto open_chunk = [&](int kc) {
+    wait_vmcnt<(DEPTH - 1) * LOADS>();
+    __builtin_amdgcn_s_barrier();
+    int st = stage + DEPTH;
+    st = st >= STAGES ? st - STAGES : st;
+    request(kc + DEPTH, st);
+  };
+  auto close_chunk = [&]() { stage = stage + 1 == STAGES ? 0 : stage + 1; };
+  // chunk with a block that is outside the band or the sequence, or crosses their edge
+  auto edge_chunk = [&](int kc) {
+    open_chunk(kc);
+    const uint16_t *kt = k_lds[stage], *vt = v_lds[stage];
+#pragma unroll
+    for (int kb = 0; kb < 2; ++kb) {
+      const int cb = kc * AT_KC + 32 * kb;
+      if (cb + 31 < qw0 - w || cb > qw0 + 31 + w || cb >= M) continue;  // scalar
+      f32x16 s = scores(kt, kb);
+      mask_edge(s, cb);  // also where the block happens to need no mask: one code path, no register shuffling
+      raise_to(across_halves_max(block_max(s)) * c);
+      accumulate(vt, kb, s);
+    }
+    close_chunk();
+  };
+  // The wavefront's chunks [pair_lo, pair_hi] lie wholly inside its band and the sequence; every
+  // wavefront of the workgroup passes the same number of barriers, whichever loop it is in.
+  const int pair_lo = max(kc_lo, (qw0 + 31 - w + 63) >> 6);
+  const int pair_hi = min(kc_hi, (min(qw0 + w, M - 1) - 63) >> 6);
+  const int lead_end = pair_lo <= pair_hi ? pair_lo : kc_hi + 1;
+  int kc = kc_lo;
+  for (; kc < lead_end; ++kc) edge_chunk(kc);
+  for (; kc <= pair_hi; ++kc) {
+    open_chunk(kc);
+    const uint16_t *kt = k_lds[stage], *vt = v_lds[stage];
+    const f32x16 s0 = scores(kt, 0), s1 = scores(kt, 1);
+    raise_to(across_halves_max(fmaxf(block_max(s0), block_max(s1))) * c);
+    accumulate(vt, 0, s0);
+    accumulate(vt, 1, s1);
+    close_chunk();
+  }
+  for (; kc <= kc_hi; ++kc) edge_chunk(kc);
+
+  float l = across_halves_sum(l_part);
+  if (!MASK) {
+    // Band entries outside the sequence: score 0 each, no value row (scalar test first).
+    if (qw0 < w || qw0 + 31 + w > M - 1) {
+      const int n_out = max(0, w - qi) + max(0, qi + w - (M - 1));
+      if (n_out > 0) {
+        const float m_new = fmaxf(m_used, 0.0f);
+        const float alpha = __builtin_amdgcn_exp2f(m_used - m_new);
+        l = l * alpha + (float)n_out * __builtin_amdgcn_exp2f(-m_new);
+        m_used = m_new;
+#pragma unroll
+        for (int hb = 0; hb < NB; ++hb)
+#pragma unroll
+          for (int v = 0; v < 16; ++v) o[hb][v] *= alpha;
+      }
+    }
+  }
+  if (qi >= M) l = 1.0f;  // rows past the end: keep the arithmetic finite, nothing is stored
+  const float inv = 1.0f / l;
+  if (L != nullptr && half == 0 && qi < M) L[(int64_t)b * M + qi] = (m_used + __builtin_amdgcn_logf(l)) * kLn2F;
+  // The chunks requested past the last one must have landed before their tiles are reused, and
+  // every wavefront must be done with the last chunk: then the key tiles stage the result rows.
+  wait_vmcnt<0>();
+  __builtin_amdgcn_s_barrier();
+  static_assert(4 * RowStage<NB>::ELEMS <= STAGES * TILE, "the four staging areas must fit the key tiles");
+  store_wave_rows<T, NB>(&k_lds[0][0] + wave * RowStage<NB>::ELEMS, o, inv, O + (int64_t)b * osb, osr, qw0, M, N, lane);
+}
+
 template <typename T, int NK>
 hipError_t launch_forward(const Problem &p, const View &q, const View &k, const View &v, const View &o, float *lse,
                           double scale, int mask) {
@@ -401,6 +633,20 @@ hipError_t launch_forward(const Problem &p, const View &q, const View &k, const 
       WM_AT((attention_forward_narrow_kernel<T, NK, 3, true>));
     else
       WM_AT((attention_forward_narrow_kernel<T, NK, 3, false>));
+  } else if constexpr (NK == 4 || NK == 8) {
+    // the buffer loads of the LDS-direct kernel address a batch element with 32-bit byte offsets
+    const int64_t lim = 0x7fffffff;
+    const bool fits = (p.M + 3 * AT_KC) * k.sr * 2 < lim && (p.M + 3 * AT_KC) * v.sr * 2 < lim && k.sr > 0 && v.sr > 0;
+    if (fits && !(p.flags & WM_FLAG_NO_LDS_DIRECT)) {
+      if (mask)
+        WM_AT((attention_forward_dma_kernel<T, NK, true>));
+      else
+        WM_AT((attention_forward_dma_kernel<T, NK, false>));
+    } else if (mask) {
+      WM_AT((attention_forward_kernel<T, NK, true>));
+    } else {
+      WM_AT((attention_forward_kernel<T, NK, false>));
+    }
   } else {
     if (mask)
       WM_AT((attention_forward_kernel<T, NK, true>));

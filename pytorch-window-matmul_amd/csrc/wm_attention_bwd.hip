@@ -373,6 +373,386 @@ __global__ __launch_bounds__(kThreads, NK <= 4 ? 2 : 1) void attention_backward_
   if (dV != nullptr) store_wave_rows<T, NB>(stage, dv, 1.0f, dV + (int64_t)b * dvsb, dvsr, kw0, M, N, lane);
 }
 
+
+// ---------------------------------------------------------------------------------------------
+// N = 64 and N = 128: the streamed tiles go from memory straight into LDS
+// ---------------------------------------------------------------------------------------------
+// Same arithmetic as the two kernels above, organised like attention_forward_dma_kernel
+// (wm_attention.hip): swizzled tiles filled by buffer loads with the lds modifier, requested DEPTH
+// chunks ahead and counted by the kernel itself; scalar control flow; one branch-free loop for the
+// chunks that lie wholly inside a wavefront's band and a general one for the chunks at its edges.
+// The workspace holds two float32 values per row: D = sum_h dO * O at [b * M + i] and the row's
+// log-sum-exp in log2 units at [B * M + b * M + i]; the query kernel writes both, the key kernel
+// streams both.  dS is formed without the factor `scale`, which multiplies the finished dQ and dK.
+constexpr float kLog2e = 1.4426950408889634f;
+
+template <int NK>
+struct BwdTile {
+  static constexpr int N = 16 * NK, NB = NK / 2, PPR = 2 * NK, ROWB = 2 * N, TILE = AB_KC * N;
+  static constexpr int STAGES = NK <= 4 ? 3 : 2, DEPTH = STAGES - 1;
+  typedef s16x4 __attribute__((address_space(3))) * lds_tr_ptr;
+  // byte offsets inside a tile for the two ways a tile is read (see attention_forward_dma_kernel)
+  static __device__ __forceinline__ uint32_t row_at(int lane) {
+    const int r32 = lane & 31, half = lane >> 5;
+    return (uint32_t)(r32 * ROWB + ((half ^ swz(r32)) << 4));
+  }
+  static __device__ __forceinline__ uint32_t tr_at(int lane) {
+    const int s16 = lane & 15, grp = lane >> 4, rowl = 4 * (grp >> 1) + (s16 >> 2);
+    return (uint32_t)(rowl * ROWB + (((2 * (grp & 1) + ((s16 & 3) >> 1)) ^ swz(rowl)) << 4) + 8 * (s16 & 1));
+  }
+  // rows 32 blk + lane % 32 of the tile, pieces 2 ks + half: A operand of a product contracted over N
+  static __device__ __forceinline__ u32x4 rows(const uint16_t *tile, uint32_t at, int blk, int ks) {
+    return *reinterpret_cast<const u32x4 *>(reinterpret_cast<const char *>(tile) + 32 * blk * ROWB + (at ^ (32 * ks)));
+  }
+  // columns 32 hb .. + 31 of rows 32 blk + 16 t .. + 15, transposed: A operand of a product contracted over rows
+  static __device__ __forceinline__ u32x4 cols(const uint16_t *tile, uint32_t at, int blk, int t, int hb) {
+    const char *p = reinterpret_cast<const char *>(tile) + (32 * blk + 16 * t) * ROWB + (at ^ (64 * hb));
+    const u32x2 lo = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr_ptr)(p)));
+    const u32x2 hi = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr_ptr)(p + 8 * ROWB)));
+    const u32x4 r = {lo[0], lo[1], hi[0], hi[1]};
+    return r;
+  }
+};
+
+
+// D and the log-sum-exp in log2 units for the key kernel when grad_q is not wanted.
+template <typename T, int NK>
+__global__ __launch_bounds__(kThreads) void attention_backward_stats_kernel(
+    const uint16_t *__restrict__ O, const uint16_t *__restrict__ dO, const float *__restrict__ L, float *__restrict__ D,
+    int B, int M, int nblk, int64_t osb, int64_t osr, int64_t gsb, int64_t gsr) {
+  int b, blk;
+  if (!decode_block(nblk, B, &b, &blk)) return;
+  const int lane = threadIdx.x & 63, half = lane >> 5;
+  const int qi = blk * AB_TM + 32 * (threadIdx.x >> 6) + (lane & 31);
+  const bool q_ok = qi < M;
+  const uint16_t *gr = dO + (int64_t)b * gsb + (int64_t)qi * gsr + 8 * half;
+  const uint16_t *orow = O + (int64_t)b * osb + (int64_t)qi * osr + 8 * half;
+  float delta = 0.0f;
+#pragma unroll
+  for (int ks = 0; ks < NK; ++ks)
+    delta += dot8<T>(load_row_chunk(gr + 16 * ks, dO, q_ok), load_row_chunk(orow + 16 * ks, O, q_ok));
+  delta = halves_sum(delta);
+  if (q_ok && half == 0) {
+    D[(int64_t)b * M + qi] = delta;
+    D[((int64_t)B + b) * M + qi] = L[(int64_t)b * M + qi] * kLog2e;
+  }
+}
+
+template <typename T, int NK>
+__global__ __launch_bounds__(kThreads, NK <= 4 ? 3 : 1) void attention_backward_query_dma_kernel(
+    const uint16_t *__restrict__ Q, const uint16_t *__restrict__ K, const uint16_t *__restrict__ V,
+    const uint16_t *__restrict__ O, const uint16_t *__restrict__ dO, const float *__restrict__ L,
+    uint16_t *__restrict__ dQ, float *__restrict__ D, int B, int M, int w, int nblk, float scale, int64_t qsb,
+    int64_t qsr, int64_t ksb, int64_t ksr, int64_t vsb, int64_t vsr, int64_t osb, int64_t osr, int64_t gsb, int64_t gsr,
+    int64_t dqsb, int64_t dqsr) {
+  typedef BwdTile<NK> TL;
+  constexpr int N = TL::N, NB = TL::NB, PPR = TL::PPR, ROWB = TL::ROWB, TILE = TL::TILE;
+  constexpr int STAGES = TL::STAGES, DEPTH = TL::DEPTH;
+  constexpr int LOADS = 2 * (PPR / 4);  // loads per wavefront and chunk (K and V)
+  __shared__ __attribute__((aligned(1024))) uint16_t k_lds[STAGES][TILE];
+  __shared__ __attribute__((aligned(1024))) uint16_t v_lds[STAGES][TILE];
+
+  int b, blk;
+  if (!decode_block(nblk, B, &b, &blk)) return;
+  const int tid = threadIdx.x, lane = tid & 63, half = lane >> 5;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int i0 = blk * AB_TM;
+  const int qw0 = i0 + 32 * wave;  // scalar
+  const int qi = qw0 + (lane & 31);
+  const bool q_ok = qi < M;
+  const float c = scale * kLog2e;
+
+  const u32x4 k_rsrc = make_rsrc(K + (int64_t)b * ksb, (uint32_t)((M - 1) * ksr * 2 + ROWB));
+  const u32x4 v_rsrc = make_rsrc(V + (int64_t)b * vsb, (uint32_t)((M - 1) * vsr * 2 + ROWB));
+  const uint32_t k_voff = dma_lane_offset<PPR>(wave, lane, ksr), v_voff = dma_lane_offset<PPR>(wave, lane, vsr);
+  const uint32_t k_step = (uint32_t)(256 / PPR * ksr * 2), v_step = (uint32_t)(256 / PPR * vsr * 2);
+  const uint32_t k_chunk = (uint32_t)(AB_KC * ksr * 2), v_chunk = (uint32_t)(AB_KC * vsr * 2);
+  auto request = [&](int kc, int stage) {
+    dma_chunk<PPR>(k_rsrc, k_lds[stage], wave, k_voff, k_chunk * (uint32_t)kc, k_step);
+    dma_chunk<PPR>(v_rsrc, v_lds[stage], wave, v_voff, v_chunk * (uint32_t)kc, v_step);
+  };
+  const int kc_lo = max(i0 - w, 0) / AB_KC;
+  const int kc_hi = min(i0 + AB_TM - 1 + w, M - 1) / AB_KC;
+#pragma unroll
+  for (int d = 0; d < DEPTH; ++d) request(kc_lo + d, d);
+
+  // stationary side in registers: the query rows and their upstream gradient rows (B operands)
+  u32x4 qf[NK], gf[NK];
+  float delta = 0.0f;
+  {
+    const uint16_t *qr = Q + (int64_t)b * qsb + (int64_t)qi * qsr + 8 * half;
+    const uint16_t *gr = dO + (int64_t)b * gsb + (int64_t)qi * gsr + 8 * half;
+    const uint16_t *orow = O + (int64_t)b * osb + (int64_t)qi * osr + 8 * half;
+#pragma unroll
+    for (int ks = 0; ks < NK; ++ks) {
+      qf[ks] = load_row_chunk(qr + 16 * ks, Q, q_ok);
+      gf[ks] = load_row_chunk(gr + 16 * ks, dO, q_ok);
+      delta += dot8<T>(gf[ks], load_row_chunk(orow + 16 * ks, O, q_ok));
+    }
+  }
+  delta = halves_sum(delta);
+  const float l2 = (q_ok ? L[(int64_t)b * M + qi] : 0.0f) * kLog2e;
+  if (q_ok && half == 0) {
+    D[(int64_t)b * M + qi] = delta;
+    D[((int64_t)B + b) * M + qi] = l2;
+  }
+
+  const uint32_t row_at = TL::row_at(lane), tr_at = TL::tr_at(lane);
+  f32x16 dq[NB];
+#pragma unroll
+  for (int hb = 0; hb < NB; ++hb)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) dq[hb][v] = 0.0f;
+  const float ninf = -__builtin_huge_valf();
+
+  // one block of 32 keys: S^T, dP^T, dS^T, dQ^T += K^T dS^T (LDS reads hoisted as in the key kernel below)
+  auto block = [&](const uint16_t *kt, const uint16_t *vt, int kb, int c0, auto edge) {
+    constexpr bool EDGE = decltype(edge)::value;
+    f32x16 s, dp;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) s[v] = 0.0f, dp[v] = 0.0f;
+    u32x4 ka[NK], va[NK];
+#pragma unroll
+    for (int ks = 0; ks < NK; ++ks) ka[ks] = TL::rows(kt, row_at, kb, ks), va[ks] = TL::rows(vt, row_at, kb, ks);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int ks = 0; ks < NK; ++ks) {
+      s = Mma<T>::run(ka[ks], qf[ks], s);
+      dp = Mma<T>::run(va[ks], gf[ks], dp);
+    }
+    u32x4 kc[2][NB];
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int hb = 0; hb < NB; ++hb) kc[t][hb] = TL::cols(kt, tr_at, kb, t, hb);
+    __builtin_amdgcn_sched_barrier(0);
+    if (EDGE) {
+      const int d0 = c0 + 4 * half - qi;  // key - query at offset 0; valid offsets: first..last
+      const int first = -w - d0, last = min(w - d0, M - 1 - c0 - 4 * half);
+      const int origin = last < first ? 0x100000 : first;
+      const unsigned span = last < first ? 0u : (unsigned)(last - first);
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int ofs = 8 * (v / 4) + v % 4;
+        s[v] = (unsigned)(ofs - origin) <= span ? s[v] : ninf;
+      }
+    }
+    float ds[16];
+#pragma unroll
+    for (int v = 0; v < 16; ++v) ds[v] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[v], c, -l2)) * (dp[v] - delta);
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      const u32x4 dsf = pack8<T>(ds + 8 * t);
+#pragma unroll
+      for (int hb = 0; hb < NB; ++hb) dq[hb] = Mma<T>::run(kc[t][hb], dsf, dq[hb]);
+    }
+  };
+
+  int stage = 0;
+  auto open_chunk = [&](int kc) {
+    wait_vmcnt<(DEPTH - 1) * LOADS>();
+    __builtin_amdgcn_s_barrier();
+    int st = stage + DEPTH;
+    st = st >= STAGES ? st - STAGES : st;
+    request(kc + DEPTH, st);
+  };
+  auto close_chunk = [&]() { stage = stage + 1 == STAGES ? 0 : stage + 1; };
+  auto edge_chunk = [&](int kc) {
+    open_chunk(kc);
+#pragma unroll
+    for (int kb = 0; kb < 2; ++kb) {
+      const int cb = kc * AB_KC + 32 * kb;
+      if (cb + 31 < qw0 - w || cb > qw0 + 31 + w || cb >= M) continue;  // scalar
+      // one instantiation for every block of an edge chunk, masked whether it needs it or not: two
+      // code paths that update the accumulators make the compiler copy them between register sets
+      block(k_lds[stage], v_lds[stage], kb, cb, std::true_type());
+    }
+    close_chunk();
+  };
+  const int pair_lo = max(kc_lo, (qw0 + 31 - w + 63) >> 6);
+  const int pair_hi = min(kc_hi, (min(qw0 + w, M - 1) - 63) >> 6);
+  const int lead_end = pair_lo <= pair_hi ? pair_lo : kc_hi + 1;
+  int kc = kc_lo;
+  for (; kc < lead_end; ++kc) edge_chunk(kc);
+  for (; kc <= pair_hi; ++kc) {
+    open_chunk(kc);
+    block(k_lds[stage], v_lds[stage], 0, 0, std::false_type());
+    block(k_lds[stage], v_lds[stage], 1, 0, std::false_type());
+    close_chunk();
+  }
+  for (; kc <= kc_hi; ++kc) edge_chunk(kc);
+
+  wait_vmcnt<0>();
+  __builtin_amdgcn_s_barrier();
+  static_assert(4 * RowStage<NB>::ELEMS <= STAGES * TILE, "the four staging areas must fit the key tiles");
+  store_wave_rows<T, NB>(&k_lds[0][0] + wave * RowStage<NB>::ELEMS, dq, scale, dQ + (int64_t)b * dqsb, dqsr, qw0, M, N,
+                         lane);
+}
+
+template <typename T, int NK>
+__global__ __launch_bounds__(kThreads, NK <= 4 ? 2 : 1) void attention_backward_key_dma_kernel(
+    const uint16_t *__restrict__ Q, const uint16_t *__restrict__ K, const uint16_t *__restrict__ V,
+    const uint16_t *__restrict__ dO, const float *__restrict__ D, uint16_t *__restrict__ dK,
+    uint16_t *__restrict__ dV, int B, int M, int w, int nblk, float scale, int64_t qsb, int64_t qsr, int64_t ksb,
+    int64_t ksr, int64_t vsb, int64_t vsr, int64_t gsb, int64_t gsr, int64_t dksb, int64_t dksr, int64_t dvsb,
+    int64_t dvsr) {
+  typedef BwdTile<NK> TL;
+  constexpr int N = TL::N, NB = TL::NB, PPR = TL::PPR, ROWB = TL::ROWB, TILE = TL::TILE;
+  constexpr int STAGES = TL::STAGES, DEPTH = TL::DEPTH;
+  constexpr int LOADS = 2 * (PPR / 4) + 1;  // loads per wavefront and chunk: Q, dO and one row statistic
+  __shared__ __attribute__((aligned(1024))) uint16_t q_lds[STAGES][TILE];
+  __shared__ __attribute__((aligned(1024))) uint16_t g_lds[STAGES][TILE];
+  __shared__ __attribute__((aligned(256))) float stat_lds[STAGES][2][AB_KC];  // [0] D, [1] log-sum-exp (log2 units)
+
+  int b, blk;
+  if (!decode_block(nblk, B, &b, &blk)) return;
+  const int tid = threadIdx.x, lane = tid & 63, half = lane >> 5;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int c0 = blk * AB_TM;
+  const int kw0 = c0 + 32 * wave;  // first key of this wavefront (scalar)
+  const int kj = kw0 + (lane & 31);
+  const bool k_ok = kj < M;
+  const float c = scale * kLog2e;
+
+  const u32x4 q_rsrc = make_rsrc(Q + (int64_t)b * qsb, (uint32_t)((M - 1) * qsr * 2 + ROWB));
+  const u32x4 g_rsrc = make_rsrc(dO + (int64_t)b * gsb, (uint32_t)((M - 1) * gsr * 2 + ROWB));
+  // waves 0 and 2 fetch D, waves 1 and 3 the log-sum-exp (twice the same 256 bytes each: every
+  // wavefront then has the same number of loads in flight, which is what the waits count)
+  const u32x4 s_rsrc = make_rsrc(D + ((int64_t)(wave & 1) * B + b) * M, (uint32_t)(M * 4));
+  const uint32_t q_voff = dma_lane_offset<PPR>(wave, lane, qsr), g_voff = dma_lane_offset<PPR>(wave, lane, gsr);
+  const uint32_t q_step = (uint32_t)(256 / PPR * qsr * 2), g_step = (uint32_t)(256 / PPR * gsr * 2);
+  const uint32_t q_chunk = (uint32_t)(AB_KC * qsr * 2), g_chunk = (uint32_t)(AB_KC * gsr * 2);
+  auto request = [&](int qc, int stage) {
+    dma_chunk<PPR>(q_rsrc, q_lds[stage], wave, q_voff, q_chunk * (uint32_t)qc, q_step);
+    dma_chunk<PPR>(g_rsrc, g_lds[stage], wave, g_voff, g_chunk * (uint32_t)qc, g_step);
+    dma_dword(s_rsrc, lds_address(stat_lds[stage][wave & 1]), 4 * lane, (uint32_t)(qc * AB_KC * 4));
+  };
+  const int qc_lo = max(c0 - w, 0) / AB_KC;
+  const int qc_hi = min(c0 + AB_TM - 1 + w, M - 1) / AB_KC;
+#pragma unroll
+  for (int d = 0; d < DEPTH; ++d) request(qc_lo + d, d);
+
+  u32x4 kf[NK], vf[NK];
+  {
+    const uint16_t *kr = K + (int64_t)b * ksb + (int64_t)kj * ksr + 8 * half;
+    const uint16_t *vr = V + (int64_t)b * vsb + (int64_t)kj * vsr + 8 * half;
+#pragma unroll
+    for (int ks = 0; ks < NK; ++ks) {
+      kf[ks] = load_row_chunk(kr + 16 * ks, K, k_ok);
+      vf[ks] = load_row_chunk(vr + 16 * ks, V, k_ok);
+    }
+  }
+
+  const uint32_t row_at = TL::row_at(lane), tr_at = TL::tr_at(lane);
+  f32x16 dk[NB], dv[NB];
+#pragma unroll
+  for (int hb = 0; hb < NB; ++hb)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) dk[hb][v] = 0.0f, dv[hb][v] = 0.0f;
+  const float ninf = -__builtin_huge_valf();
+
+  // one block of 32 queries: S, dP, then dV^T += dO^T P and dK^T += Q^T dS.  The LDS reads of a
+  // phase are all issued before its first product (left to itself the compiler reuses one register
+  // set for consecutive operands, which puts one LDS latency in front of every MFMA), and those of
+  // the second phase are in flight while the exponentials run.
+  auto block = [&](const uint16_t *qt, const uint16_t *gt, const float *st, int qb, int r0, auto edge) {
+    constexpr bool EDGE = decltype(edge)::value;
+    f32x16 s, dp;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) s[v] = 0.0f, dp[v] = 0.0f;
+    u32x4 qa[NK], ga[NK];
+    f32x4 dl[4], l2[4];
+#pragma unroll
+    for (int ks = 0; ks < NK; ++ks) qa[ks] = TL::rows(qt, row_at, qb, ks), ga[ks] = TL::rows(gt, row_at, qb, ks);
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      dl[g] = *reinterpret_cast<const f32x4 *>(st + 32 * qb + 8 * g + 4 * half);
+      l2[g] = *reinterpret_cast<const f32x4 *>(st + AB_KC + 32 * qb + 8 * g + 4 * half);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int ks = 0; ks < NK; ++ks) {
+      s = Mma<T>::run(qa[ks], kf[ks], s);
+      dp = Mma<T>::run(ga[ks], vf[ks], dp);
+    }
+    u32x4 gc[2][NB], qc[2][NB];
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int hb = 0; hb < NB; ++hb) gc[t][hb] = TL::cols(gt, tr_at, qb, t, hb), qc[t][hb] = TL::cols(qt, tr_at, qb, t, hb);
+    __builtin_amdgcn_sched_barrier(0);
+    // accumulator v of this lane: query r0 + 8 (v / 4) + 4 half + v % 4, key kj
+    if (EDGE) {
+      const int d0 = r0 + 4 * half - kj;  // query - key at offset 0; valid offsets: first..last
+      const int first = -w - d0, last = min(w - d0, M - 1 - r0 - 4 * half);
+      const int origin = last < first ? 0x100000 : first;
+      const unsigned span = last < first ? 0u : (unsigned)(last - first);
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int ofs = 8 * (v / 4) + v % 4;
+        s[v] = (unsigned)(ofs - origin) <= span ? s[v] : ninf;
+      }
+    }
+    float p[16], ds[16];
+#pragma unroll
+    for (int g = 0; g < 4; ++g)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int v = 4 * g + r;
+        p[v] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[v], c, -l2[g][r]));
+        ds[v] = p[v] * (dp[v] - dl[g][r]);
+      }
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      const u32x4 pf = pack8<T>(p + 8 * t), dsf = pack8<T>(ds + 8 * t);
+#pragma unroll
+      for (int hb = 0; hb < NB; ++hb) {
+        dv[hb] = Mma<T>::run(gc[t][hb], pf, dv[hb]);
+        dk[hb] = Mma<T>::run(qc[t][hb], dsf, dk[hb]);
+      }
+    }
+  };
+
+  int stage = 0;
+  auto open_chunk = [&](int qc) {
+    wait_vmcnt<(DEPTH - 1) * LOADS>();
+    __builtin_amdgcn_s_barrier();
+    int st = stage + DEPTH;
+    st = st >= STAGES ? st - STAGES : st;
+    request(qc + DEPTH, st);
+  };
+  auto close_chunk = [&]() { stage = stage + 1 == STAGES ? 0 : stage + 1; };
+  auto edge_chunk = [&](int qc) {
+    open_chunk(qc);
+#pragma unroll
+    for (int qb = 0; qb < 2; ++qb) {
+      const int rb = qc * AB_KC + 32 * qb;
+      if (rb + 31 < kw0 - w || rb > kw0 + 31 + w || rb >= M) continue;  // scalar
+      block(q_lds[stage], g_lds[stage], stat_lds[stage][0], qb, rb, std::true_type());  // see the query kernel
+    }
+    close_chunk();
+  };
+  const int pair_lo = max(qc_lo, (kw0 + 31 - w + 63) >> 6);
+  const int pair_hi = min(qc_hi, (min(kw0 + w, M - 1) - 63) >> 6);
+  const int lead_end = pair_lo <= pair_hi ? pair_lo : qc_hi + 1;
+  int qc = qc_lo;
+  for (; qc < lead_end; ++qc) edge_chunk(qc);
+  for (; qc <= pair_hi; ++qc) {
+    open_chunk(qc);
+    block(q_lds[stage], g_lds[stage], stat_lds[stage][0], 0, 0, std::false_type());
+    block(q_lds[stage], g_lds[stage], stat_lds[stage][0], 1, 0, std::false_type());
+    close_chunk();
+  }
+  for (; qc <= qc_hi; ++qc) edge_chunk(qc);
+
+  wait_vmcnt<0>();
+  __builtin_amdgcn_s_barrier();
+  static_assert(4 * RowStage<NB>::ELEMS <= STAGES * TILE, "the four staging areas must fit the query tiles");
+  uint16_t *stage_rows = &q_lds[0][0] + wave * RowStage<NB>::ELEMS;
+  if (dK != nullptr) store_wave_rows<T, NB>(stage_rows, dk, scale, dK + (int64_t)b * dksb, dksr, kw0, M, N, lane);
+  if (dV != nullptr) store_wave_rows<T, NB>(stage_rows, dv, 1.0f, dV + (int64_t)b * dvsb, dvsr, kw0, M, N, lane);
+}
+
 template <typename T, int NK>
 hipError_t launch_backward(const Problem &p, const View &q, const View &k, const View &v, const View &o,
                            const View &go, const float *lse, float *delta, const View &gq, const View &gk,
@@ -383,6 +763,29 @@ hipError_t launch_backward(const Problem &p, const View &q, const View &k, const
   const dim3 grid((unsigned)(groups * 8 * nblk)), block(kThreads);
   typedef const uint16_t *in_t;
   typedef uint16_t *out_t;
+  if constexpr (NK == 4 || NK == 8) {
+    // the LDS-direct kernels address a batch element with 32-bit byte offsets
+    const int64_t lim = 0x7fffffff;
+    bool fits = !(p.flags & WM_FLAG_NO_LDS_DIRECT) && (p.M + 3 * AB_KC) * 4 < lim;
+    for (const View *t : {&q, &k, &v, &go}) fits = fits && t->sr > 0 && (p.M + 3 * AB_KC) * t->sr * 2 < lim;
+    if (fits) {
+      if (gq.data != nullptr)
+        hipLaunchKernelGGL((attention_backward_query_dma_kernel<T, NK>), grid, block, 0, p.stream, (in_t)q.data,
+                           (in_t)k.data, (in_t)v.data, (in_t)o.data, (in_t)go.data, lse, (out_t)gq.data, delta, (int)p.B,
+                           (int)p.M, (int)p.w, nblk, (float)scale, q.sb, q.sr, k.sb, k.sr, v.sb, v.sr, o.sb, o.sr, go.sb,
+                           go.sr, gq.sb, gq.sr);
+      else
+        hipLaunchKernelGGL((attention_backward_stats_kernel<T, NK>), grid, block, 0, p.stream, (in_t)o.data,
+                           (in_t)go.data, lse, delta, (int)p.B, (int)p.M, nblk, o.sb, o.sr, go.sb, go.sr);
+      hipError_t err = hipGetLastError();
+      if (err != hipSuccess || (gk.data == nullptr && gv.data == nullptr)) return err;
+      hipLaunchKernelGGL((attention_backward_key_dma_kernel<T, NK>), grid, block, 0, p.stream, (in_t)q.data,
+                         (in_t)k.data, (in_t)v.data, (in_t)go.data, (const float *)delta, (out_t)gk.data,
+                         (out_t)gv.data, (int)p.B, (int)p.M, (int)p.w, nblk, (float)scale, q.sb, q.sr, k.sb, k.sr, v.sb,
+                         v.sr, go.sb, go.sr, gk.sb, gk.sr, gv.sb, gv.sr);
+      return hipGetLastError();
+    }
+  }
 #define WM_ABQ(WITH_DQ)                                                                                              \
   hipLaunchKernelGGL((attention_backward_query_kernel<T, NK, WITH_DQ>), grid, block, 0, p.stream, (in_t)q.data,      \
                      (in_t)k.data, (in_t)v.data, (in_t)o.data, (in_t)go.data, lse, (out_t)gq.data, delta, (int)p.B,  \

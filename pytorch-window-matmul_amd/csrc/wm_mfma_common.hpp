@@ -227,6 +227,74 @@ __device__ __forceinline__ void store_wave_rows(uint16_t *stage, const f32x16 (&
   }
 }
 
+// ---------------------------------------------------------------------------------------------
+// Tiles that global memory writes straight into LDS (buffer_load ... lds), no registers in between
+// ---------------------------------------------------------------------------------------------
+// One wave-level load moves 64 pieces of 16 bytes; lane l's piece lands at LDS base + 16 l, so a
+// tile of R rows x PPR pieces is a flat, unpadded row-major array of 16-byte slots and WHICH piece
+// a lane fetches is the only freedom.  Rows of 128 or 256 bytes (PPR 8 or 16) would put a column of
+// the tile into one bank group, so the piece that lives in slot p of row r is piece p ^ swz(r):
+//   rows r..r+7, same piece (ds_read_b128 by 8 consecutive lanes)       -> 8 distinct bank groups
+//   rows 4n..4n+3, same 32-byte block (ds_read_b64_tr_b16, 16 lanes)     -> 4 distinct blocks
+__device__ __forceinline__ int swz(int r) { return ((r & 3) << 1) | ((r >> 2) & 1); }
+
+// s_waitcnt vmcnt(n) alone (gfx9 encoding: vmcnt in bits 3:0 and 15:14, expcnt 6:4, lgkmcnt 11:8).
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {
+  __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (15 << 8));
+}
+
+// Raw buffer descriptor (four scalar registers) over `bytes` bytes at p: loads beyond the end
+// return zeros.
+__device__ __forceinline__ u32x4 make_rsrc(const void *p, uint32_t bytes) {
+  const uint64_t a = reinterpret_cast<uint64_t>(p);
+  const u32x4 r = {(uint32_t)a, (uint32_t)(a >> 32) & 0xffffu, bytes, 0x00020000u};
+  return r;
+}
+
+// One wave-level load of 64 x 16 bytes into LDS at byte address lds_base (+ 16 lane, added by the
+// hardware); lane l fetches buffer offset voff + soff.  Written as assembly on purpose: the
+// compiler would make every later LDS read wait for all such loads in flight (it cannot tell the
+// tiles apart), which is exactly the wait a multi-stage pipeline must not have.  The kernels
+// count these loads themselves (wait_vmcnt) before the barrier that publishes a tile.  M0 is
+// written here and is not on the clobber list (it is a reserved register; the compiler sets it
+// right before each of its own uses, none of which these kernels contain).
+__device__ __forceinline__ void dma_piece(u32x4 rsrc, uint32_t lds_base, uint32_t voff, uint32_t soff) {
+  asm volatile("s_mov_b32 m0, %3\n\ts_nop 0\n\tbuffer_load_dwordx4 %0, %1, %2 offen lds"
+               :
+               : "v"(voff), "s"(rsrc), "s"(soff), "s"(lds_base)
+               : "memory");
+}
+// The same with 4 bytes per lane: 256 consecutive bytes of LDS per wave-level load.
+__device__ __forceinline__ void dma_dword(u32x4 rsrc, uint32_t lds_base, uint32_t voff, uint32_t soff) {
+  asm volatile("s_mov_b32 m0, %3\n\ts_nop 0\n\tbuffer_load_dword %0, %1, %2 offen lds"
+               :
+               : "v"(voff), "s"(rsrc), "s"(soff), "s"(lds_base)
+               : "memory");
+}
+__device__ __forceinline__ uint32_t lds_address(const void *p) {
+  return (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const void *)p;
+}
+
+// Loads the chunk of 64 rows that starts `row_bytes0` bytes into the buffer into a tile at `tile`
+// (LDS, 64 * PPR slots).  `voff` is the lane's byte offset inside a chunk for the first of the
+// wave's loads (row and swizzled piece of slot 64 wave + lane); the wave's further loads are
+// 256 / PPR rows apart, which is `step` bytes in memory and 4096 bytes in LDS.
+template <int PPR>
+__device__ __forceinline__ void dma_chunk(u32x4 rsrc, const uint16_t *tile, int wave, uint32_t voff,
+                                          uint32_t row_bytes0, uint32_t step) {
+  constexpr int LOADS = PPR / 4;  // per wave: 64 PPR pieces / 64 lanes / 4 waves
+  const uint32_t base = lds_address(tile) + 1024 * wave;
+#pragma unroll
+  for (int j = 0; j < LOADS; ++j) dma_piece(rsrc, base + 4096 * j, voff, row_bytes0 + step * j);
+}
+// The lane's offset for the above: slot 64 wave + lane of the tile -> row, logical piece.
+template <int PPR>
+__device__ __forceinline__ uint32_t dma_lane_offset(int wave, int lane, int64_t row_stride_elems) {
+  const int slot = 64 * wave + lane, row = slot / PPR, piece = (slot % PPR) ^ swz(row);
+  return (uint32_t)(row * row_stride_elems * 2 + piece * 16);
+}
+
 // Workgroup -> (batch, block).  Workgroups are dealt round-robin to the 8 XCDs, each with
 // its own L2; all blocks of one batch element are given to one XCD so that neighbouring
 // blocks find the rows they share (the +-w halo) in that L2.

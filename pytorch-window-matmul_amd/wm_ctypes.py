@@ -19,6 +19,7 @@ DTYPES = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2, torch.float64: 
 FORCE_STRIDED = 0x1
 NO_ALIGNED_BAND = 0x2
 NO_NARROW_BAND = 0x4
+NO_LDS_DIRECT = 0x8
 
 
 class Operand(ctypes.Structure):
@@ -172,7 +173,7 @@ def attention_backward(q, k, v, o, lse, go, w, scale=1.0, flags=0, want=(True, T
     """Gradients (gq, gk, gv), all (B,M,N) row-major, from the forward's o and lse; None where not wanted."""
     B, M, N = q.shape
     gq, gk, gv = (torch.empty(B, M, N, dtype=q.dtype, device=q.device) if x else None for x in want)
-    delta = torch.empty(B, M, dtype=torch.float32, device=q.device)
+    delta = torch.empty(2, B, M, dtype=torch.float32, device=q.device)
     _check(lib().wm_window_attention_backward(op(q), op(k), op(v), op(o), ctypes.c_void_p(lse.data_ptr()), op(go),
                                              op(gq), op(gk), op(gv), ctypes.c_void_p(delta.data_ptr()), B, M, N, w,
                                              float(scale), DTYPES[q.dtype], flags, _stream()),
