@@ -12,18 +12,24 @@ are resident in HBM before the timed region starts.  The value reported is whole
 throughput on the band FLOPs (6 band units per step; the torch softmax adds no FLOPs to
 the count but its time is inside the step).  Next to it:
 
-  roofline      the slowest of the six kernels, timed alone with HIP events on the stream
-                it is launched on, priced against the 8 TB/s HBM peak on its algorithmic
-                bytes (each operand touched once);
-  cpu_baseline  the reference's own scalar CPU path (oracle/_ref, where built) or its C
-                restatement, one thread, on a slice of the batch.
+  roofline       the slowest of the six kernels, timed alone with HIP events on the stream
+                 it is launched on (median of the launches), priced against the 8 TB/s HBM
+                 peak on its algorithmic bytes (each operand touched once);
+  cpu_baseline   the C restatement of the reference's scalar CPU path (and, where it is
+                 built, the reference's own compiled CPU path beside it), one thread, on a
+                 slice of the batch;
+  other_configs  per-kernel timings, band softmax and fused attention at the other shapes
+                 the targets are stated on: the narrow window (w = 8), the wide head
+                 (N = 128, w = 512, float16) and the float32 band that covers the sequence.
 
-Usage: python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c2|c4] [--no-cpu]
+Usage: python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c2|c4|c5] [--no-cpu] [--no-others]
        python bench.py --kernels-only [--shape B M N w] [--dtype bf16|fp16|fp32] [--family auto|wide|strided]
 """
 import argparse
+import hashlib
 import json
 import os
+import statistics
 import sys
 import time
 
@@ -33,17 +39,22 @@ for _p in (REPO, PKG):
     if _p not in sys.path:
         sys.path.insert(0, _p)
 
-HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
+HBM_PEAK_GBS = 8000.0      # MI355X published HBM3E bandwidth
+MFMA_PEAK_TFLOPS = 2500.0  # dense bf16 / fp16 matrix peak
+FP32_PEAK_TFLOPS = 157.3   # float32 matrix peak
 
 WORKLOADS = {
-    # name: (B, M, N, w, dtype, qk_scale, backward)
     "c3": dict(B=96, M=4096, N=64, w=256, dtype="bf16", qk_scale=0.125, backward=True,
                label="B96 M4096 N64 w256 bf16, window->softmax->unwindow, fwd+bwd"),
     "c2": dict(B=96, M=16384, N=64, w=8, dtype="bf16", qk_scale=1.0, backward=False,
                label="B96 M16384 N64 w8 bf16, window->softmax->unwindow, fwd"),
     "c4": dict(B=16, M=32768, N=128, w=512, dtype="fp16", qk_scale=1.0, backward=True,
                label="B16 M32768 N128 w512 fp16, window->softmax->unwindow, fwd+bwd"),
+    "c5": dict(B=7, M=3001, N=80, w=1500, dtype="fp32", qk_scale=1.0, backward=True,
+               label="B7 M3001 N80 w1500 fp32, window->softmax->unwindow, fwd+bwd"),
 }
+# source files of the kernels whose HBM traffic profiles/config3_bf16_hbm_traffic.md records
+TRAFFIC_SOURCES = ("wm_mfma.hip", "wm_mfma_common.hpp")
 
 
 def band_unit_flops(B, M, N, w):
@@ -58,23 +69,38 @@ def kernel_bytes(B, M, N, w, es):
     return band + 2 * mat  # P1: X, Y in, band out;  P2 / P3: band, Y in, C out
 
 
+def kernel_source_digest():
+    h = hashlib.sha256()
+    for name in TRAFFIC_SOURCES:
+        with open(os.path.join(PKG, "csrc", name), "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()[:16]
+
+
 def profiled_traffic(kernel_label):
     """HBM bytes per launch of the dominant kernel as measured with rocprofv3 counters (FETCH_SIZE and
-    WRITE_SIZE runs, scaled by a copy of known size); read from the committed summary, None if absent."""
+    WRITE_SIZE runs, scaled by a copy of known size), read from the committed summary.  The summary
+    names the digest of the kernel sources it was measured on: when the sources have changed since,
+    the stored figure says nothing about this run and None is returned."""
     path = os.path.join(REPO, "profiles", "config3_bf16_hbm_traffic.md")
     prim = {"P1": "p1", "P2": "p2", "P3": "p3"}.get(kernel_label[-3:-1])
+    value, digest = None, None
     try:
         for line in open(path):
             parts = line.split()
             if len(parts) == 3 and parts[0] == "traffic_bytes_per_launch" and parts[1] == prim:
-                return int(parts[2])
+                value = int(parts[2])
+            if len(parts) == 2 and parts[0] == "kernel_source_digest":
+                digest = parts[1]
     except OSError:
-        pass
-    return None
+        return None, None
+    if digest != kernel_source_digest():
+        return None, digest
+    return value, digest
 
 
 def time_gpu(fn, iters, warmup):
-    """Mean duration of one launch, each launch bracketed by its own pair of HIP events on the
+    """Median duration of one launch, each launch bracketed by its own pair of HIP events on the
     current stream (so that the gap between dependent launches is not counted as kernel time)."""
     import torch
 
@@ -87,52 +113,163 @@ def time_gpu(fn, iters, warmup):
         fn()
         stop.record()
     torch.cuda.synchronize()
-    return sum(a.elapsed_time(b) for a, b in pairs) / iters  # ms
+    return statistics.median(a.elapsed_time(b) for a, b in pairs)  # ms
+
+
+def time_steps(fn, steps, warmup):
+    import torch
+
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        fn()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) * 1e3 / steps
 
 
 def cpu_baseline(cfg, seconds_budget=20.0):
-    """Times the reference CPU path (or its restatement) on one thread over a batch slice."""
+    """Times the C restatement of the reference's scalar CPU path on one thread over a batch slice, and
+    the reference's own compiled CPU path beside it where that build is present."""
     import torch
 
     import oracle
 
     torch.set_num_threads(1)
-    ref = oracle.reference_module()
-    kind = "reference" if ref is not None else "port"
-    impl = ref if ref is not None else oracle
     M, N, w = cfg["M"], cfg["N"], cfg["w"]
-    g = torch.Generator().manual_seed(0)
     rnd = {"bf16": torch.bfloat16, "fp16": torch.float16, "fp32": torch.float32}[cfg["dtype"]]
 
-    def rounded(*shape, scale=1.0):
-        return (torch.randn(*shape, generator=g) * scale).to(rnd).float()
+    def run(impl, budget):
+        g = torch.Generator().manual_seed(0)
 
-    slice_b, done, elapsed = 1, 0, 0.0
-    flops = 0.0
-    while elapsed < seconds_budget * 0.5 and done < cfg["B"]:
-        q, k, v, go = (rounded(slice_b, M, N, scale=s) for s in (cfg["qk_scale"], cfg["qk_scale"], 1.0, 1.0))
-        kt = k.transpose(1, 2).contiguous()
-        t0 = time.perf_counter()
-        att = impl.window_matmul_forward(q, kt, w)
-        probs = att.softmax(-1)
-        impl.unwindow_matmul_forward(probs, v, w)
-        units = 2
-        if cfg["backward"]:
-            ga, _ = impl.unwindow_matmul_backward(probs, v, w, go)
-            impl.window_matmul_backward(q, kt, w, ga)
-            units = 6
-        elapsed += time.perf_counter() - t0
-        done += slice_b
-        flops += units * band_unit_flops(slice_b, M, N, w)
-    return {
-        "value": flops / elapsed / 1e12,
+        def rounded(*shape, scale=1.0):
+            return (torch.randn(*shape, generator=g) * scale).to(rnd).float()
+
+        done, elapsed, flops = 0, 0.0, 0.0
+        while elapsed < budget and done < cfg["B"]:
+            q, k, v, go = (rounded(1, M, N, scale=s) for s in (cfg["qk_scale"], cfg["qk_scale"], 1.0, 1.0))
+            kt = k.transpose(1, 2).contiguous()
+            t0 = time.perf_counter()
+            att = impl.window_matmul_forward(q, kt, w)
+            probs = att.softmax(-1)
+            impl.unwindow_matmul_forward(probs, v, w)
+            units = 2
+            if cfg["backward"]:
+                ga, _ = impl.unwindow_matmul_backward(probs, v, w, go)
+                impl.window_matmul_backward(q, kt, w, ga)
+                units = 6
+            elapsed += time.perf_counter() - t0
+            done += 1
+            flops += units * band_unit_flops(1, M, N, w)
+        return flops / elapsed / 1e12, done, elapsed
+
+    ref = oracle.reference_module()
+    value, done, elapsed = run(oracle, seconds_budget * (0.35 if ref is not None else 0.5))
+    out = {
+        "value": value,
         "unit": "TFLOP/s",
         "cores": 1,
-        "kind": kind,
+        "kind": "port",
         "sample": f"{done} of {cfg['B']} batch elements at full M, N, w; float32 copies of the rounded inputs; "
                   f"{elapsed:.1f} s of CPU time (softmax between the ops included, as on the GPU)",
         "host_cpus": os.cpu_count(),
     }
+    if ref is not None:
+        rvalue, rdone, relapsed = run(ref, seconds_budget * 0.15)
+        out["reference_cpu_path"] = {"value": rvalue, "unit": "TFLOP/s", "cores": 1,
+                                     "sample": f"{rdone} batch elements, {relapsed:.1f} s; the reference's own "
+                                               "scalar kernels compiled from its sources"}
+    return out
+
+
+class Bench:
+    """Tensors and launches of one configuration."""
+
+    def __init__(self, cfg, family):
+        import torch
+
+        import wm_ctypes as abi
+
+        self.cfg, self.abi, self.torch, self.fam = cfg, abi, torch, family
+        self.B, self.M, self.N, self.w = cfg["B"], cfg["M"], cfg["N"], cfg["w"]
+        self.dtype = {"bf16": torch.bfloat16, "fp16": torch.float16, "fp32": torch.float32}[cfg["dtype"]]
+        self.es = 4 if self.dtype == torch.float32 else 2
+        self.dev = torch.device("cuda:0")
+        self.g = torch.Generator().manual_seed(0)
+        self.q, self.k = self.synth(cfg["qk_scale"]), self.synth(cfg["qk_scale"])
+        self.v, self.go = self.synth(), self.synth()
+        self.unit = band_unit_flops(self.B, self.M, self.N, self.w)
+
+    def synth(self, scale=1.0):
+        return (self.torch.randn(self.B, self.M, self.N, generator=self.g) * scale).to(self.dtype).to(self.dev)
+
+    def kernels(self, iters):
+        """Per-kernel timing through the C ABI (one launch per call), same tensors, same stream."""
+        torch, abi, cfg, w, fam = self.torch, self.abi, self.cfg, self.w, self.fam
+        B, M, N, es = self.B, self.M, self.N, self.es
+        out = {}
+        with torch.no_grad():
+            q, k, v, go = self.q.detach(), self.k.detach(), self.v.detach(), self.go
+            kt = k.transpose(1, 2)
+            att = abi.window_forward(q, kt, w)
+            probs = torch.softmax(att, dim=-1)
+            ga = None
+            launches = {
+                "window_fwd(P1)": lambda: abi.window_forward(q, kt, w, fam, out=att),
+                "unwindow_fwd(P2)": lambda: abi.unwindow_forward(probs, v, w, fam),
+            }
+            if cfg["backward"]:
+                ga = torch.randn(B, M, 2 * w + 1, generator=self.g).to(self.dtype).to(self.dev)
+                launches.update({
+                    "grad_a(P1)": lambda: abi.unwindow_backward(probs, v, w, go, fam, want_v=False),
+                    "grad_v(P3)": lambda: abi.unwindow_backward(probs, v, w, go, fam, want_a=False),
+                    "grad_q(P2)": lambda: abi.window_backward(q, kt, w, ga, fam, want_k=False),
+                    "grad_k(P3)": lambda: abi.window_backward(q, kt, w, ga, fam, want_q=False),
+                })
+            kb = kernel_bytes(B, M, N, w, es)
+            per_kernel = {}
+            for name, fn in launches.items():
+                ms = time_gpu(fn, iters, 3)
+                per_kernel[name] = {"ms": round(ms, 4), "GBps": round(kb / ms / 1e6, 1),
+                                    "hbm_frac": round(kb / ms / 1e6 / HBM_PEAK_GBS, 4),
+                                    "TFLOPs": round(self.unit / ms / 1e9, 1)}
+            out["kernels"], out["algorithmic_bytes_per_launch"] = per_kernel, kb
+            out["softmax_fwd_ms"] = round(time_gpu(lambda: torch.softmax(att, dim=-1), iters, 3), 4)
+            band_bytes = att.numel() * es
+            sm_out = torch.empty_like(att)
+            bs_fwd = time_gpu(lambda: abi.band_softmax_forward(att, 1.0, out=sm_out), iters, 3)
+            bs_bwd = time_gpu(lambda: abi.band_softmax_backward(probs, ga if ga is not None else att, 1.0, out=sm_out),
+                              iters, 3)
+            out["band_softmax"] = {"fwd_ms": round(bs_fwd, 4), "fwd_GBps": round(2 * band_bytes / bs_fwd / 1e6, 1),
+                                   "bwd_ms": round(bs_bwd, 4), "bwd_GBps": round(3 * band_bytes / bs_bwd / 1e6, 1)}
+            if es == 2:  # the fused kernels are 16-bit only; float32 runs the chain of separate ops
+                fo, flse = abi.attention_forward(q, k, v, w, 1.0)
+                fwd = time_gpu(lambda: abi.attention_forward(q, k, v, w, 1.0), iters, 3)
+                fused = {"fwd_ms": round(fwd, 4), "fwd_TFLOPs": round(2 * self.unit / fwd / 1e9, 1),
+                         "fwd_mfma_frac": round(2 * self.unit / fwd / 1e9 / MFMA_PEAK_TFLOPS, 4),
+                         "fwd_hbm_frac": round((4 * B * M * N * es + 4 * B * M) / fwd / 1e6 / HBM_PEAK_GBS, 4)}
+                if cfg["backward"]:
+                    bwd = time_gpu(lambda: abi.attention_backward(q, k, v, fo, flse, go, w, 1.0), iters, 3)
+                    fused.update({"bwd_ms": round(bwd, 4), "bwd_TFLOPs": round(4 * self.unit / bwd / 1e9, 1),
+                                  "bwd_mfma_frac": round(4 * self.unit / bwd / 1e9 / MFMA_PEAK_TFLOPS, 4),
+                                  "step_mfma_frac": round(6 * self.unit / (fwd + bwd) / 1e9 / MFMA_PEAK_TFLOPS, 4)})
+                out["fused_attention"] = fused
+                del fo, flse
+            # device-to-device copy of the band as the achievable-bandwidth yardstick
+            scratch = torch.empty_like(att)
+            copy_ms = time_gpu(lambda: scratch.copy_(att), iters, 3)
+            out["copy_yardstick_GBps"] = round(2 * att.numel() * es / copy_ms / 1e6, 1)
+            out["copy_bytes_each_way"] = att.numel() * es
+        dom = max(per_kernel, key=lambda n: per_kernel[n]["ms"])
+        out["slowest_kernel"] = dom
+        if self.dtype == torch.float32:
+            out["bound"] = "mfma (float32 matrix peak %.1f TFLOP/s)" % FP32_PEAK_TFLOPS
+            out["slowest_kernel_frac"] = round(per_kernel[dom]["TFLOPs"] / FP32_PEAK_TFLOPS, 4)
+        else:
+            out["bound"] = "hbm"
+            out["slowest_kernel_frac"] = per_kernel[dom]["hbm_frac"]
+        return out
 
 
 def main():
@@ -149,6 +286,7 @@ def main():
                     help="kernel family for the per-kernel timings: the library's choice, the wide-band MFMA "
                          "kernels even for a narrow band, or the strided kernels (A/B measurements)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-others", action="store_true", help="skip the per-kernel timings at the other configurations")
     ap.add_argument("--kernels-only", action="store_true",
                     help="launch each of the six kernels --steps times and a reference copy, nothing else "
                          "(for rocprofv3 counter passes)")
@@ -171,16 +309,19 @@ def main():
                    label=f"B{sb} M{sm} N{sn} w{sw} {args.dtype}, window->softmax->unwindow, fwd+bwd")
         args.workload = "custom"
     fam = {"auto": 0, "wide": abi.NO_NARROW_BAND, "strided": abi.FORCE_STRIDED}[args.family]
-    B, M, N, w = cfg["B"], cfg["M"], cfg["N"], cfg["w"]
-    dtype = {"bf16": torch.bfloat16, "fp16": torch.float16, "fp32": torch.float32}[cfg["dtype"]]
-    es = 4 if dtype == torch.float32 else 2
-    dev = torch.device("cuda:0")
-    g = torch.Generator().manual_seed(0)
+    iters = max(args.steps, 10)
+    bench = Bench(cfg, fam)
+    B, M, N, w = bench.B, bench.M, bench.N, bench.w
 
-    def synth(scale=1.0):
-        return (torch.randn(B, M, N, generator=g) * scale).to(dtype).to(dev)
+    if args.kernels_only:
+        k = bench.kernels(iters)
+        print(json.dumps({"workload": cfg["label"], "family": args.family, "kernels": k["kernels"],
+                          "fused_attention": k.get("fused_attention"), "band_softmax": k["band_softmax"],
+                          "copy_yardstick_GBps": k["copy_yardstick_GBps"],
+                          "copy_bytes_each_way": k["copy_bytes_each_way"]}), flush=True)
+        return
 
-    q, k, v, go = synth(cfg["qk_scale"]), synth(cfg["qk_scale"]), synth(), synth()
+    q, k, v, go = bench.q, bench.k, bench.v, bench.go
     if cfg["backward"]:  # forward-only workloads are inference: no autograd graph is recorded
         q.requires_grad_(True), k.requires_grad_(True), v.requires_grad_(True)
 
@@ -193,91 +334,35 @@ def main():
             out.backward(go)
         return out
 
-    units = 6 if cfg["backward"] else 2
-    flops = units * band_unit_flops(B, M, N, w)
-    ms_per_step = float("nan")
-    if not args.kernels_only:
-        for _ in range(args.warmup):
-            step()
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        for _ in range(args.steps):
-            step()
-        torch.cuda.synchronize()
-        ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
-        # the same chain with this library's band softmax in place of torch's (one changed line
-        # in caller code; reported beside the drop-in figure, never as `value`)
-        for _ in range(args.warmup):
-            step(band_softmax)
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        for _ in range(args.steps):
-            step(band_softmax)
-        torch.cuda.synchronize()
-        band_ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
-
-        # and the whole chain as one call: fused kernels, the band never reaches memory
-        def fused_step():
-            out = window_attention(q, k, v, w, scale=1.0)
-            if cfg["backward"]:
-                q.grad = k.grad = v.grad = None
-                out.backward(go)
-            return out
-
-        for _ in range(args.warmup):
-            fused_step()
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        for _ in range(args.steps):
-            fused_step()
-        torch.cuda.synchronize()
-        fused_ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
-
-    # per-kernel timing through the C ABI (one launch per call), same tensors, same stream
-    with torch.no_grad():
-        kt = k.detach().transpose(1, 2)
-        att = abi.window_forward(q.detach(), kt, w)
-        probs = torch.softmax(att, dim=-1)
-        ga = torch.randn(B, M, 2 * w + 1, generator=g).to(dtype).to(dev) if cfg["backward"] else None
-        qd, vd = q.detach(), v.detach()
-        launches = {
-            "window_fwd(P1)": lambda: abi.window_forward(qd, kt, w, fam, out=att),
-            "unwindow_fwd(P2)": lambda: abi.unwindow_forward(probs, vd, w, fam),
-        }
+    def fused_step():  # the whole chain as one call: fused kernels, the band never reaches memory
+        out = window_attention(q, k, v, w, scale=1.0)
         if cfg["backward"]:
-            launches.update({
-                "grad_a(P1)": lambda: abi.unwindow_backward(probs, vd, w, go, fam, want_v=False),
-                "grad_v(P3)": lambda: abi.unwindow_backward(probs, vd, w, go, fam, want_a=False),
-                "grad_q(P2)": lambda: abi.window_backward(qd, kt, w, ga, fam, want_k=False),
-                "grad_k(P3)": lambda: abi.window_backward(qd, kt, w, ga, fam, want_q=False),
-            })
-        kb = kernel_bytes(B, M, N, w, es)
-        per_kernel = {}
-        for name, fn in launches.items():
-            ms = time_gpu(fn, max(args.steps, 10), 3)
-            per_kernel[name] = {"ms": round(ms, 4), "GBps": round(kb / ms / 1e6, 1),
-                                "TFLOPs": round(band_unit_flops(B, M, N, w) / ms / 1e9, 1)}
-        softmax_ms = time_gpu(lambda: torch.softmax(att, dim=-1), max(args.steps, 10), 3)
-        band_bytes = att.numel() * es
-        sm_out = torch.empty_like(att)
-        bs_fwd_ms = time_gpu(lambda: abi.band_softmax_forward(att, 1.0, out=sm_out), max(args.steps, 10), 3)
-        bs_bwd_ms = time_gpu(lambda: abi.band_softmax_backward(probs, ga if ga is not None else att, 1.0, out=sm_out),
-                             max(args.steps, 10), 3)
-        del sm_out
-        fused_fwd_ms = fused_bwd_ms = None
-        if es == 2:  # the fused kernels are 16-bit only; float32 runs the chain of separate ops
-            fo, flse = abi.attention_forward(qd, k.detach(), vd, w, 1.0)
-            fused_fwd_ms = time_gpu(lambda: abi.attention_forward(qd, k.detach(), vd, w, 1.0), max(args.steps, 10), 3)
-            if cfg["backward"]:
-                fused_bwd_ms = time_gpu(lambda: abi.attention_backward(qd, k.detach(), vd, fo, flse, go, w, 1.0),
-                                        max(args.steps, 10), 3)
-            del fo, flse
-        # device-to-device copy of the band as the achievable-bandwidth yardstick
-        scratch = torch.empty_like(att)
-        copy_ms = time_gpu(lambda: scratch.copy_(att), 20, 3)
-        copy_gbs = 2 * att.numel() * es / copy_ms / 1e6
-    dom = max(per_kernel, key=lambda n: per_kernel[n]["ms"])
+            q.grad = k.grad = v.grad = None
+            out.backward(go)
+        return out
+
+    units = 6 if cfg["backward"] else 2
+    flops = units * bench.unit
+    ms_per_step = time_steps(step, args.steps, args.warmup)
+    # the same chain with this library's band softmax in place of torch's (one changed line in
+    # caller code; reported beside the drop-in figure, never as `value`)
+    band_ms_per_step = time_steps(lambda: step(band_softmax), args.steps, args.warmup)
+    fused_ms_per_step = time_steps(fused_step, args.steps, args.warmup)
+
+    kern = bench.kernels(iters)
+    per_kernel, kb = kern["kernels"], kern["algorithmic_bytes_per_launch"]
+    dom = kern["slowest_kernel"]
     achieved = per_kernel[dom]["GBps"]
+    traffic, digest = profiled_traffic(dom) if args.workload == "c3" else (None, None)
+    fused = dict(kern.get("fused_attention") or {})
+    fused.update({"ms_per_step": round(fused_ms_per_step, 4), "TFLOPs": round(flops / fused_ms_per_step / 1e9, 2),
+                  "mfma_frac": round(flops / fused_ms_per_step / 1e9 / MFMA_PEAK_TFLOPS, 4),
+                  "note": "same chain as one call, window_matmul.window_attention (autograd step); band FLOPs "
+                          "credited as for the separate ops (recomputation in the backward not counted); "
+                          "fractions against 2.5 PFLOP/s"})
+    band = dict(kern["band_softmax"])
+    band.update({"ms_per_step": round(band_ms_per_step, 4), "TFLOPs": round(flops / band_ms_per_step / 1e9, 2),
+                 "note": "same chain with window_matmul.band_softmax replacing torch.softmax"})
     result = {
         "metric": "fwd+bwd TFLOP/s & HBM GB/s, window+unwindow, B96 M4096 N64 w256 bf16" if args.workload == "c3"
                   else f"band TFLOP/s, window+unwindow, {cfg['label']}",
@@ -295,35 +380,30 @@ def main():
         "config": {"workload": cfg["label"], "B": B, "M": M, "N": N, "w": w,
                    "band_gflop_per_step": round(flops / 1e9, 2)},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBS, 4),
-                     "traffic": profiled_traffic(dom) if args.workload == "c3" else None, "kernel": dom,
-                     "algorithmic_bytes_per_launch": kb, "avg_launch_ms": per_kernel[dom]["ms"]},
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic,
+                     "traffic_source": "profiles/config3_bf16_hbm_traffic.md, kernel sources %s" % digest
+                                       if traffic is not None else
+                                       "not measured in this run; the committed counter summary is for other kernel sources",
+                     "kernel": dom, "algorithmic_bytes_per_launch": kb, "median_launch_ms": per_kernel[dom]["ms"]},
         "kernels": per_kernel,
-        "softmax_fwd_ms": round(softmax_ms, 4),
-        "band_softmax": None if args.kernels_only else {
-            "ms_per_step": round(band_ms_per_step, 4), "TFLOPs": round(flops / band_ms_per_step / 1e9, 2),
-            "fwd_ms": round(bs_fwd_ms, 4), "fwd_GBps": round(2 * band_bytes / bs_fwd_ms / 1e6, 1),
-            "bwd_ms": round(bs_bwd_ms, 4), "bwd_GBps": round(3 * band_bytes / bs_bwd_ms / 1e6, 1),
-            "note": "same chain with window_matmul.band_softmax replacing torch.softmax"},
-        "fused_attention": None if args.kernels_only else {
-            "ms_per_step": round(fused_ms_per_step, 4), "TFLOPs": round(flops / fused_ms_per_step / 1e9, 2),
-            "fwd_ms": None if fused_fwd_ms is None else round(fused_fwd_ms, 4),
-            "bwd_ms": None if fused_bwd_ms is None else round(fused_bwd_ms, 4),
-            "mfma_frac": round(flops / fused_ms_per_step / 1e9 / 2500.0, 4),
-            "note": "same chain as one call, window_matmul.window_attention; band FLOPs credited as for the "
-                    "separate ops (recomputation in the backward not counted); mfma_frac against 2.5 PFLOP/s"},
-        "copy_yardstick_GBps": round(copy_gbs, 1),
-        "kernel_sum_GBps": round(len(per_kernel) * kb / sum(v["ms"] for v in per_kernel.values()) / 1e6, 1),
+        "softmax_fwd_ms": kern["softmax_fwd_ms"],
+        "band_softmax": band,
+        "fused_attention": fused,
+        "copy_yardstick_GBps": kern["copy_yardstick_GBps"],
+        "kernel_sum_GBps": round(len(per_kernel) * kb / sum(x["ms"] for x in per_kernel.values()) / 1e6, 1),
     }
-    if args.kernels_only:
-        print(json.dumps({"workload": cfg["label"], "family": args.family, "kernels": per_kernel,
-                          "copy_yardstick_GBps": round(copy_gbs, 1),
-                          "copy_bytes_each_way": att.numel() * es}), flush=True)
-        return
-    if not args.no_cpu:
-        result["cpu_baseline"] = cpu_baseline(cfg)
-    else:
-        result["cpu_baseline"] = None
+    del bench, q, k, v, go
+    torch.cuda.empty_cache()
+    if not args.no_others and args.workload == "c3":
+        others = {}
+        for name in ("c2", "c4", "c5"):
+            ocfg = WORKLOADS[name]
+            ob = Bench(ocfg, 0)
+            others[name] = {"workload": ocfg["label"], **ob.kernels(10)}
+            del ob
+            torch.cuda.empty_cache()
+        result["other_configs"] = others
+    result["cpu_baseline"] = None if args.no_cpu else cpu_baseline(cfg)
     print(json.dumps(result), flush=True)
 
 
