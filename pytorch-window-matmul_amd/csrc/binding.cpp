@@ -37,18 +37,28 @@ int abi_dtype(const torch::Tensor &t, const char *op) {
   return -1;
 }
 
+bool aligned16(const torch::Tensor &t) { return reinterpret_cast<uintptr_t>(t.data_ptr()) % 16 == 0; }
+
 // Unit column stride and 16-byte aligned rows/batches, else a contiguous copy.
 torch::Tensor vector_friendly(const torch::Tensor &t) {
   const int64_t es = t.element_size();
-  const bool ok = t.stride(2) == 1 && (t.stride(1) * es) % 16 == 0 && (t.stride(0) * es) % 16 == 0 &&
-                  reinterpret_cast<uintptr_t>(t.data_ptr()) % 16 == 0;
+  const bool ok = t.stride(2) == 1 && (t.stride(1) * es) % 16 == 0 && (t.stride(0) * es) % 16 == 0 && aligned16(t);
   if (ok || t.numel() == 0) return t;
-  if (t.is_contiguous()) return t;  // odd N: the strided kernels take it as it is
-  return t.contiguous();
+  if (t.is_contiguous()) {
+    // rows that cannot be aligned (N * element size not a multiple of 16): the strided kernels take
+    // the tensor as it is; alignable rows behind a misaligned pointer (a view at a storage offset)
+    // move into a fresh allocation so that the tuned kernels apply
+    return (t.size(2) * es) % 16 == 0 ? t.clone(at::MemoryFormat::Contiguous) : t;
+  }
+  auto c = t.contiguous();
+  return aligned16(c) || (t.size(2) * es) % 16 != 0 ? c : c.clone(at::MemoryFormat::Contiguous);
 }
 
-// Band tensors (rows of odd length 2w+1) only need to be contiguous.
-torch::Tensor band_friendly(const torch::Tensor &t) { return t.contiguous(); }
+// Band tensors (rows of odd length 2w+1) need to be contiguous and start on a 16-byte boundary.
+torch::Tensor band_friendly(const torch::Tensor &t) {
+  auto c = t.contiguous();
+  return aligned16(c) || c.numel() == 0 ? c : c.clone(at::MemoryFormat::Contiguous);
+}
 
 // K comes as (B,N,M).  The kernels want key rows contiguous, which is what a
 // transposed view of a row-major (B,M,N) tensor already is; anything else is

@@ -55,10 +55,15 @@ typedef hipError_t (*strided_fn)(const Problem &, const View &, const View &, co
 // Kernel choice per primitive: vector-ALU kernels (the narrowest windows), else narrow-band MFMA
 // family, else wide-band MFMA family (all 16-bit storage except the float32 vector kernels), else
 // the float32 MFMA family, else strided.
+// The tiled families launch one workgroup per (batch element, block of at least 16 rows), with the
+// batch count rounded up to a multiple of 8; a grid beyond 2^31 - 1 workgroups does not exist, so
+// such extents run on the strided kernels, whose grid strides over the work.
+bool tiled_grid_fits(int64_t B, int64_t M) { return ((B + 7) / 8) * 8 * ((M + 15) / 16) <= 0x7fffffff; }
+
 int run_primitive(mfma_fn narrow, mfma_fn vector, mfma_fn fast, mfma_fn f32, strided_fn slow, const Problem &p,
                   const View &a, const View &y, const View &c) {
   hipError_t err = hipSuccess;
-  if (!(p.flags & WM_FLAG_FORCE_STRIDED)) {
+  if (!(p.flags & WM_FLAG_FORCE_STRIDED) && tiled_grid_fits(p.B, p.M)) {
     if (vector && !(p.flags & WM_FLAG_NO_NARROW_BAND) && vector(p, a, y, c, &err)) return to_status(err);
     if (narrow && !(p.flags & WM_FLAG_NO_NARROW_BAND) && narrow(p, a, y, c, &err)) return to_status(err);
     if (fast(p, a, y, c, &err)) return to_status(err);
@@ -229,7 +234,7 @@ const char *wm_band_softmax_kernel_choice(int64_t w, int dtype, int contiguous, 
 const char *wm_kernel_choice(int op, int64_t B, int64_t M, int64_t N, int64_t w, int dtype, int fast,
                              unsigned flags) {
   if (op < 1 || op > 3) return "invalid";
-  if (!(flags & WM_FLAG_FORCE_STRIDED) && fast) {
+  if (!(flags & WM_FLAG_FORCE_STRIDED) && fast && tiled_grid_fits(B, M)) {
     if (!(flags & WM_FLAG_NO_NARROW_BAND) && vector_supports(op, M, N, w, dtype)) {
       static const char *names[] = {"vector_p1", "vector_p2", "vector_p3"};
       return names[op - 1];

@@ -226,3 +226,31 @@ def test_ops_follow_the_current_stream(device):
     s1.synchronize()
     s2.synchronize()
     assert torch.equal(got, want) and torch.equal(got2, want2)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32], ids=["bf16", "f32"])
+def test_views_at_a_misaligned_storage_offset(device, dtype):
+    """Contiguous tensors whose data pointer is not 16-byte aligned (views that start one element
+    into a buffer): the ops, the band softmax and the fused attention give the numbers of aligned
+    copies, and the fused call does not refuse them."""
+    from window_matmul import band_softmax, unwindow_matmul, window_attention, window_matmul
+
+    B, M, N, w = 2, 200, 64, 6
+
+    def shifted(t):
+        flat = torch.empty(t.numel() + 1, dtype=t.dtype, device=t.device)
+        view = flat[1:].view(t.shape)
+        view.copy_(t)
+        assert view.is_contiguous() and view.data_ptr() % 16 != 0
+        return view
+
+    q, k, v = (seeded((B, M, N), s, dtype).to(device) for s in (61, 62, 63))
+    att = window_matmul(q, k.transpose(1, 2), w)
+    assert torch.equal(window_matmul(shifted(q), shifted(k).transpose(1, 2), w), att)
+    probs = band_softmax(att, 0.125)
+    assert torch.equal(band_softmax(shifted(att), 0.125), probs)
+    out = unwindow_matmul(probs, v, w)
+    assert torch.equal(unwindow_matmul(shifted(probs), shifted(v), w), out)
+    if dtype != torch.float32:
+        fused = window_attention(q, k, v, w, 0.125)
+        assert torch.equal(window_attention(shifted(q), shifted(k), shifted(v), w, 0.125), fused)
