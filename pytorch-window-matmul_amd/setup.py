@@ -25,7 +25,14 @@ class BuildNative(build_ext):
     def run(self):
         import build as native_build  # build.py next to this file
 
-        native_build.build_all(force=False)
+        # WM_PREBUILT=1 packages the shared objects that are already in the tree (a machine without
+        # hipcc, or a test that must not compile); otherwise stale or missing ones are rebuilt
+        if os.environ.get("WM_PREBUILT") == "1":
+            for name in ("window_matmul_kernel.so", "libwindow_matmul_hip.so"):
+                if not os.path.exists(os.path.join(HERE, name)):
+                    raise RuntimeError(f"WM_PREBUILT=1 but {name} is not built; run python build.py")
+        else:
+            native_build.build_all(force=False)
         for name in ("window_matmul_kernel.so", "libwindow_matmul_hip.so"):
             target = os.path.join(self.build_lib, name)
             os.makedirs(os.path.dirname(target) or ".", exist_ok=True)

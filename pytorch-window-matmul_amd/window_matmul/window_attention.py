@@ -19,11 +19,14 @@ from .band_softmax import band_softmax
 from .window_matmul import unwindow_matmul, window_matmul
 
 
-def _chain_is_faster(window_size: int) -> bool:
+def _chain_is_faster(window_size: int, width: int) -> bool:
     """Windows at which a training step is faster through the separate ops than through the fused
-    kernels (measured at B96 M16384 N64 bf16: 0.48-0.66 ms against 0.67-0.75 ms up to w = 14, equal
-    at w = 15, 0.71-1.08 ms against 0.67-0.69 ms from w = 16 to 32)."""
-    return window_size <= 14
+    kernels, whose recomputing backward costs the same at every narrow window.  Measured on bf16
+    tensors of 100 M elements with M = 16384 (chain / fused, ms per step): N = 32: 0.32 / 0.32 at
+    w = 4, 0.35 / 0.32 at w = 8; N = 64: 0.58 / 0.64 at w = 12, 0.66 / 0.64 at w = 14; N = 96:
+    0.97 / 1.07 at w = 32, 1.20 / 1.19 at w = 40; N = 128: 0.85 / 0.89 at w = 32, 1.04 / 0.98 at
+    w = 40."""
+    return window_size <= (4 if width <= 32 else 13 if width <= 64 else 36)
 
 
 class WindowAttentionFunc(torch.autograd.Function):
@@ -68,7 +71,7 @@ def window_attention(query: torch.Tensor, key: torch.Tensor, value: torch.Tensor
     # With a very narrow band the recomputing backward of the fused kernels costs more than the
     # band it avoids writing, so training there goes through the separate ops.
     training = torch.is_grad_enabled() and any(t.requires_grad for t in (q, k, v))
-    if _native.window_attention_supported(q, window_size, scale) and not (training and _chain_is_faster(window_size)):
+    if _native.window_attention_supported(q, window_size, scale) and not (training and _chain_is_faster(window_size, q.shape[-1])):
         out = WindowAttentionFunc.apply(q, k, v, window_size, scale, bool(mask_out_of_range))
     else:
         att = window_matmul(q, k.transpose(-1, -2), window_size)

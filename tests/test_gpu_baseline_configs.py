@@ -68,7 +68,8 @@ def check(got, want, tol, what):
     torch.testing.assert_close(got.double(), want, rtol=tol, atol=tol, msg=lambda s: f"{what}: {s}")
 
 
-def run_config(device, B, M, N, w, dtype, tol, qk_scale=1.0, backward=True, zero_rows=False, blocks=3, rows=192):
+def run_config(device, B, M, N, w, dtype, tol, qk_scale=1.0, backward=True, zero_rows=False, blocks=3, rows=192,
+               uniform_band=False):
     from window_matmul import unwindow_matmul, window_matmul
 
     q = seeded((B, M, N), 11, dtype, qk_scale).to(device)
@@ -82,9 +83,19 @@ def run_config(device, B, M, N, w, dtype, tol, qk_scale=1.0, backward=True, zero
         q[:, zr] = 0
     q.requires_grad_(backward), k.requires_grad_(backward), v.requires_grad_(backward)
     att = window_matmul(q, k.transpose(1, 2), w)
-    probs = torch.softmax(att.float(), -1).to(dtype).detach().requires_grad_(backward)
-    out = unwindow_matmul(probs, v, w)
     mask = oracle.band_mask(M, w, device)
+    if uniform_band:
+        # the band the configuration names for unwindow_matmul: uniform[0, 1) per entry, rows normalised
+        # to sum 1 (over all 2w+1 entries; those outside the sequence are never read)
+        g = torch.Generator().manual_seed(16)
+        probs = torch.empty(B, M, 2 * w + 1, dtype=dtype, device=device)
+        for b in range(B):  # batch element by batch element: the float32 draw of the whole band would be 2 GiB
+            u = torch.rand(M, 2 * w + 1, generator=g).to(device)
+            probs[b] = (u / u.sum(-1, keepdim=True)).to(dtype)
+        probs.requires_grad_(backward)
+    else:
+        probs = torch.softmax(att.float(), -1).to(dtype).detach().requires_grad_(backward)
+    out = unwindow_matmul(probs, v, w)
 
     # exact zeros outside the sequence; zero q rows give exact zero band rows
     assert not att.detach()[:, ~mask].view(torch.int16 if att.element_size() == 2 else torch.int32).any()
@@ -137,7 +148,7 @@ def test_config3_local_attention_bf16(device):
 
 
 def test_config4_wide_head_fp16(device):
-    run_config(device, B=16, M=32768, N=128, w=512, dtype=torch.float16, tol=2e-2, blocks=2)
+    run_config(device, B=16, M=32768, N=128, w=512, dtype=torch.float16, tol=2e-2, blocks=2, uniform_band=True)
 
 
 @pytest.mark.parametrize("w", [1, 33, 1500])
