@@ -5,14 +5,16 @@ breadth: shapes, dtypes and windows drawn from a fixed seed, the library's own k
 (narrow-band, wide-band MFMA, float32 MFMA) against the strided family, which shares no tiling,
 staging or masking code with them and is itself checked against the oracle in
 ``test_gpu_parity.py``; and the fused attention kernels against the chain of the separate ops in
-float32.  Tolerances as everywhere: float32 1e-3, 16-bit 2e-2 (here relative to the largest
-reference magnitude, since both sides round).
+float32.  Tolerances as everywhere, per element: float32 rtol = atol = 1e-3, 16-bit rtol = atol = 2e-2;
+band entries outside the sequence must be +0.0 on bits.  The float32 kernel families are also
+compared with the CPU oracle directly, one shape each.
 """
 import random
 
 import pytest
 import torch
 
+import oracle
 import wm_ctypes as abi
 
 pytestmark = pytest.mark.gpu
@@ -35,9 +37,24 @@ def _randn(shape, g, dtype, dev, scale=1.0):
 def _assert_close(got, want, tol, what):
     got, want = got.float(), want.float()
     assert torch.isfinite(got).all(), what
+    torch.testing.assert_close(got, want, rtol=tol, atol=tol, msg=lambda m: f"{what}: {m}")
+
+
+def _assert_close_in_scale(got, want, tol, what):
+    """For the fused attention against a float32 chain: the fused backward starts from the output as
+    stored (rounded to 16 bits), whose rounding enters every gradient through D = sum dO * O, so an
+    element near zero can be off by tol times the scale of the tensor rather than of itself."""
+    got, want = got.float(), want.float()
+    assert torch.isfinite(got).all(), what
     if got.numel():
-        err = (got - want).abs().max().item()
-        assert err <= tol * max(1.0, want.abs().max().item()), f"{what}: max error {err}"
+        scale = max(1.0, want.abs().max().item())
+        torch.testing.assert_close(got, want, rtol=tol, atol=tol * scale, msg=lambda m: f"{what}: {m}")
+
+
+def _assert_band_zeros(band, M, w, what):
+    outside = band[:, ~oracle.band_mask(M, w, band.device)]
+    ints = {2: torch.int16, 4: torch.int32}[outside.element_size()]
+    assert not outside.view(ints).any(), f"{what}: a band entry outside the sequence is not +0.0"
 
 
 MATMUL_CASES = _draw(1, 60, [8, 16, 24, 32, 48, 64, 80, 96, 112, 128],
@@ -84,6 +101,37 @@ def test_every_narrow_window(device, dtype, B, M, N, w):
         results.append(dict(window_fwd=att, unwindow_fwd=out, grad_a=ga, grad_v=gv, grad_q=gq, grad_k=gk))
     for name in results[0]:
         _assert_close(results[0][name], results[1][name], 1e-3 if dtype == torch.float32 else 2e-2, name)
+    for name in ("window_fwd", "grad_a"):
+        _assert_band_zeros(results[0][name], M, w, name)
+
+
+# one shape per float32 kernel family, against the CPU oracle itself (kernel_choice names the family)
+F32_FAMILIES = [("vector_p2", 3, 300, 80, 4), ("narrow_p2", 2, 333, 64, 16), ("f32_mfma_p2", 2, 400, 80, 64),
+                ("narrow_p1", 3, 257, 48, 24), ("f32_mfma_p1", 1, 515, 128, 100), ("vector_p3", 2, 129, 24, 9)]
+
+
+@pytest.mark.parametrize("family,B,M,N,w", F32_FAMILIES, ids=[f[0] for f in F32_FAMILIES])
+def test_float32_families_match_the_oracle(device, family, B, M, N, w):
+    op = int(family[-1])
+    assert abi.lib().wm_kernel_choice(op, B, M, N, w, abi.DTYPES[torch.float32], 1, 0).decode() == family
+    g = torch.Generator().manual_seed(N * 1000 + w)
+    q, k, v, go = (torch.randn(B, M, N, generator=g) for _ in range(4))
+    a = torch.randn(B, M, 2 * w + 1, generator=g) * 0.2
+    dq, dk, dv, dgo, da = (t.to(device) for t in (q, k, v, go, a))
+    kt = k.transpose(1, 2).contiguous()
+    tol = dict(rtol=1e-3, atol=1e-3)
+    att = abi.window_forward(dq, dk.transpose(1, 2), w)
+    torch.testing.assert_close(att.cpu(), oracle.window_matmul_forward(q, kt, w), **tol)
+    _assert_band_zeros(att, M, w, "window_fwd")
+    torch.testing.assert_close(abi.unwindow_forward(da, dv, w).cpu(), oracle.unwindow_matmul_forward(a, v, w), **tol)
+    ga, gv = abi.unwindow_backward(da, dv, w, dgo)
+    wa, wv = oracle.unwindow_matmul_backward(a, v, w, go)
+    torch.testing.assert_close(ga.cpu(), wa, **tol)
+    torch.testing.assert_close(gv.cpu(), wv, **tol)
+    gq, gk = abi.window_backward(dq, dk.transpose(1, 2), w, da)
+    wq, wk = oracle.window_matmul_backward(q, kt, w, a)
+    torch.testing.assert_close(gq.cpu(), wq, **tol)
+    torch.testing.assert_close(gk.cpu(), wk, **tol)
 
 
 ATTENTION_CASES = _draw(2, 40, [16, 32, 48, 64, 80, 96, 112, 128], [torch.bfloat16, torch.float16])
@@ -102,9 +150,9 @@ def test_fused_attention_agrees_with_chain_of_ops(device, dtype, B, M, N, w):
     # the same chain on float32 copies of the rounded inputs
     qf, kf, vf, gof = (t.float() for t in (q, k, v, go))
     p = abi.band_softmax_forward(abi.window_forward(qf, kf.transpose(1, 2), w), scale, mask)
-    _assert_close(o, abi.unwindow_forward(p, vf, w), 2e-2, "output")
+    _assert_close_in_scale(o, abi.unwindow_forward(p, vf, w), 2e-2, "output")
     gp, gv_ref = abi.unwindow_backward(p, vf, w, gof)
     gq_ref, gk_ref = abi.window_backward(qf, kf.transpose(1, 2), w, abi.band_softmax_backward(p, gp, scale, mask))
-    _assert_close(gq, gq_ref, 2e-2, "grad_q")
-    _assert_close(gk, gk_ref.transpose(1, 2), 2e-2, "grad_k")
-    _assert_close(gv, gv_ref, 2e-2, "grad_v")
+    _assert_close_in_scale(gq, gq_ref, 2e-2, "grad_q")
+    _assert_close_in_scale(gk, gk_ref.transpose(1, 2), 2e-2, "grad_k")
+    _assert_close_in_scale(gv, gv_ref, 2e-2, "grad_v")
