@@ -439,7 +439,7 @@ __global__ __launch_bounds__(kThreads) void attention_backward_stats_kernel(
 }
 
 template <typename T, int NK>
-__global__ __launch_bounds__(kThreads, NK <= 4 ? 3 : 1) void attention_backward_query_dma_kernel(
+__global__ __launch_bounds__(kThreads, NK <= 4 ? 3 : 2) void attention_backward_query_dma_kernel(
     const uint16_t *__restrict__ Q, const uint16_t *__restrict__ K, const uint16_t *__restrict__ V,
     const uint16_t *__restrict__ O, const uint16_t *__restrict__ dO, const float *__restrict__ L,
     uint16_t *__restrict__ dQ, float *__restrict__ D, int B, int M, int w, int nblk, float scale, int64_t qsb,
