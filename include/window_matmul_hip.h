@@ -60,7 +60,7 @@ typedef enum wm_status {
 #define WM_FLAG_FORCE_STRIDED 0x1u   /* always use the strided fallback kernels (A/B testing) */
 #define WM_FLAG_NO_ALIGNED_BAND 0x2u /* MFMA kernels: never use the 16-byte aligned band variant */
 #define WM_FLAG_NO_NARROW_BAND 0x4u  /* never use the narrow-band kernels (MFMA, w <= 63; vector ALU, w <= 14) */
-#define WM_FLAG_NO_LDS_DIRECT 0x8u   /* fused attention: never use the kernels that load chunks straight into LDS */
+#define WM_FLAG_NO_LDS_DIRECT 0x8u   /* never use the kernels that load chunks straight into LDS (fused attention; band-out product at N = 128) */
 
 /* Rank-3 operand: element (b, r, c) lives at data + b*stride_b + r*stride_r + c*stride_c. */
 typedef struct wm_operand {

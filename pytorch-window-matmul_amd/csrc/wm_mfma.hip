@@ -540,6 +540,218 @@ __global__ __launch_bounds__(kThreads, 2) void mfma_p1_kernel(const uint16_t *__
 }
 
 // ------------------------------------------------------------------------------------------
+// P1 at N = 128 with the Y chunks loaded straight into LDS
+// ------------------------------------------------------------------------------------------
+// The kernel above with one change: a Y chunk does not pass through registers on its way to LDS.
+// Buffer loads with the lds modifier write it into an unpadded, swizzled tile (wm_mfma_common.hpp),
+// one chunk ahead; rows past the end of the sequence read as zeros, rows before its start are
+// replaced by row 0 (the columns they would produce are forced to +0.0 anyway).  Without the two
+// register sets of the staged prefetch and the padding of the tile, three workgroups fit a CU
+// where the kernel above places two, which is what lets the multiplications of one workgroup run
+// under the band stores of another.  The kernel counts its own loads: a wavefront waits until its
+// part of the next chunk has landed while leaving the stores it has just issued in flight.
+template <typename T, int NK, bool ALIGNED>  // NK = N / 16
+__global__ __launch_bounds__(kThreads, 3) void mfma_p1_dma_kernel(const uint16_t *__restrict__ X,
+                                                              const uint16_t *__restrict__ Y,
+                                                              uint16_t *__restrict__ C, int B, int M, int w,
+                                                              int nblk, int galign, int64_t xsb, int64_t xsr,
+                                                              int64_t ysb, int64_t ysr, int64_t csb) {
+  constexpr int N = 16 * NK, PPR = 2 * NK, ROWB = 2 * N;  // 16-byte pieces and bytes per tile row
+  constexpr int SS = KC + 8;  // per-wave staging rows
+  constexpr int LOADS = PPR / 4;  // loads per wavefront and chunk
+  static_assert(NK == 4 || NK == 8, "tile rows of 128 or 256 bytes");
+  __shared__ __attribute__((aligned(1024))) uint16_t y_lds[2][KC * N];
+  __shared__ __attribute__((aligned(16))) uint16_t s_lds[4][32 * SS];
+  // Seam buffer.  The 16-byte chunk that holds the first band entries of row i also holds the
+  // last entries of row i-1 (band rows have odd length).  The head piece is parked here when
+  // its tile is produced; when the tail piece of the row above turns up, many column chunks
+  // later, the two are merged and leave as one aligned 16-byte store.
+  __shared__ __attribute__((aligned(16))) uint16_t seam[TM * 8];
+
+  int b, blk;
+  if (!decode_block(nblk, B, &b, &blk)) return;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wave_s = __builtin_amdgcn_readfirstlane(wave);
+  const int W = 2 * w + 1;
+  const int i0 = blk * TM;
+  const int rows = min(TM, M - i0);
+  const int c_lo = i0 - w, c_hi = i0 + rows - 1 + w;  // not clipped: out-of-sequence entries are written as zeros
+  const int c_start = ALIGNED ? c_lo - (int)(((int64_t)c_lo + (int64_t)b * csb + w) & (galign - 1)) : c_lo;
+  const int nk = (c_hi - c_start + KC) / KC;
+  const uint16_t *Yb = Y + (int64_t)b * ysb;
+  uint16_t *Cb = C + (int64_t)b * csb;
+  // Head and tail pieces of neighbouring rows meet through the seam buffer when both rows belong
+  // to this wave, or to any wave of the workgroup if a workgroup barrier is certain to separate
+  // the two tiles (the tail is produced 2w-1 columns after the head: at least two chunks later).
+  const bool seam_across_waves = ALIGNED && (2 * w - 1 >= 2 * KC);
+
+  // B-operand: this wave's 32 rows of X, all of N, kept in registers
+  u32x4 xop[NK];
+  {
+    const int i = i0 + wave * 32 + (lane & 31);
+    const uint16_t *xr = X + (int64_t)b * xsb + (int64_t)i * xsr + 8 * (lane >> 5);
+#pragma unroll
+    for (int ks = 0; ks < NK; ++ks) xop[ks] = load_row_chunk(xr + 16 * ks, X, i < M);
+  }
+
+  // Y chunk k into tile k & 1: the chunk position is a scalar offset of the loads; only a chunk that
+  // starts before the sequence needs per-lane addresses (row 0 stands in for the rows before it)
+  const u32x4 y_rsrc = make_rsrc(Yb, (uint32_t)((int64_t)(M - 1) * ysr * 2 + ROWB));
+  const uint32_t y_voff = dma_lane_offset<PPR>(wave_s, lane, ysr);
+  const uint32_t y_step = (uint32_t)(256 / PPR * ysr * 2), y_row_bytes = (uint32_t)(ysr * 2);
+  auto request = [&](int k) {
+    const int cb = c_start + k * KC;
+    if (cb >= 0) {
+      dma_chunk<PPR>(y_rsrc, y_lds[k & 1], wave_s, y_voff, (uint32_t)cb * y_row_bytes, y_step);
+    } else {
+      const uint32_t base = lds_address(y_lds[k & 1]) + 1024 * wave_s;
+#pragma unroll
+      for (int j = 0; j < LOADS; ++j) {
+        const int slot = 64 * (wave_s + 4 * j) + lane, row = slot / PPR, piece = (slot % PPR) ^ swz(row);
+        dma_piece(y_rsrc, base + 4096 * j, (uint32_t)max(cb + row, 0) * y_row_bytes + 16 * piece, 0);
+      }
+    }
+  };
+
+  uint16_t *stage = s_lds[wave];
+  // Store slots: lane -> row r = lane / 8 + 8 s of the wave's 32 rows, column group g = lane % 8.
+  const int iw_first = i0 + wave * 32;
+  int st_lo[4], st_hi[4];   // chunk-relative valid element range is [st_lo - cb, st_hi - cb]
+  uint16_t *st_dst[4];      // address of dense column 8 g of the row (add cb)
+  const uint16_t *st_src[4];
+#pragma unroll
+  for (int s = 0; s < 4; ++s) {
+    const int r = (lane >> 3) + 8 * s, g = lane & 7;
+    const int i = iw_first + r;
+    st_lo[s] = i - w - 8 * g;
+    st_hi[s] = i < M ? i + w - 8 * g : -0x40000000;
+    st_dst[s] = Cb + (int64_t)i * W + (w - i) + 8 * g;
+    st_src[s] = stage + r * SS + 8 * g;
+  }
+  uint16_t *stage_wr = stage + (lane & 31) * SS + 4 * (lane >> 5);
+  const uint32_t y_at = (uint32_t)((lane & 31) * ROWB + (((lane >> 5) ^ swz(lane & 31)) << 4));  // byte offset, piece of ks = 0
+
+  // One slot: multiply chunk k, stage the 32 x 64 result and store it.  Returns whether the slot
+  // issued exactly the four whole-line stores per lane of a chunk inside the band.
+  auto slot = [&](int k) {
+    const int buf = k & 1;
+    const int cb = c_start + k * KC;
+    bool four_stores = false;
+    // multiply and stage; the version for chunks with columns outside the sequence forces those
+    // columns to +0.0 (by definition, whatever X holds) and is kept out of the common path
+    auto multiply_and_stage = [&](auto edge) {
+#pragma unroll
+      for (int mt = 0; mt < KC / 32; ++mt) {
+        f32x16 acc;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[v] = 0.f;
+        const char *yl = reinterpret_cast<const char *>(y_lds[buf]) + 32 * mt * ROWB;
+#pragma unroll
+        for (int ks = 0; ks < NK; ++ks)
+          acc = Mma<T>::run(*reinterpret_cast<const u32x4 *>(yl + (y_at ^ (32 * ks))), xop[ks], acc);
+        // acc[v]: dense column = 32 mt + 8 (v / 4) + 4 (lane / 32) + v % 4, row = lane % 32
+#pragma unroll
+        for (int q4 = 0; q4 < 4; ++q4) {
+          uint32_t lo = Mma<T>::pack2(acc[4 * q4], acc[4 * q4 + 1]);
+          uint32_t hi = Mma<T>::pack2(acc[4 * q4 + 2], acc[4 * q4 + 3]);
+          if (decltype(edge)::value) {
+            const int c = cb + 32 * mt + 8 * q4 + 4 * (lane >> 5);
+            if (c < 0 || c >= M) lo &= 0xffff0000u;
+            if (c + 1 < 0 || c + 1 >= M) lo &= 0x0000ffffu;
+            if (c + 2 < 0 || c + 2 >= M) hi &= 0xffff0000u;
+            if (c + 3 < 0 || c + 3 >= M) hi &= 0x0000ffffu;
+          }
+          u32x2 o = {lo, hi};
+          *reinterpret_cast<u32x2 *>(stage_wr + 32 * mt + 8 * q4) = o;
+        }
+      }
+    };
+    if (cb < 0 || cb + KC > M)
+      multiply_and_stage(std::true_type{});
+    else
+      multiply_and_stage(std::false_type{});
+    wave_sync_lds();
+    // Row-contiguous stores: 8 lanes cover the 64 dense columns of one row.
+    if (cb >= iw_first + 31 - w && cb + KC - 1 <= iw_first + w && iw_first + 31 < M) {
+      // every chunk of the wave's tile lies inside the band: nothing to decide, and each group of 8
+      // lanes writes one whole 128-byte line, which is what makes the streaming store pay
+#pragma unroll
+      for (int s = 0; s < 4; ++s) {
+        const u32x4 val = *reinterpret_cast<const u32x4 *>(st_src[s]);
+        if (ALIGNED)
+          store_chunk_streaming(st_dst[s] + cb, val);
+        else
+          store_chunk<false>(st_dst[s] + cb, val);
+      }
+      wave_sync_lds();
+      four_stores = true;
+    } else {
+      // pass A: whole chunks go out; head pieces are parked in the seam buffer.
+      u32x4 v[4];
+      int tail_hi[4];  // >= 0: this slot holds a tail piece with elements 0..tail_hi, handled in pass B
+#pragma unroll
+      for (int s = 0; s < 4; ++s) {
+        const int rw = wave * 32 + (lane >> 3) + 8 * s, r = rw & 31;
+        const int e_lo = st_lo[s] - cb, e_hi = st_hi[s] - cb;
+        tail_hi[s] = -1;
+        if (e_hi >= 0 && e_lo <= 7) {
+          v[s] = *reinterpret_cast<const u32x4 *>(st_src[s]);
+          uint16_t *dst = st_dst[s] + cb;
+          if (e_lo <= 0 && e_hi >= 7) {
+            store_chunk<ALIGNED>(dst, v[s]);  // (plain: lines of edge tiles are completed piecewise)
+          } else if (e_lo > 0) {  // head piece: elements e_lo..7 (W >= 17, so it reaches the chunk's end)
+            if (ALIGNED && rw > 0 && (r > 0 || seam_across_waves))
+              *reinterpret_cast<u32x4 *>(&seam[rw * 8]) = v[s];
+            else
+              store_chunk_elements(dst, v[s], e_lo, 7);
+          } else {
+            tail_hi[s] = e_hi;
+          }
+        }
+      }
+      wave_sync_lds();
+      // pass B: tail pieces pick up the head piece of the row below and leave as whole chunks.
+#pragma unroll
+      for (int s = 0; s < 4; ++s) {
+        if (tail_hi[s] >= 0) {
+          const int rw = wave * 32 + (lane >> 3) + 8 * s, r = rw & 31;
+          uint16_t *dst = st_dst[s] + cb;
+          if (ALIGNED && rw + 1 < TM && i0 + rw + 1 < M && (r < 31 || seam_across_waves)) {
+            const u32x4 head = *reinterpret_cast<const u32x4 *>(&seam[(rw + 1) * 8]);
+            const u32x4 mine_part = keep_range(v[s], 0, tail_hi[s]);
+            const u32x4 head_part = keep_range(head, tail_hi[s] + 1, 7);
+            u32x4 merged = {mine_part[0] | head_part[0], mine_part[1] | head_part[1], mine_part[2] | head_part[2],
+                            mine_part[3] | head_part[3]};
+            store_chunk<true>(dst, merged);
+          } else {
+            store_chunk_elements(dst, v[s], 0, tail_hi[s]);
+          }
+        }
+      }
+    }
+    return four_stores;
+  };
+
+  request(0);
+  bool four_stores = false;  // scalar: every lane of a wavefront takes the same store path
+  for (int k = 0; k < nk; ++k) {
+    // This wavefront's loads of chunk k are older than the stores of the slot before: when that slot
+    // issued exactly four of them they stay in flight, otherwise everything is waited for.  All LDS
+    // traffic of the wavefront (staging, seam buffer) is complete as well before the barrier, after
+    // which chunk k is in LDS for everyone and nobody reads chunk k - 1 any more.
+    if (four_stores)
+      wait_vmcnt_lgkm0<4>();
+    else
+      wait_vmcnt_lgkm0<0>();
+    __builtin_amdgcn_s_barrier();
+    request(k + 1);  // past the last chunk: zeros into a tile nobody reads
+    four_stores = slot(k);
+  }
+  wait_vmcnt<0>();  // the load past the last chunk must not outlive the workgroup's LDS
+}
+
+
+// ------------------------------------------------------------------------------------------
 // host side
 // ------------------------------------------------------------------------------------------
 bool shape_ok(int64_t M, int64_t N, int64_t w, int dtype) {
@@ -612,6 +824,18 @@ hipError_t launch_p1(const Problem &p, const View &x, const View &y, const View 
   hipLaunchKernelGGL((mfma_p1_kernel<T, NK, ALIGNED>), grid, block, 0, p.stream, (const uint16_t *)x.data,   \
                      (const uint16_t *)y.data, (uint16_t *)c.data, (int)p.B, (int)p.M, (int)p.w, nblk, galign, \
                      x.sb, x.sr, y.sb, y.sr, c.sb)
+  // N = 128 with whole-line band stores: Y chunks straight into LDS, three workgroups per CU (32-bit
+  // byte offsets inside a batch element).  With 16-byte column groups most slots take the piecewise
+  // store path, whose stores this kernel waits for: 10 % slower there than the kernel above.
+  if (ALIGNED && galign == 64 && !(p.flags & WM_FLAG_NO_LDS_DIRECT) && y.sr > 0 &&
+      (p.M + 2 * KC) * y.sr * 2 < 0x7fffffff && p.N == 128) {
+    // (at N = 64, where the kernel above already places four workgroups on a CU, this variant measured
+    // equal at w = 256 and 512 and 8 % slower at w = 64)
+    hipLaunchKernelGGL((mfma_p1_dma_kernel<T, 8, ALIGNED>), grid, block, 0, p.stream, (const uint16_t *)x.data,
+                       (const uint16_t *)y.data, (uint16_t *)c.data, (int)p.B, (int)p.M, (int)p.w, nblk, galign, x.sb,
+                       x.sr, y.sb, y.sr, c.sb);
+    return hipGetLastError();
+  }
   switch (p.N / 16) {
     case 1: WM_P1(1); break;
     case 2: WM_P1(2); break;

@@ -244,6 +244,12 @@ __device__ __forceinline__ void wait_vmcnt() {
   __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (15 << 8));
 }
 
+// s_waitcnt vmcnt(n) lgkmcnt(0): additionally all of the wave's LDS traffic is complete.
+template <int N>
+__device__ __forceinline__ void wait_vmcnt_lgkm0() {
+  __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (0 << 8));
+}
+
 // Raw buffer descriptor (four scalar registers) over `bytes` bytes at p: loads beyond the end
 // return zeros.
 __device__ __forceinline__ u32x4 make_rsrc(const void *p, uint32_t bytes) {
