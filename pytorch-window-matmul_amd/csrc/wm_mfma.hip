@@ -752,6 +752,220 @@ __global__ __launch_bounds__(kThreads, 3) void mfma_p1_dma_kernel(const uint16_t
 
 
 // ------------------------------------------------------------------------------------------
+// P3 with band tile and Y chunk loaded straight into LDS (whole-line column groups, N = 64 or 128)
+// ------------------------------------------------------------------------------------------
+// Same tiling and arithmetic as mfma_p3_kernel.  Nothing passes through registers on its way to LDS:
+// when the column groups are whole 128-byte lines every row of the skewed tile is 256 aligned bytes
+// of memory, 2w elements below the row before it, so the tile is a strided block that buffer loads
+// with the lds modifier copy as it is (swizzled through which piece a lane fetches).  What the
+// register path did to a chunk before storing it to LDS -- clearing the entries that belong to a
+// neighbouring band row or lie past the sequence -- is done on the operand after it is read from
+// LDS, and only in the chunks of a wavefront's 32 columns that need it; chunks that lie wholly
+// outside those columns' band are not multiplied at all.  Rows of Y past the sequence read as zeros
+// (buffer range check); DEPTH chunks are in flight per workgroup, counted by the kernel itself.
+#ifndef WM_P3_DMA_KC
+#define WM_P3_DMA_KC 64
+#endif
+#ifndef WM_P3_DMA_STAGES
+#define WM_P3_DMA_STAGES 2
+#endif
+template <typename T, int NK, int KCH, int STAGES>
+__global__ __launch_bounds__(kThreads, (160 * 1024 / (STAGES * KCH * (2 * TM + 32 * NK)) >= 3 ? 3 : 2)) void mfma_p3_dma_kernel(
+    const uint16_t *__restrict__ A, const uint16_t *__restrict__ Y, uint16_t *__restrict__ C, int B, int M, int w,
+    int nblk, int galign, int64_t asb, int64_t ysb, int64_t ysr, int64_t csb, int64_t csr) {
+  constexpr int N = 16 * NK, NT = NK / 2, CH = KCH, DEPTH = STAGES - 1;
+  using TT = LdsTile<CH, TM / 8>;      // [CH rows r][TM columns c]
+  using YT = LdsTile<CH, N / 8>;       // [CH rows r][N]
+  constexpr int LOADS = TT::LOADS + YT::LOADS;
+  static_assert(NK == 4 || NK == 8, "Y tile rows of 128 or 256 bytes");
+  static_assert(CH % 16 == 0 && STAGES >= 2 && DEPTH * LOADS < 64, "vmcnt holds 6 bits");
+  __shared__ __attribute__((aligned(1024))) uint16_t t_lds[STAGES][TT::ELEMS];
+  __shared__ __attribute__((aligned(1024))) uint16_t y_lds[STAGES][YT::ELEMS];
+
+  int b, blk;
+  if (!decode_block(nblk, B, &b, &blk)) return;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int W = 2 * w + 1;
+  const int64_t a0 = (int64_t)b * asb;
+  const int a_rem = (int)(a0 & 63);
+  // element (r, c0) of this batch element starts a 128-byte line (galign 64) or a 16-byte piece (8)
+  const int c0 = blk * TM - ((a_rem + w) & (galign - 1));
+  const int c_first = max(c0, 0), c_last = min(c0 + TM, M) - 1;
+  if (c_first > c_last) return;
+  const int r_lo = max(c_first - w, 0), r_hi = min(c_last + w, M - 1);
+  const int nk = (r_hi - r_lo + CH) / CH;
+
+  // band: the buffer starts at the 128-byte line that holds the batch element's first entry and ends
+  // with the batch element; tile row r, column c0 is at element a_rem + r 2w + c0 + w of it
+  const u32x4 t_rsrc = make_rsrc(A + (a0 - a_rem), (uint32_t)(((int64_t)a_rem + (int64_t)M * W) * 2));
+  const uint32_t t_voff = TT::lane_offset(wave, lane, 2 * w), t_step = TT::step(2 * w);
+  const uint32_t t_col0 = (uint32_t)(a_rem + c0 + w) * 2, t_row = (uint32_t)(4 * w);  // bytes
+  const u32x4 y_rsrc = make_rsrc(Y + (int64_t)b * ysb, (uint32_t)(((int64_t)(M - 1) * ysr + N) * 2));
+  const uint32_t y_voff = YT::lane_offset(wave, lane, ysr), y_step = YT::step(ysr), y_row = (uint32_t)(ysr * 2);
+  auto request = [&](int k, int stage) {  // chunks past the last one read zeros or rows nobody multiplies
+    const uint32_t rb = (uint32_t)(r_lo + k * CH);
+    TT::request(t_rsrc, t_lds[stage], wave, t_voff, t_col0 + rb * t_row, t_step);
+    YT::request(y_rsrc, y_lds[stage], wave, y_voff, rb * y_row, y_step);
+  };
+
+  f32x16 acc[NT];
+#pragma unroll
+  for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) acc[nt][v] = 0.f;
+
+  // this wavefront's columns and, per lane, the band rows that hold an entry of its column
+  const int cw0 = c0 + 32 * wave;
+  const int c_mine = cw0 + (lane & 31);
+  const int row_lo = c_mine - w, row_hi = min(c_mine + w, M - 1);
+  const uint32_t t_at = TT::tr_at(lane), y_at = YT::tr_at(lane);
+  auto multiply = [&](int rb, int stage, auto edge) {
+    u32x4 bop[CH / 16], aop[CH / 16][NT];
+#pragma unroll
+    for (int ks = 0; ks < CH / 16; ++ks) {
+      bop[ks] = TT::cols(t_lds[stage], t_at, 16 * ks, wave);
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt) aop[ks][nt] = YT::cols(y_lds[stage], y_at, 16 * ks, nt);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int ks = 0; ks < CH / 16; ++ks) {
+      if (decltype(edge)::value) bop[ks] = keep_rows_tr(bop[ks], rb + 16 * ks + 4 * (lane >> 5), row_lo, row_hi);
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt) acc[nt] = Mma<T>::run(aop[ks][nt], bop[ks], acc[nt]);
+    }
+  };
+
+#pragma unroll
+  for (int s = 0; s < DEPTH; ++s) request(s, s);
+  int stage = 0, ahead = DEPTH % STAGES;  // stage of chunk k, stage of chunk k + DEPTH
+  for (int k = 0; k < nk; ++k) {
+    // this wavefront's part of chunk k has landed; after the barrier all of it has, and nobody reads
+    // chunk k - 1 any more, whose stage the next request overwrites
+    wait_vmcnt<(DEPTH - 1) * LOADS>();
+    __builtin_amdgcn_s_barrier();
+    request(k + DEPTH, ahead);
+    const int rb = r_lo + k * CH;
+    if (rb - w <= cw0 + 31 && cw0 <= rb + CH - 1 + w) {  // else: no row of the chunk reaches these columns
+      if (rb + CH - 1 - w <= cw0 && cw0 + 31 <= rb + w && rb + CH - 1 <= M - 1)
+        multiply(rb, stage, std::false_type{});
+      else
+        multiply(rb, stage, std::true_type{});
+    }
+    stage = stage + 1 == STAGES ? 0 : stage + 1;
+    ahead = ahead + 1 == STAGES ? 0 : ahead + 1;
+  }
+  // the loads past the last chunk must have landed before the tiles are reused for the result rows
+  wait_vmcnt<0>();
+  __syncthreads();
+  static_assert(4 * RowStage<NT>::ELEMS <= STAGES * TT::ELEMS, "the four staging areas must fit the band tile buffers");
+  store_wave_rows<T, NT>(&t_lds[0][0] + wave * RowStage<NT>::ELEMS, acc, 1.0f, C + (int64_t)b * csb, csr, cw0, M, N,
+                         lane);
+}
+
+// ------------------------------------------------------------------------------------------
+// P2 with band tile and Y chunk loaded straight into LDS (aligned column groups, N = 64 or 128)
+// ------------------------------------------------------------------------------------------
+// mfma_p2_kernel organised like mfma_p3_dma_kernel above: the band tile [128 rows][64 dense columns]
+// is a strided block of 128-byte rows in memory, 2w elements apart.  The first chunk of a tile may
+// begin before dense column 0: its position goes into the lanes' offsets, so that exactly the
+// pieces before the buffer read as zeros.
+template <typename T, int NK, int STAGES>
+__global__ __launch_bounds__(kThreads, (160 * 1024 / (STAGES * KC * (2 * TM + 32 * NK)) >= 3 ? 3 : 2)) void mfma_p2_dma_kernel(
+    const uint16_t *__restrict__ A, const uint16_t *__restrict__ Y, uint16_t *__restrict__ C, int B, int M, int w,
+    int nblk, int galign, int64_t asb, int64_t ysb, int64_t ysr, int64_t csb, int64_t csr) {
+  constexpr int N = 16 * NK, NT = NK / 2, DEPTH = STAGES - 1;
+  using TT = LdsTile<TM, KC / 8>;  // [TM rows i][KC dense columns c]
+  using YT = LdsTile<KC, N / 8>;   // [KC rows c][N]
+  constexpr int LOADS = TT::LOADS + YT::LOADS;
+  static_assert(NK == 4 || NK == 8, "Y tile rows of 128 or 256 bytes");
+  static_assert(KC == 64 && STAGES >= 2 && DEPTH * LOADS < 64, "band tile rows of 128 bytes; vmcnt holds 6 bits");
+  __shared__ __attribute__((aligned(1024))) uint16_t t_lds[STAGES][TT::ELEMS];
+  __shared__ __attribute__((aligned(1024))) uint16_t y_lds[STAGES][YT::ELEMS];
+
+  int b, blk;
+  if (!decode_block(nblk, B, &b, &blk)) return;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int W = 2 * w + 1;
+  const int i0 = blk * TM;
+  const int rows = min(TM, M - i0);
+  const int c_lo = max(i0 - w, 0), c_hi = min(i0 + rows - 1 + w, M - 1);
+  const int64_t a0 = (int64_t)b * asb;
+  const int a_rem = (int)(a0 & 63);
+  const int c_start = c_lo - ((c_lo + a_rem + w) & (galign - 1));
+  const int nk = (c_hi - c_start + KC) / KC;
+
+  // band: buffer from the 128-byte line that holds the batch element's first entry to the end of the
+  // batch element; tile row i, dense column c is at element a_rem + i 2w + c + w of it
+  const u32x4 t_rsrc = make_rsrc(A + (a0 - a_rem), (uint32_t)(((int64_t)a_rem + (int64_t)M * W) * 2));
+  const uint32_t t_voff = TT::lane_offset(wave, lane, 2 * w) + (uint32_t)(a_rem + (int64_t)i0 * 2 * w + w) * 2;
+  const uint32_t t_step = TT::step(2 * w);
+  const u32x4 y_rsrc = make_rsrc(Y + (int64_t)b * ysb, (uint32_t)(((int64_t)(M - 1) * ysr + N) * 2));
+  const uint32_t y_voff = YT::lane_offset(wave, lane, ysr), y_step = YT::step(ysr), y_row = (uint32_t)(ysr * 2);
+  auto request = [&](int k, int stage) {  // 32-bit wrap-around on purpose: rows before the buffer are out of range
+    const int cb = c_start + k * KC;
+    TT::request_at(t_rsrc, t_lds[stage], wave, t_voff + (uint32_t)(2 * cb), t_step);
+    YT::request_at(y_rsrc, y_lds[stage], wave, y_voff + (uint32_t)cb * y_row, y_step);
+  };
+
+  f32x16 acc[NT];
+#pragma unroll
+  for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) acc[nt][v] = 0.f;
+
+  // this wavefront's rows and, per lane, the dense columns that its row's band holds
+  const int iw0 = i0 + 32 * wave;
+  const int i_mine = iw0 + (lane & 31);
+  const int col_lo = max(i_mine - w, 0), col_hi = i_mine < M ? min(i_mine + w, M - 1) : -1;
+  const uint32_t t_at = TT::row_at(lane), y_at = YT::tr_at_seq(lane);
+  auto multiply = [&](int cb, int stage, auto edge) {
+    u32x4 bop[KC / 16], aop[KC / 16][NT];
+#pragma unroll
+    for (int ks = 0; ks < KC / 16; ++ks) {
+      bop[ks] = TT::rows(t_lds[stage], t_at, wave, ks);
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt) aop[ks][nt] = YT::cols_seq(y_lds[stage], y_at, 16 * ks, nt);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int ks = 0; ks < KC / 16; ++ks) {
+      if (decltype(edge)::value) {
+        const int c8 = cb + 16 * ks + 8 * (lane >> 5);
+        bop[ks] = mask_band_chunk(bop[ks], col_lo - c8, col_hi - c8);
+      }
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt) acc[nt] = Mma<T>::run(aop[ks][nt], bop[ks], acc[nt]);
+    }
+  };
+
+#pragma unroll
+  for (int s = 0; s < DEPTH; ++s) request(s, s);
+  int stage = 0, ahead = DEPTH % STAGES;
+  for (int k = 0; k < nk; ++k) {
+    wait_vmcnt<(DEPTH - 1) * LOADS>();
+    __builtin_amdgcn_s_barrier();
+    request(k + DEPTH, ahead);
+    const int cb = c_start + k * KC;
+    if (cb <= iw0 + 31 + w && iw0 - w <= cb + KC - 1) {  // else: no column of the chunk lies in these rows' bands
+      if (cb >= max(iw0 + 31 - w, 0) && cb + KC - 1 <= min(iw0 + w, M - 1) && iw0 + 31 <= M - 1)
+        multiply(cb, stage, std::false_type{});
+      else
+        multiply(cb, stage, std::true_type{});
+    }
+    stage = stage + 1 == STAGES ? 0 : stage + 1;
+    ahead = ahead + 1 == STAGES ? 0 : ahead + 1;
+  }
+  wait_vmcnt<0>();
+  __syncthreads();
+  static_assert(4 * RowStage<NT>::ELEMS <= STAGES * TT::ELEMS, "the four staging areas must fit the band tile buffers");
+  store_wave_rows<T, NT>(&t_lds[0][0] + wave * RowStage<NT>::ELEMS, acc, 1.0f, C + (int64_t)b * csb, csr, iw0, M, N,
+                         lane);
+}
+
+// ------------------------------------------------------------------------------------------
 // host side
 // ------------------------------------------------------------------------------------------
 bool shape_ok(int64_t M, int64_t N, int64_t w, int dtype) {
@@ -772,6 +986,12 @@ int band_group(const View &v, int64_t w) { return (w % 32 == 0 && ((uintptr_t)v.
 
 unsigned grid_size(int64_t B, int64_t nblk) { return (unsigned)(((B + 7) / 8) * 8 * nblk); }
 
+// Shapes the kernels that load their tiles straight into LDS accept (band-in products).
+bool lds_direct_ok(bool aligned, const Problem &p, const View &y) {
+  return aligned && !(p.flags & WM_FLAG_NO_LDS_DIRECT) && (p.N == 64 || p.N == 128) && y.sr > 0 &&
+         (p.M + 4 * KC) * (2 * p.w + 1) * 2 + 256 < 0x7fffffff && (p.M + 4 * KC) * y.sr * 2 < 0x7fffffff;
+}
+
 // Chunk length of P2 (64: the result rows are staged in the band tile buffers, which 32 would make
 // too small; 32 and 128 were measured slower before that).
 #ifndef WM_P2_KC
@@ -782,6 +1002,23 @@ hipError_t launch_p2(const Problem &p, const View &a, const View &y, const View 
   const int nblk = (int)((p.M + TM - 1) / TM);
   const int galign = band_group(a, p.w);
   const dim3 grid(grid_size(p.B, nblk)), block(kThreads);
+  // Tiles straight into LDS (N = 64 / 128, 16-byte column groups, 32-bit byte offsets inside a batch
+  // element of the band and of Y, chunks past the end included) where that was measured faster than
+  // the register-staged kernel: up to w = 128 (30 % at w = 36, 14 % at w = 64) and at N = 128 with
+  // whole-line groups (3-5 % at w = 512).  At N = 64 and w = 256 the two are equal, and once the band
+  // outgrows the last-level cache the staged kernel, with two chunks per workgroup in flight, is
+  // 7-9 % faster (B = 384 at w = 256, B = 32 at M = 32768 and w = 512).
+  if (lds_direct_ok(ALIGNED, p, y) && (p.w <= 128 || (p.N == 128 && galign == 64))) {
+    if (p.N == 64)
+      hipLaunchKernelGGL((mfma_p2_dma_kernel<T, 4, 2>), grid, block, 0, p.stream, (const uint16_t *)a.data,
+                         (const uint16_t *)y.data, (uint16_t *)c.data, (int)p.B, (int)p.M, (int)p.w, nblk, galign, a.sb,
+                         y.sb, y.sr, c.sb, c.sr);
+    else
+      hipLaunchKernelGGL((mfma_p2_dma_kernel<T, 8, 2>), grid, block, 0, p.stream, (const uint16_t *)a.data,
+                         (const uint16_t *)y.data, (uint16_t *)c.data, (int)p.B, (int)p.M, (int)p.w, nblk, galign, a.sb,
+                         y.sb, y.sr, c.sb, c.sr);
+    return hipGetLastError();
+  }
 #define WM_P2(NT)                                                                                              \
   hipLaunchKernelGGL((mfma_p2_kernel<T, NT, ALIGNED, WM_P2_KC>), grid, block, 0, p.stream, (const uint16_t *)a.data,     \
                      (const uint16_t *)y.data, (uint16_t *)c.data, (int)p.B, (int)p.M, (int)p.N, (int)p.w, nblk, \
@@ -801,6 +1038,21 @@ hipError_t launch_p3(const Problem &p, const View &a, const View &y, const View 
   const int galign = band_group(a, p.w);
   const int nblk = (int)((p.M + (ALIGNED ? galign - 1 : 0) + TM - 1) / TM);
   const dim3 grid(grid_size(p.B, nblk)), block(kThreads);
+  // Tiles straight into LDS, as for the band-in product above; measured against the register-staged
+  // kernel: whole-line column groups 6-10 % faster at w = 256 and 512, 22 % at w = 64, equal to 2 %
+  // slower once the band outgrows the last-level cache; 16-byte groups 36 % faster at w = 36, 10 % at
+  // w = 100, 9 % slower at w = 260.
+  if (lds_direct_ok(ALIGNED, p, y) && (galign == 64 || p.w <= 128)) {
+    if (p.N == 64)
+      hipLaunchKernelGGL((mfma_p3_dma_kernel<T, 4, WM_P3_DMA_KC, WM_P3_DMA_STAGES>), grid, block, 0, p.stream,
+                         (const uint16_t *)a.data, (const uint16_t *)y.data, (uint16_t *)c.data, (int)p.B, (int)p.M,
+                         (int)p.w, nblk, galign, a.sb, y.sb, y.sr, c.sb, c.sr);
+    else
+      hipLaunchKernelGGL((mfma_p3_dma_kernel<T, 8, WM_P3_DMA_KC, WM_P3_DMA_STAGES>), grid, block, 0, p.stream,
+                         (const uint16_t *)a.data, (const uint16_t *)y.data, (uint16_t *)c.data, (int)p.B, (int)p.M,
+                         (int)p.w, nblk, galign, a.sb, y.sb, y.sr, c.sb, c.sr);
+    return hipGetLastError();
+  }
 #define WM_P3(NT)                                                                                              \
   hipLaunchKernelGGL((mfma_p3_kernel<T, NT, ALIGNED>), grid, block, 0, p.stream, (const uint16_t *)a.data,     \
                      (const uint16_t *)y.data, (uint16_t *)c.data, (int)p.B, (int)p.M, (int)p.N, (int)p.w, nblk, \

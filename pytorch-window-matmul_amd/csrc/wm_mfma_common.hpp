@@ -301,6 +301,92 @@ __device__ __forceinline__ uint32_t dma_lane_offset(int wave, int lane, int64_t 
   return (uint32_t)(row * row_stride_elems * 2 + piece * 16);
 }
 
+// A swizzled tile of ROWS rows x PPR pieces as the loads above fill it, generalised to any row count
+// whose pieces divide evenly over the four wavefronts: the loading side (which piece a lane
+// fetches, how the wave's loads step through the rows) and the two ways the MFMA kernels read it.
+template <int ROWS, int PPR>
+struct LdsTile {
+  static_assert((ROWS * PPR) % 256 == 0 && (PPR == 8 || PPR == 16), "whole wave-level loads; rows of 128 or 256 bytes");
+  static constexpr int LOADS = ROWS * PPR / 256;  // wave-level loads per wavefront and tile
+  static constexpr int ROWB = 16 * PPR;           // bytes per row
+  static constexpr int ELEMS = ROWS * PPR * 8;    // 16-bit elements per tile
+  typedef s16x4 __attribute__((address_space(3))) * lds_tr_ptr;
+  // the lane's byte offset inside a tile's memory image for the first of the wave's loads
+  static __device__ __forceinline__ uint32_t lane_offset(int wave, int lane, int64_t row_stride_elems) {
+    return dma_lane_offset<PPR>(wave, lane, row_stride_elems);
+  }
+  // bytes in memory between two of the wave's loads (256 / PPR rows)
+  static __device__ __forceinline__ uint32_t step(int64_t row_stride_elems) {
+    return (uint32_t)(256 / PPR * row_stride_elems * 2);
+  }
+  static __device__ __forceinline__ void request(u32x4 rsrc, const uint16_t *tile, int wave, uint32_t voff,
+                                                 uint32_t bytes0, uint32_t step_bytes) {
+    const uint32_t base = lds_address(tile) + 1024 * wave;
+#pragma unroll
+    for (int j = 0; j < LOADS; ++j) dma_piece(rsrc, base + 4096 * j, voff, bytes0 + step_bytes * j);
+  }
+  // Reading.  row_at: lane -> row lane % 32, piece lane / 32 (add 32 r0 ROWB for other rows, XOR
+  // 32 ks for pieces 2 ks + lane / 32): operand with the contraction along the row.
+  static __device__ __forceinline__ uint32_t row_at(int lane) {
+    const int r32 = lane & 31, half = lane >> 5;
+    return (uint32_t)(r32 * ROWB + ((half ^ swz(r32)) << 4));
+  }
+  static __device__ __forceinline__ u32x4 rows(const uint16_t *tile, uint32_t at, int blk, int ks) {
+    return *reinterpret_cast<const u32x4 *>(reinterpret_cast<const char *>(tile) + 32 * blk * ROWB + (at ^ (32 * ks)));
+  }
+  // tr_at / cols: operand with the contraction along the rows of the tile, read transposed.  The
+  // lane gets column 32 cb + lane % 32 of rows r0 + 4 (lane / 32) + {0, 1, 2, 3, 8, 9, 10, 11},
+  // r0 a multiple of 16.
+  static __device__ __forceinline__ uint32_t tr_at(int lane) {
+    const int s16 = lane & 15, grp = lane >> 4, rowl = 4 * (grp >> 1) + (s16 >> 2);
+    return (uint32_t)(rowl * ROWB + (((2 * (grp & 1) + ((s16 & 3) >> 1)) ^ swz(rowl)) << 4) + 8 * (s16 & 1));
+  }
+  static __device__ __forceinline__ u32x4 cols(const uint16_t *tile, uint32_t at, int r0, int cb) {
+    const char *p = reinterpret_cast<const char *>(tile) + r0 * ROWB + (at ^ (64 * cb));
+    const u32x2 lo = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr_ptr)(p)));
+    const u32x2 hi = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr_ptr)(p + 8 * ROWB)));
+    const u32x4 r = {lo[0], lo[1], hi[0], hi[1]};
+    return r;
+  }
+  // tr_at_seq / cols_seq: the same read with the lane's eight rows consecutive,
+  // r0 + 8 (lane / 32) + {0 .. 7}: the order in which `rows` of another tile delivers its pieces.
+  static __device__ __forceinline__ uint32_t tr_at_seq(int lane) {
+    const int s16 = lane & 15, grp = lane >> 4, rowl = 8 * (grp >> 1) + (s16 >> 2);
+    return (uint32_t)(rowl * ROWB + (((2 * (grp & 1) + ((s16 & 3) >> 1)) ^ swz(rowl)) << 4) + 8 * (s16 & 1));
+  }
+  static __device__ __forceinline__ u32x4 cols_seq(const uint16_t *tile, uint32_t at, int r0, int cb) {
+    const char *p = reinterpret_cast<const char *>(tile) + r0 * ROWB;
+    // four rows further down the swizzle differs in its lowest bit
+    const u32x2 lo = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr_ptr)(p + (at ^ (64 * cb)))));
+    const u32x2 hi = __builtin_bit_cast(
+        u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr_ptr)(p + 4 * ROWB + (at ^ 16 ^ (64 * cb)))));
+    const u32x4 r = {lo[0], lo[1], hi[0], hi[1]};
+    return r;
+  }
+  // `request` with the position of the tile folded into the lane's offset: a tile that begins
+  // before the buffer then has its first rows out of range (zeros) instead of all of them
+  static __device__ __forceinline__ void request_at(u32x4 rsrc, const uint16_t *tile, int wave, uint32_t voff,
+                                                    uint32_t step_bytes) {
+    const uint32_t base = lds_address(tile) + 1024 * wave;
+#pragma unroll
+    for (int j = 0; j < LOADS; ++j) dma_piece(rsrc, base + 4096 * j, voff + step_bytes * j, 0);
+  }
+};
+
+// Clears the elements of a transposed-read operand (LdsTile::cols) whose row lies outside [lo, hi];
+// r_first is the row of the lane's element 0.
+__device__ __forceinline__ u32x4 keep_rows_tr(u32x4 v, int r_first, int lo, int hi) {
+  u32x4 r;
+#pragma unroll
+  for (int d = 0; d < 4; ++d) {
+    const int ra = r_first + 2 * (d & 1) + 8 * (d >> 1);
+    const uint32_t l = (ra >= lo && ra <= hi) ? 0x0000ffffu : 0u;
+    const uint32_t h = (ra + 1 >= lo && ra + 1 <= hi) ? 0xffff0000u : 0u;
+    r[d] = v[d] & (l | h);
+  }
+  return r;
+}
+
 // Workgroup -> (batch, block).  Workgroups are dealt round-robin to the 8 XCDs, each with
 // its own L2; all blocks of one batch element are given to one XCD so that neighbouring
 // blocks find the rows they share (the +-w halo) in that L2.

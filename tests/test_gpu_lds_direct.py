@@ -1,0 +1,97 @@
+"""The kernels that load their tiles straight into LDS, against the register-staged kernels and the oracle.
+
+At N = 64 / 128 the wide-band family has a second implementation of each product whose chunks never
+pass through registers (band-out product at N = 128 with whole-line column groups; band-in
+products for windows that are a multiple of 4).  ``WM_FLAG_NO_LDS_DIRECT`` switches them off, so
+every shape here runs both ways: the results must agree within the 16-bit tolerance (rtol = atol =
+2e-2; bit for bit where the order of the sums is the same: band-out and band-in product), and both
+must match the CPU oracle.  Shapes cover ragged sequence ends, sequences shorter than a tile,
+batch elements whose band does not start on a 128-byte line, operands with padded rows and
+batches, and invalid band entries filled with NaN.
+"""
+import pytest
+import torch
+
+import oracle
+import wm_ctypes as abi
+from conftest import seeded
+
+pytestmark = pytest.mark.gpu
+
+TOL = dict(rtol=2e-2, atol=2e-2)
+# (B, M, N, w): windows that are multiples of 32 (whole-line column groups) and of 4 only
+SHAPES = [(3, 1000, 64, 64), (2, 777, 128, 32), (2, 300, 64, 96), (5, 129, 128, 64), (3, 50, 64, 32), (1, 1, 64, 32),
+          (2, 515, 128, 160), (3, 1000, 64, 100), (2, 777, 128, 36), (5, 515, 64, 8), (3, 301, 64, 44), (2, 64, 128, 12),
+          (2, 2049, 64, 1024), (1, 700, 64, 128)]
+
+
+def bits(t):
+    return t.contiguous().view(torch.int16)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bfloat16", "float16"])
+@pytest.mark.parametrize("B,M,N,w", SHAPES, ids=[f"B{B}-M{M}-N{N}-w{w}" for B, M, N, w in SHAPES])
+def test_both_implementations_and_oracle(device, B, M, N, w, dtype):
+    print(f"case B{B} M{M} N{N} w{w} {dtype}", flush=True)
+    q, k, v, go = (seeded((B, M, N), 300 + s, dtype) for s in range(4))
+    a, ga = (seeded((B, M, 2 * w + 1), 310 + s, dtype, 0.25) for s in range(2))
+    # entries of an input band outside the sequence must never be read as numbers
+    outside = ~oracle.band_mask(M, w, torch.device("cpu"))
+    a[:, outside] = float("nan")
+    ga[:, outside] = float("nan")
+    dq, dk, dv, dgo, da, dga = (t.to(device) for t in (q, k, v, go, a, ga))
+    kt = dk.transpose(1, 2)
+    res = []
+    for flags in (0, abi.NO_LDS_DIRECT):
+        att = abi.window_forward(dq, kt, w, flags)
+        out = abi.unwindow_forward(da, dv, w, flags)
+        g_a, g_v = abi.unwindow_backward(da, dv, w, dgo, flags)
+        g_q, g_k = abi.window_backward(dq, kt, w, dga, flags)
+        res.append(dict(window_fwd=att, unwindow_fwd=out, grad_a=g_a, grad_v=g_v, grad_q=g_q, grad_k=g_k))
+    for name in res[0]:
+        torch.testing.assert_close(res[0][name].float(), res[1][name].float(), **TOL, msg=lambda m: f"{name}: {m}")
+    for name in ("window_fwd", "grad_a", "unwindow_fwd", "grad_q"):
+        assert torch.equal(bits(res[0][name]), bits(res[1][name])), f"{name}: the two implementations sum in the same order"
+    if B * M * (2 * w + 1) <= 2_500_000:  # the oracle's loops finish in seconds
+        f = lambda t: t.float()  # noqa: E731
+        a0, ga0 = a.clone(), ga.clone()
+        a0[:, outside] = 0
+        ga0[:, outside] = 0
+        ktc = f(k).transpose(1, 2).contiguous()
+        want_a, want_v = oracle.unwindow_matmul_backward(f(a0), f(v), w, f(go))
+        want_q, want_k = oracle.window_matmul_backward(f(q), ktc, w, f(ga0))
+        want = dict(window_fwd=oracle.window_matmul_forward(f(q), ktc, w), unwindow_fwd=oracle.unwindow_matmul_forward(f(a0), f(v), w),
+                    grad_a=want_a, grad_v=want_v, grad_q=want_q, grad_k=want_k)
+        for name in want:
+            torch.testing.assert_close(res[0][name].cpu().float(), want[name], **TOL, msg=lambda m: f"{name} vs oracle: {m}")
+
+
+@pytest.mark.parametrize("w", [32, 44])
+def test_padded_operands(device, w):
+    """Rows of v / grad_o / q padded to a longer stride, batch elements of the band padded so that they
+    start at every 16-byte position of a 128-byte line, results written into padded tensors."""
+    B, M, N, dtype = 4, 333, 64, torch.bfloat16
+    W = 2 * w + 1
+    pad_rows = lambda t: torch.cat([t, torch.full_like(t, float("nan"))], -1)[..., :N]  # noqa: E731  row stride 2N
+    v, go = (seeded((B, M, N), 320 + s, dtype).to(device) for s in range(2))
+    band_store = torch.full((B, M * W + 24), float("nan"), dtype=dtype, device=device)  # batch stride not a multiple of 64
+    a = band_store[:, :M * W].view(B, M, W)
+    a.copy_(seeded((B, M, W), 330, dtype, 0.25))
+    vp, gop = pad_rows(v), pad_rows(go)
+    assert vp.stride(1) == 2 * N and a.stride(0) == M * W + 24
+    for flags in (abi.NO_LDS_DIRECT, 0):
+        out = abi.unwindow_forward(a, vp, w, flags)
+        _, g_v = abi.unwindow_backward(a, vp, w, gop, flags, want_a=False)
+        if flags:
+            want_out, want_gv = out, g_v
+    assert torch.equal(bits(out), bits(want_out))
+    torch.testing.assert_close(g_v.float(), want_gv.float(), **TOL)
+    ref_out = abi.unwindow_forward(a.contiguous(), v, w, abi.FORCE_STRIDED)
+    torch.testing.assert_close(out.float(), ref_out.float(), **TOL)
+
+
+def test_kernel_choice_is_unchanged_by_the_switch(device):
+    """Both implementations belong to the wide-band family: wm_kernel_choice names the family."""
+    for op in (1, 2, 3):
+        for flags in (0, abi.NO_LDS_DIRECT):
+            assert abi.lib().wm_kernel_choice(op, 8, 4096, 128, 64, abi.DTYPES[torch.bfloat16], 1, flags).decode() == f"mfma_p{op}"
