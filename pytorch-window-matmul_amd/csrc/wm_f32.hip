@@ -14,6 +14,8 @@
 // 16-byte LDS read per group (4 steps) instead of one 4-byte read per step.
 #include "wm_common.hpp"
 
+#include <algorithm>
+
 namespace wm {
 namespace {
 
@@ -105,8 +107,11 @@ __global__ __launch_bounds__(kThreads, NT <= 2 ? 3 : 2) void f32_band_in_kernel(
   const int k_lo = max(o0 - w, 0), k_hi = min(o1 + w, M - 1);  // contraction range (c for P2, r for P3)
   const int nk = (k_hi - k_lo + KC) / KC;
   const float *Ab = A + (int64_t)b * asb;
-  const float *Yb = Y + (int64_t)b * ysb;
-  const int ncg = N >> 2, ychunks = KC * ncg;
+  // blockIdx.y selects which NP columns of Y and C this workgroup works on (one workgroup does all
+  // of them unless the launch splits the columns to fill the chip)
+  const int h0 = NP * blockIdx.y;
+  const float *Yb = Y + (int64_t)b * ysb + h0;
+  const int ncg = min(N - h0, NP) >> 2, ychunks = KC * ncg;
   int y_row[NT], y_col[NT];  // this thread's pieces of a Y chunk; row KC = none
 #pragma unroll
   for (int s = 0; s < NT; ++s) {
@@ -264,7 +269,8 @@ __global__ __launch_bounds__(kThreads, NT <= 2 ? 3 : 2) void f32_band_in_kernel(
   // of its rows at a time in a private area and the rows leave as 16-byte pieces, 8 consecutive
   // lanes on one 128-byte line (non-temporal: the result is not read again here).
   float *stage = &t_lds[0][0] + wave * (32 * kStage);
-  float *Cb = C + (int64_t)b * csb;
+  float *Cb = C + (int64_t)b * csb + h0;
+  N -= h0;
 #pragma unroll
   for (int t = 0; t < NT; ++t) {
     wave_sync_lds();
@@ -311,8 +317,14 @@ __global__ __launch_bounds__(kThreads, NK8 <= 8 ? 4 : 2) void f32_band_out_kerne
   const int W = 2 * w + 1;
   const int i0 = blk * TM;
   const int rows = min(TM, M - i0);
-  const int c_lo = i0 - w, c_hi = i0 + rows - 1 + w;  // not clipped: entries outside the sequence are zeros
-  const int nk = (c_hi - c_lo + KC) / KC;
+  int c_lo = i0 - w;  // not clipped: entries outside the sequence are zeros
+  const int c_hi = i0 + rows - 1 + w;
+  int nk = (c_hi - c_lo + KC) / KC;
+  {  // blockIdx.y selects this workgroup's share of the chunks (all of them unless the launch splits them)
+    const int first = (int)((int64_t)nk * blockIdx.y / gridDim.y), last = (int)((int64_t)nk * (blockIdx.y + 1) / gridDim.y);
+    c_lo += first * KC;
+    nk = last - first;
+  }
   const float *Yb = Y + (int64_t)b * ysb;
   float *Cb = C + (int64_t)b * csb;
 
@@ -429,10 +441,25 @@ bool f32_shape_ok(int64_t M, int64_t N, int64_t w, int dtype) {
 bool f32_band_ok(const View &v, int64_t W) { return v.sc == 1 && v.sr == W && ((uintptr_t)v.data % 4) == 0; }
 unsigned f32_grid(int64_t B, int64_t nblk) { return (unsigned)(((B + 7) / 8) * 8 * nblk); }
 
+constexpr int64_t kCUs = 256;
+
 template <bool TRANSPOSED>
 hipError_t launch_band_in(const Problem &p, const View &a, const View &y, const View &c) {
   const int nblk = (int)((p.M + TM - 1) / TM);
-  const dim3 grid(f32_grid(p.B, nblk)), block(kThreads);
+  dim3 grid(f32_grid(p.B, nblk)), block(kThreads);
+  // A wavefront multiplies its 32 rows by every 32-column block of Y in turn.  When the workgroups
+  // do not even fill the CUs once or twice (config 5 at w = 1500: 168 of them), each block of
+  // columns gets workgroups of its own: the band tile is then fetched once per block (the
+  // workgroups that share it run on the same XCD at the same time), and the chip holds NB times
+  // as many wavefronts with a third or half of the work each.
+  const int64_t wgs = p.B * nblk, nb = (p.N + 31) / 32;
+  if (nb > 1 && wgs < 2 * kCUs && (wgs * nb + kCUs - 1) / kCUs < nb * ((wgs + kCUs - 1) / kCUs)) {
+    grid.y = (unsigned)nb;
+    hipLaunchKernelGGL((f32_band_in_kernel<1, TRANSPOSED>), grid, block, 0, p.stream, (const float *)a.data,
+                       (const float *)y.data, (float *)c.data, (int)p.B, (int)p.M, (int)p.N, (int)p.w, nblk, a.sb, y.sb,
+                       y.sr, c.sb, c.sr);
+    return hipGetLastError();
+  }
 #define WM_F32_IN(NT)                                                                                        \
   hipLaunchKernelGGL((f32_band_in_kernel<NT, TRANSPOSED>), grid, block, 0, p.stream, (const float *)a.data,  \
                      (const float *)y.data, (float *)c.data, (int)p.B, (int)p.M, (int)p.N, (int)p.w, nblk,   \
@@ -449,7 +476,11 @@ hipError_t launch_band_in(const Problem &p, const View &a, const View &y, const 
 
 hipError_t launch_band_out(const Problem &p, const View &x, const View &y, const View &c) {
   const int nblk = (int)((p.M + TM - 1) / TM);
-  const dim3 grid(f32_grid(p.B, nblk)), block(kThreads);
+  dim3 grid(f32_grid(p.B, nblk)), block(kThreads);
+  // too few workgroups to fill the chip: each takes a share of its tile's dense columns instead of
+  // all of them (nothing is fetched or computed twice: the shares produce disjoint parts of the band)
+  const int64_t wgs = p.B * nblk, chunks = (TM + 2 * p.w + KC - 1) / KC;
+  if (wgs < 2 * kCUs) grid.y = (unsigned)std::max<int64_t>(1, std::min<int64_t>(2 * kCUs / wgs, chunks / 4));
 #define WM_F32_OUT(NK8)                                                                                     \
   case NK8:                                                                                                 \
     hipLaunchKernelGGL((f32_band_out_kernel<NK8>), grid, block, 0, p.stream, (const float *)x.data,         \
