@@ -803,9 +803,20 @@ __global__ __launch_bounds__(kThreads, (160 * 1024 / (STAGES * KCH * (2 * TM + 3
   const uint32_t t_col0 = (uint32_t)(a_rem + c0 + w) * 2, t_row = (uint32_t)(4 * w);  // bytes
   const u32x4 y_rsrc = make_rsrc(Y + (int64_t)b * ysb, (uint32_t)(((int64_t)(M - 1) * ysr + N) * 2));
   const uint32_t y_voff = YT::lane_offset(wave, lane, ysr), y_step = YT::step(ysr), y_row = (uint32_t)(ysr * 2);
+  // A piece of the band tile (8 columns from c8 of band row r) holds an entry of the band only if
+  // c8 - r lies in [-w - 7, w]; the others are requested beyond the end of the buffer, which costs no
+  // memory traffic (a quarter of the tile's pieces at w = 2 TM).  c8 - r falls by CH per chunk.
+  int t_skew[TT::LOADS];
+#pragma unroll
+  for (int j = 0; j < TT::LOADS; ++j)
+    t_skew[j] = c0 + 8 * TT::load_piece(wave, lane) - (r_lo + TT::load_row(wave, lane, j)) + w + 7;
   auto request = [&](int k, int stage) {  // chunks past the last one read zeros or rows nobody multiplies
     const uint32_t rb = (uint32_t)(r_lo + k * CH);
-    TT::request(t_rsrc, t_lds[stage], wave, t_voff, t_col0 + rb * t_row, t_step);
+    uint32_t voff[TT::LOADS];
+#pragma unroll
+    for (int j = 0; j < TT::LOADS; ++j)
+      voff[j] = (uint32_t)(t_skew[j] - k * CH) <= (uint32_t)(2 * w + 7) ? t_voff : 0x80000000u;
+    TT::request_some(t_rsrc, t_lds[stage], wave, voff, t_col0 + rb * t_row, t_step);
     YT::request(y_rsrc, y_lds[stage], wave, y_voff, rb * y_row, y_step);
   };
 
@@ -904,9 +915,21 @@ __global__ __launch_bounds__(kThreads, (160 * 1024 / (STAGES * KC * (2 * TM + 32
   const uint32_t t_step = TT::step(2 * w);
   const u32x4 y_rsrc = make_rsrc(Y + (int64_t)b * ysb, (uint32_t)(((int64_t)(M - 1) * ysr + N) * 2));
   const uint32_t y_voff = YT::lane_offset(wave, lane, ysr), y_step = YT::step(ysr), y_row = (uint32_t)(ysr * 2);
+  // pieces of the band tile that hold no entry of the band (8 columns from c8 of row i with c8 - i
+  // outside [-w - 7, w]) are requested beyond the end of the buffer: no memory traffic for them
+  int t_skew[TT::LOADS];
+#pragma unroll
+  for (int j = 0; j < TT::LOADS; ++j)
+    t_skew[j] = c_start + 8 * TT::load_piece(wave, lane) - (i0 + TT::load_row(wave, lane, j)) + w + 7;
   auto request = [&](int k, int stage) {  // 32-bit wrap-around on purpose: rows before the buffer are out of range
     const int cb = c_start + k * KC;
-    TT::request_at(t_rsrc, t_lds[stage], wave, t_voff + (uint32_t)(2 * cb), t_step);
+    uint32_t voff[TT::LOADS];
+#pragma unroll
+    for (int j = 0; j < TT::LOADS; ++j)
+      voff[j] = (uint32_t)(t_skew[j] + k * KC) <= (uint32_t)(2 * w + 7)
+                    ? t_voff + (uint32_t)(2 * cb) + t_step * j
+                    : 0x80000000u;
+    TT::request_some(t_rsrc, t_lds[stage], wave, voff, 0, 0);
     YT::request_at(y_rsrc, y_lds[stage], wave, y_voff + (uint32_t)cb * y_row, y_step);
   };
 
@@ -1003,12 +1026,12 @@ hipError_t launch_p2(const Problem &p, const View &a, const View &y, const View 
   const int galign = band_group(a, p.w);
   const dim3 grid(grid_size(p.B, nblk)), block(kThreads);
   // Tiles straight into LDS (N = 64 / 128, 16-byte column groups, 32-bit byte offsets inside a batch
-  // element of the band and of Y, chunks past the end included) where that was measured faster than
-  // the register-staged kernel: up to w = 128 (30 % at w = 36, 14 % at w = 64) and at N = 128 with
-  // whole-line groups (3-5 % at w = 512).  At N = 64 and w = 256 the two are equal, and once the band
-  // outgrows the last-level cache the staged kernel, with two chunks per workgroup in flight, is
-  // 7-9 % faster (B = 384 at w = 256, B = 32 at M = 32768 and w = 512).
-  if (lds_direct_ok(ALIGNED, p, y) && (p.w <= 128 || (p.N == 128 && galign == 64))) {
+  // element of the band and of Y, chunks past the end included).  Measured against the kernel below
+  // at B = 96, M = 4096, N = 64: 28 % faster at w = 36, 30 % at w = 100, 6-13 % at w = 256, 19 % at
+  // w = 260; 14 % at B = 32, M = 32768, w = 64; 4-7 % at config 4, 10 % at N = 128 and w = 260.  Once
+  // the band outgrows the last-level cache the kernel below, with two chunks per workgroup in flight,
+  // is 2-4 % faster at N = 64 (B = 384 at w = 256; B = 32, M = 32768 at w = 512): not worth a rule.
+  if (lds_direct_ok(ALIGNED, p, y)) {
     if (p.N == 64)
       hipLaunchKernelGGL((mfma_p2_dma_kernel<T, 4, 2>), grid, block, 0, p.stream, (const uint16_t *)a.data,
                          (const uint16_t *)y.data, (uint16_t *)c.data, (int)p.B, (int)p.M, (int)p.w, nblk, galign, a.sb,
@@ -1038,11 +1061,11 @@ hipError_t launch_p3(const Problem &p, const View &a, const View &y, const View 
   const int galign = band_group(a, p.w);
   const int nblk = (int)((p.M + (ALIGNED ? galign - 1 : 0) + TM - 1) / TM);
   const dim3 grid(grid_size(p.B, nblk)), block(kThreads);
-  // Tiles straight into LDS, as for the band-in product above; measured against the register-staged
-  // kernel: whole-line column groups 6-10 % faster at w = 256 and 512, 22 % at w = 64, equal to 2 %
-  // slower once the band outgrows the last-level cache; 16-byte groups 36 % faster at w = 36, 10 % at
-  // w = 100, 9 % slower at w = 260.
-  if (lds_direct_ok(ALIGNED, p, y) && (galign == 64 || p.w <= 128)) {
+  // Tiles straight into LDS, as for the band-in product above.  Measured against the kernel below at
+  // B = 96, M = 4096, N = 64: 35 % faster at w = 36, 30 % at w = 100, 12-15 % at w = 256 and 260;
+  // 23 % at B = 32, M = 32768, w = 64; 9-13 % at config 4; 4 % at B = 384, w = 256; equal at B = 32,
+  // M = 32768, w = 512.
+  if (lds_direct_ok(ALIGNED, p, y)) {
     if (p.N == 64)
       hipLaunchKernelGGL((mfma_p3_dma_kernel<T, 4, WM_P3_DMA_KC, WM_P3_DMA_STAGES>), grid, block, 0, p.stream,
                          (const uint16_t *)a.data, (const uint16_t *)y.data, (uint16_t *)c.data, (int)p.B, (int)p.M,

@@ -315,6 +315,12 @@ struct LdsTile {
   static __device__ __forceinline__ uint32_t lane_offset(int wave, int lane, int64_t row_stride_elems) {
     return dma_lane_offset<PPR>(wave, lane, row_stride_elems);
   }
+  // row of the tile that the lane's j-th load fills, and which 16 bytes of that row it fetches
+  static __device__ __forceinline__ int load_row(int wave, int lane, int j) { return (64 * wave + lane) / PPR + 256 / PPR * j; }
+  static __device__ __forceinline__ int load_piece(int wave, int lane) {
+    const int slot = 64 * wave + lane;
+    return (slot % PPR) ^ swz(slot / PPR);
+  }
   // bytes in memory between two of the wave's loads (256 / PPR rows)
   static __device__ __forceinline__ uint32_t step(int64_t row_stride_elems) {
     return (uint32_t)(256 / PPR * row_stride_elems * 2);
@@ -324,6 +330,16 @@ struct LdsTile {
     const uint32_t base = lds_address(tile) + 1024 * wave;
 #pragma unroll
     for (int j = 0; j < LOADS; ++j) dma_piece(rsrc, base + 4096 * j, voff, bytes0 + step_bytes * j);
+  }
+  // `request` for a tile of which a lane needs only some pieces: load j is made from voff[j], which
+  // the caller sets beyond the end of the buffer for pieces nobody will read (such a load returns
+  // zeros without touching memory)
+  static __device__ __forceinline__ void request_some(u32x4 rsrc, const uint16_t *tile, int wave,
+                                                      const uint32_t (&voff)[LOADS], uint32_t bytes0,
+                                                      uint32_t step_bytes) {
+    const uint32_t base = lds_address(tile) + 1024 * wave;
+#pragma unroll
+    for (int j = 0; j < LOADS; ++j) dma_piece(rsrc, base + 4096 * j, voff[j], bytes0 + step_bytes * j);
   }
   // Reading.  row_at: lane -> row lane % 32, piece lane / 32 (add 32 r0 ROWB for other rows, XOR
   // 32 ks for pieces 2 ks + lane / 32): operand with the contraction along the row.
