@@ -770,14 +770,14 @@ __global__ __launch_bounds__(kThreads, 3) void mfma_p1_dma_kernel(const uint16_t
 #define WM_P3_DMA_STAGES 2
 #endif
 template <typename T, int NK, int KCH, int STAGES>
-__global__ __launch_bounds__(kThreads, (160 * 1024 / (STAGES * KCH * (2 * TM + 32 * NK)) >= 3 ? 3 : 2)) void mfma_p3_dma_kernel(
+__global__ __launch_bounds__(kThreads, (160 * 1024 / (STAGES * KCH * (2 * TM + (NK <= 4 ? 128 : 256))) >= 3 ? 3 : 2)) void mfma_p3_dma_kernel(
     const uint16_t *__restrict__ A, const uint16_t *__restrict__ Y, uint16_t *__restrict__ C, int B, int M, int w,
     int nblk, int galign, int64_t asb, int64_t ysb, int64_t ysr, int64_t csb, int64_t csr) {
-  constexpr int N = 16 * NK, NT = NK / 2, CH = KCH, DEPTH = STAGES - 1;
-  using TT = LdsTile<CH, TM / 8>;      // [CH rows r][TM columns c]
-  using YT = LdsTile<CH, N / 8>;       // [CH rows r][N]
+  constexpr int N = 16 * NK, NT = (NK + 1) / 2, CH = KCH, DEPTH = STAGES - 1;
+  using TT = LdsTile<CH, TM / 8>;            // [CH rows r][TM columns c]
+  using YT = LdsTile<CH, NK <= 4 ? 8 : 16>;  // [CH rows r][64 or 128 columns, of which N are fetched]
   constexpr int LOADS = TT::LOADS + YT::LOADS;
-  static_assert(NK == 4 || NK == 8, "Y tile rows of 128 or 256 bytes");
+  static_assert(NK >= 1 && NK <= 8, "N = 16 ... 128");
   static_assert(CH % 16 == 0 && STAGES >= 2 && DEPTH * LOADS < 64, "vmcnt holds 6 bits");
   __shared__ __attribute__((aligned(1024))) uint16_t t_lds[STAGES][TT::ELEMS];
   __shared__ __attribute__((aligned(1024))) uint16_t y_lds[STAGES][YT::ELEMS];
@@ -802,7 +802,9 @@ __global__ __launch_bounds__(kThreads, (160 * 1024 / (STAGES * KCH * (2 * TM + 3
   const uint32_t t_voff = TT::lane_offset(wave, lane, 2 * w), t_step = TT::step(2 * w);
   const uint32_t t_col0 = (uint32_t)(a_rem + c0 + w) * 2, t_row = (uint32_t)(4 * w);  // bytes
   const u32x4 y_rsrc = make_rsrc(Y + (int64_t)b * ysb, (uint32_t)(((int64_t)(M - 1) * ysr + N) * 2));
-  const uint32_t y_voff = YT::lane_offset(wave, lane, ysr), y_step = YT::step(ysr), y_row = (uint32_t)(ysr * 2);
+  // (pieces of the Y tile beyond column N are requested out of range: zeros, no memory traffic)
+  const uint32_t y_voff = YT::load_piece(wave, lane) < N / 8 ? YT::lane_offset(wave, lane, ysr) : 0x80000000u;
+  const uint32_t y_step = YT::step(ysr), y_row = (uint32_t)(ysr * 2);
   // A piece of the band tile (8 columns from c8 of band row r) holds an entry of the band only if
   // c8 - r lies in [-w - 7, w]; the others are requested beyond the end of the buffer, which costs no
   // memory traffic (a quarter of the tile's pieces at w = 2 TM).  c8 - r falls by CH per chunk.
@@ -883,14 +885,14 @@ __global__ __launch_bounds__(kThreads, (160 * 1024 / (STAGES * KCH * (2 * TM + 3
 // begin before dense column 0: its position goes into the lanes' offsets, so that exactly the
 // pieces before the buffer read as zeros.
 template <typename T, int NK, int STAGES>
-__global__ __launch_bounds__(kThreads, (160 * 1024 / (STAGES * KC * (2 * TM + 32 * NK)) >= 3 ? 3 : 2)) void mfma_p2_dma_kernel(
+__global__ __launch_bounds__(kThreads, (160 * 1024 / (STAGES * KC * (2 * TM + (NK <= 4 ? 128 : 256))) >= 3 ? 3 : 2)) void mfma_p2_dma_kernel(
     const uint16_t *__restrict__ A, const uint16_t *__restrict__ Y, uint16_t *__restrict__ C, int B, int M, int w,
     int nblk, int galign, int64_t asb, int64_t ysb, int64_t ysr, int64_t csb, int64_t csr) {
-  constexpr int N = 16 * NK, NT = NK / 2, DEPTH = STAGES - 1;
-  using TT = LdsTile<TM, KC / 8>;  // [TM rows i][KC dense columns c]
-  using YT = LdsTile<KC, N / 8>;   // [KC rows c][N]
+  constexpr int N = 16 * NK, NT = (NK + 1) / 2, DEPTH = STAGES - 1;
+  using TT = LdsTile<TM, KC / 8>;            // [TM rows i][KC dense columns c]
+  using YT = LdsTile<KC, NK <= 4 ? 8 : 16>;  // [KC rows c][64 or 128 columns, of which N are fetched]
   constexpr int LOADS = TT::LOADS + YT::LOADS;
-  static_assert(NK == 4 || NK == 8, "Y tile rows of 128 or 256 bytes");
+  static_assert(NK >= 1 && NK <= 8, "N = 16 ... 128");
   static_assert(KC == 64 && STAGES >= 2 && DEPTH * LOADS < 64, "band tile rows of 128 bytes; vmcnt holds 6 bits");
   __shared__ __attribute__((aligned(1024))) uint16_t t_lds[STAGES][TT::ELEMS];
   __shared__ __attribute__((aligned(1024))) uint16_t y_lds[STAGES][YT::ELEMS];
@@ -914,6 +916,7 @@ __global__ __launch_bounds__(kThreads, (160 * 1024 / (STAGES * KC * (2 * TM + 32
   const uint32_t t_voff = TT::lane_offset(wave, lane, 2 * w) + (uint32_t)(a_rem + (int64_t)i0 * 2 * w + w) * 2;
   const uint32_t t_step = TT::step(2 * w);
   const u32x4 y_rsrc = make_rsrc(Y + (int64_t)b * ysb, (uint32_t)(((int64_t)(M - 1) * ysr + N) * 2));
+  const bool y_piece = YT::load_piece(wave, lane) < N / 8;  // else: beyond column N, requested out of range
   const uint32_t y_voff = YT::lane_offset(wave, lane, ysr), y_step = YT::step(ysr), y_row = (uint32_t)(ysr * 2);
   // pieces of the band tile that hold no entry of the band (8 columns from c8 of row i with c8 - i
   // outside [-w - 7, w]) are requested beyond the end of the buffer: no memory traffic for them
@@ -930,7 +933,7 @@ __global__ __launch_bounds__(kThreads, (160 * 1024 / (STAGES * KC * (2 * TM + 32
                     ? t_voff + (uint32_t)(2 * cb) + t_step * j
                     : 0x80000000u;
     TT::request_some(t_rsrc, t_lds[stage], wave, voff, 0, 0);
-    YT::request_at(y_rsrc, y_lds[stage], wave, y_voff + (uint32_t)cb * y_row, y_step);
+    YT::request_at(y_rsrc, y_lds[stage], wave, y_piece ? y_voff + (uint32_t)cb * y_row : 0x80000000u, y_piece ? y_step : 0u);
   };
 
   f32x16 acc[NT];
@@ -1009,10 +1012,15 @@ int band_group(const View &v, int64_t w) { return (w % 32 == 0 && ((uintptr_t)v.
 
 unsigned grid_size(int64_t B, int64_t nblk) { return (unsigned)(((B + 7) / 8) * 8 * nblk); }
 
-// Shapes the kernels that load their tiles straight into LDS accept (band-in products).
-bool lds_direct_ok(bool aligned, const Problem &p, const View &y) {
-  return aligned && !(p.flags & WM_FLAG_NO_LDS_DIRECT) && (p.N == 64 || p.N == 128) && y.sr > 0 &&
-         (p.M + 4 * KC) * (2 * p.w + 1) * 2 + 256 < 0x7fffffff && (p.M + 4 * KC) * y.sr * 2 < 0x7fffffff;
+// Shapes the kernels that load their tiles straight into LDS accept (band-in products): 32-bit byte
+// offsets inside a batch element of the band and of Y (chunks past the end included), and band rows
+// that can be cut into 16-byte pieces at 4-byte aligned addresses.  Returns the column-group
+// alignment to launch with (64, 8 or 2 elements), 0 if the shape is not accepted.
+template <bool ALIGNED>
+int lds_direct_group(const Problem &p, const View &a, const View &y) {
+  if ((p.flags & WM_FLAG_NO_LDS_DIRECT) || y.sr <= 0 || ((uintptr_t)a.data % 4) != 0) return 0;
+  if ((p.M + 4 * KC) * (2 * p.w + 1) * 2 + 256 >= 0x7fffffff || (p.M + 4 * KC) * y.sr * 2 >= 0x7fffffff) return 0;
+  return ALIGNED ? band_group(a, p.w) : 2;
 }
 
 // Chunk length of P2 (64: the result rows are staged in the band tile buffers, which 32 would make
@@ -1031,15 +1039,17 @@ hipError_t launch_p2(const Problem &p, const View &a, const View &y, const View 
   // w = 260; 14 % at B = 32, M = 32768, w = 64; 4-7 % at config 4, 10 % at N = 128 and w = 260.  Once
   // the band outgrows the last-level cache the kernel below, with two chunks per workgroup in flight,
   // is 2-4 % faster at N = 64 (B = 384 at w = 256; B = 32, M = 32768 at w = 512): not worth a rule.
-  if (lds_direct_ok(ALIGNED, p, y)) {
-    if (p.N == 64)
-      hipLaunchKernelGGL((mfma_p2_dma_kernel<T, 4, 2>), grid, block, 0, p.stream, (const uint16_t *)a.data,
-                         (const uint16_t *)y.data, (uint16_t *)c.data, (int)p.B, (int)p.M, (int)p.w, nblk, galign, a.sb,
-                         y.sb, y.sr, c.sb, c.sr);
-    else
-      hipLaunchKernelGGL((mfma_p2_dma_kernel<T, 8, 2>), grid, block, 0, p.stream, (const uint16_t *)a.data,
-                         (const uint16_t *)y.data, (uint16_t *)c.data, (int)p.B, (int)p.M, (int)p.w, nblk, galign, a.sb,
-                         y.sb, y.sr, c.sb, c.sr);
+  if (const int g = lds_direct_group<ALIGNED>(p, a, y)) {
+#define WM_P2_DMA(NK)                                                                                          \
+  case NK:                                                                                                     \
+    hipLaunchKernelGGL((mfma_p2_dma_kernel<T, NK, 2>), grid, block, 0, p.stream, (const uint16_t *)a.data,     \
+                       (const uint16_t *)y.data, (uint16_t *)c.data, (int)p.B, (int)p.M, (int)p.w, nblk, g,    \
+                       a.sb, y.sb, y.sr, c.sb, c.sr);                                                          \
+    break;
+    switch (p.N / 16) {
+      WM_P2_DMA(1) WM_P2_DMA(2) WM_P2_DMA(3) WM_P2_DMA(4) WM_P2_DMA(5) WM_P2_DMA(6) WM_P2_DMA(7) WM_P2_DMA(8)
+    }
+#undef WM_P2_DMA
     return hipGetLastError();
   }
 #define WM_P2(NT)                                                                                              \
@@ -1065,15 +1075,19 @@ hipError_t launch_p3(const Problem &p, const View &a, const View &y, const View 
   // B = 96, M = 4096, N = 64: 35 % faster at w = 36, 30 % at w = 100, 12-15 % at w = 256 and 260;
   // 23 % at B = 32, M = 32768, w = 64; 9-13 % at config 4; 4 % at B = 384, w = 256; equal at B = 32,
   // M = 32768, w = 512.
-  if (lds_direct_ok(ALIGNED, p, y)) {
-    if (p.N == 64)
-      hipLaunchKernelGGL((mfma_p3_dma_kernel<T, 4, WM_P3_DMA_KC, WM_P3_DMA_STAGES>), grid, block, 0, p.stream,
-                         (const uint16_t *)a.data, (const uint16_t *)y.data, (uint16_t *)c.data, (int)p.B, (int)p.M,
-                         (int)p.w, nblk, galign, a.sb, y.sb, y.sr, c.sb, c.sr);
-    else
-      hipLaunchKernelGGL((mfma_p3_dma_kernel<T, 8, WM_P3_DMA_KC, WM_P3_DMA_STAGES>), grid, block, 0, p.stream,
-                         (const uint16_t *)a.data, (const uint16_t *)y.data, (uint16_t *)c.data, (int)p.B, (int)p.M,
-                         (int)p.w, nblk, galign, a.sb, y.sb, y.sr, c.sb, c.sr);
+  if (const int g = lds_direct_group<ALIGNED>(p, a, y)) {
+    const dim3 grid_g(grid_size(p.B, (p.M + g - 1 + TM - 1) / TM));
+    const int nblk_g = (int)((p.M + g - 1 + TM - 1) / TM);
+#define WM_P3_DMA(NK)                                                                                          \
+  case NK:                                                                                                     \
+    hipLaunchKernelGGL((mfma_p3_dma_kernel<T, NK, WM_P3_DMA_KC, WM_P3_DMA_STAGES>), grid_g, block, 0, p.stream, \
+                       (const uint16_t *)a.data, (const uint16_t *)y.data, (uint16_t *)c.data, (int)p.B,       \
+                       (int)p.M, (int)p.w, nblk_g, g, a.sb, y.sb, y.sr, c.sb, c.sr);                           \
+    break;
+    switch (p.N / 16) {
+      WM_P3_DMA(1) WM_P3_DMA(2) WM_P3_DMA(3) WM_P3_DMA(4) WM_P3_DMA(5) WM_P3_DMA(6) WM_P3_DMA(7) WM_P3_DMA(8)
+    }
+#undef WM_P3_DMA
     return hipGetLastError();
   }
 #define WM_P3(NT)                                                                                              \
