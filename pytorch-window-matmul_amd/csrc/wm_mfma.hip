@@ -799,6 +799,8 @@ __global__ __launch_bounds__(kThreads, (160 * 1024 / (STAGES * KCH * (2 * TM + (
   // band: the buffer starts at the 128-byte line that holds the batch element's first entry and ends
   // with the batch element; tile row r, column c0 is at element a_rem + r 2w + c0 + w of it
   const u32x4 t_rsrc = make_rsrc(A + (a0 - a_rem), (uint32_t)(((int64_t)a_rem + (int64_t)M * W) * 2));
+  // whole-line column groups: the band is streamed (non-temporal), each line is fetched by one load
+  const bool lines = galign == 64;
   const uint32_t t_voff = TT::lane_offset(wave, lane, 2 * w), t_step = TT::step(2 * w);
   const uint32_t t_col0 = (uint32_t)(a_rem + c0 + w) * 2, t_row = (uint32_t)(4 * w);  // bytes
   const u32x4 y_rsrc = make_rsrc(Y + (int64_t)b * ysb, (uint32_t)(((int64_t)(M - 1) * ysr + N) * 2));
@@ -818,7 +820,7 @@ __global__ __launch_bounds__(kThreads, (160 * 1024 / (STAGES * KCH * (2 * TM + (
 #pragma unroll
     for (int j = 0; j < TT::LOADS; ++j)
       voff[j] = (uint32_t)(t_skew[j] - k * CH) <= (uint32_t)(2 * w + 7) ? t_voff : 0x80000000u;
-    TT::request_some(t_rsrc, t_lds[stage], wave, voff, t_col0 + rb * t_row, t_step);
+    TT::request_some(t_rsrc, t_lds[stage], wave, voff, t_col0 + rb * t_row, t_step, lines);
     YT::request(y_rsrc, y_lds[stage], wave, y_voff, rb * y_row, y_step);
   };
 
@@ -913,6 +915,7 @@ __global__ __launch_bounds__(kThreads, (160 * 1024 / (STAGES * KC * (2 * TM + (N
   // band: buffer from the 128-byte line that holds the batch element's first entry to the end of the
   // batch element; tile row i, dense column c is at element a_rem + i 2w + c + w of it
   const u32x4 t_rsrc = make_rsrc(A + (a0 - a_rem), (uint32_t)(((int64_t)a_rem + (int64_t)M * W) * 2));
+  const bool lines = galign == 64;  // whole-line column groups: the band is streamed (non-temporal)
   const uint32_t t_voff = TT::lane_offset(wave, lane, 2 * w) + (uint32_t)(a_rem + (int64_t)i0 * 2 * w + w) * 2;
   const uint32_t t_step = TT::step(2 * w);
   const u32x4 y_rsrc = make_rsrc(Y + (int64_t)b * ysb, (uint32_t)(((int64_t)(M - 1) * ysr + N) * 2));
@@ -932,7 +935,7 @@ __global__ __launch_bounds__(kThreads, (160 * 1024 / (STAGES * KC * (2 * TM + (N
       voff[j] = (uint32_t)(t_skew[j] + k * KC) <= (uint32_t)(2 * w + 7)
                     ? t_voff + (uint32_t)(2 * cb) + t_step * j
                     : 0x80000000u;
-    TT::request_some(t_rsrc, t_lds[stage], wave, voff, 0, 0);
+    TT::request_some(t_rsrc, t_lds[stage], wave, voff, 0, 0, lines);
     YT::request_at(y_rsrc, y_lds[stage], wave, y_piece ? y_voff + (uint32_t)cb * y_row : 0x80000000u, y_piece ? y_step : 0u);
   };
 

@@ -271,6 +271,15 @@ __device__ __forceinline__ void dma_piece(u32x4 rsrc, uint32_t lds_base, uint32_
                : "v"(voff), "s"(rsrc), "s"(soff), "s"(lds_base)
                : "memory");
 }
+// The same marked non-temporal, for data that is read exactly once and in whole cache lines (a band
+// whose column groups are lines): it should not push the rows that neighbouring workgroups share out
+// of the L2.  Not for pieces whose line-mates are fetched by another load: those would miss again.
+__device__ __forceinline__ void dma_piece_streaming(u32x4 rsrc, uint32_t lds_base, uint32_t voff, uint32_t soff) {
+  asm volatile("s_mov_b32 m0, %3\n\ts_nop 0\n\tbuffer_load_dwordx4 %0, %1, %2 offen nt lds"
+               :
+               : "v"(voff), "s"(rsrc), "s"(soff), "s"(lds_base)
+               : "memory");
+}
 // The same with 4 bytes per lane: 256 consecutive bytes of LDS per wave-level load.
 __device__ __forceinline__ void dma_dword(u32x4 rsrc, uint32_t lds_base, uint32_t voff, uint32_t soff) {
   asm volatile("s_mov_b32 m0, %3\n\ts_nop 0\n\tbuffer_load_dword %0, %1, %2 offen lds"
@@ -333,13 +342,19 @@ struct LdsTile {
   }
   // `request` for a tile of which a lane needs only some pieces: load j is made from voff[j], which
   // the caller sets beyond the end of the buffer for pieces nobody will read (such a load returns
-  // zeros without touching memory)
+  // zeros without touching memory).  `streaming` (uniform over the wavefront) marks the loads
+  // non-temporal.
   static __device__ __forceinline__ void request_some(u32x4 rsrc, const uint16_t *tile, int wave,
                                                       const uint32_t (&voff)[LOADS], uint32_t bytes0,
-                                                      uint32_t step_bytes) {
+                                                      uint32_t step_bytes, bool streaming) {
     const uint32_t base = lds_address(tile) + 1024 * wave;
+    if (streaming) {
 #pragma unroll
-    for (int j = 0; j < LOADS; ++j) dma_piece(rsrc, base + 4096 * j, voff[j], bytes0 + step_bytes * j);
+      for (int j = 0; j < LOADS; ++j) dma_piece_streaming(rsrc, base + 4096 * j, voff[j], bytes0 + step_bytes * j);
+    } else {
+#pragma unroll
+      for (int j = 0; j < LOADS; ++j) dma_piece(rsrc, base + 4096 * j, voff[j], bytes0 + step_bytes * j);
+    }
   }
   // Reading.  row_at: lane -> row lane % 32, piece lane / 32 (add 32 r0 ROWB for other rows, XOR
   // 32 ks for pieces 2 ks + lane / 32): operand with the contraction along the row.
