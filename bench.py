@@ -23,7 +23,7 @@ the count but its time is inside the step).  Next to it:
                  (N = 128, w = 512, float16) and the float32 band that covers the sequence.
 
 Usage: python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c2|c4|c5] [--no-cpu] [--no-others]
-       python bench.py --kernels-only [--shape B M N w] [--dtype bf16|fp16|fp32] [--family auto|wide|strided]
+       python bench.py --kernels-only [--shape B M N w] [--dtype bf16|fp16|fp32] [--family auto|wide|staged|strided]
 """
 import argparse
 import hashlib
@@ -282,9 +282,10 @@ def main():
                     help="time this shape instead of a named workload (forward + backward)")
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp16", "fp32"],
                     help="storage type for --shape")
-    ap.add_argument("--family", default="auto", choices=["auto", "wide", "strided"],
+    ap.add_argument("--family", default="auto", choices=["auto", "wide", "staged", "strided"],
                     help="kernel family for the per-kernel timings: the library's choice, the wide-band MFMA "
-                         "kernels even for a narrow band, or the strided kernels (A/B measurements)")
+                         "kernels even for a narrow band, the library's choice without the kernels that load "
+                         "their tiles straight into LDS, or the strided kernels (A/B measurements)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-others", action="store_true", help="skip the per-kernel timings at the other configurations")
     ap.add_argument("--kernels-only", action="store_true",
@@ -308,7 +309,7 @@ def main():
         cfg = dict(B=sb, M=sm, N=sn, w=sw, dtype=args.dtype, qk_scale=sn ** -0.25, backward=True,
                    label=f"B{sb} M{sm} N{sn} w{sw} {args.dtype}, window->softmax->unwindow, fwd+bwd")
         args.workload = "custom"
-    fam = {"auto": 0, "wide": abi.NO_NARROW_BAND, "strided": abi.FORCE_STRIDED}[args.family]
+    fam = {"auto": 0, "wide": abi.NO_NARROW_BAND, "staged": abi.NO_LDS_DIRECT, "strided": abi.FORCE_STRIDED}[args.family]
     iters = max(args.steps, 10)
     bench = Bench(cfg, fam)
     B, M, N, w = bench.B, bench.M, bench.N, bench.w

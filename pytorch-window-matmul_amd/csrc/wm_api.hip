@@ -239,7 +239,7 @@ const char *wm_kernel_choice(int op, int64_t B, int64_t M, int64_t N, int64_t w,
       static const char *names[] = {"vector_p1", "vector_p2", "vector_p3"};
       return names[op - 1];
     }
-    if (!(flags & WM_FLAG_NO_NARROW_BAND) && small_supports(op, M, N, w, dtype)) {
+    if (!(flags & WM_FLAG_NO_NARROW_BAND) && small_supports(op, M, N, w, dtype, flags)) {
       static const char *names[] = {"narrow_p1", "narrow_p2", "narrow_p3"};
       return names[op - 1];
     }

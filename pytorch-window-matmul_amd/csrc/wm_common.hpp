@@ -48,7 +48,7 @@ bool try_launch_mfma_p3(const Problem &p, const View &a, const View &y, const Vi
 bool try_launch_small_p1(const Problem &p, const View &x, const View &y, const View &c, hipError_t *err);
 bool try_launch_small_p2(const Problem &p, const View &a, const View &y, const View &c, hipError_t *err);
 bool try_launch_small_p3(const Problem &p, const View &a, const View &y, const View &c, hipError_t *err);
-bool small_supports(int op, int64_t M, int64_t N, int64_t w, int dtype);
+bool small_supports(int op, int64_t M, int64_t N, int64_t w, int dtype, unsigned flags);
 bool small_f32_in_supports(int64_t M, int64_t N, int64_t w);  // float32 band-in kernels of the narrow-band family
 bool small_f32_p1_supports(int64_t M, int64_t N, int64_t w);  // float32 band-out kernel of the narrow-band family
 // Vector-ALU kernels for the narrowest windows: 16-bit up to w = 3 (band-in) and w = 2 (band-out),

@@ -920,10 +920,26 @@ bool small_f32_in_supports(int64_t M, int64_t N, int64_t w) {
          (64 + 2 * w) * (2 * w + 1) + 6 <= 8 * 4 * 256 && small_in_f32_lds(w, N) <= kSmallLdsLimit;
 }
 
-bool small_supports(int op, int64_t M, int64_t N, int64_t w, int dtype) {
+// Windows at which the wide-band band-in kernels that load their tiles straight into LDS were
+// measured faster than the kernels of this file (16-bit tensors of 100 M elements at M = 16384, both
+// directions of each product; e.g. N = 64, w = 24: 110-128 us against 131-150 us; N = 48, w = 28,
+// P3: 143-151 against 172-184; N = 128, w = 12: 88-92 against 101-107).
+bool wide_band_in_is_faster(int op, int64_t N, int64_t w) {
+  switch (N) {
+    case 32: return op == 3 && w >= 28;
+    case 48: return op == 3 ? w >= 24 : w >= 28;
+    case 64: return op == 3 ? w >= 13 : w >= 16;
+    case 112: return op == 3 ? w >= 12 : (w >= 16 && w <= 24);
+    case 128: return w >= 12 && w <= 16;
+    default: return false;
+  }
+}
+
+bool small_supports(int op, int64_t M, int64_t N, int64_t w, int dtype, unsigned flags) {
   if (dtype == WM_DTYPE_F32) return op == 1 ? small_f32_p1_supports(M, N, w) : small_f32_in_supports(M, N, w);
   if (op == 1) return small_p1_shape_ok(M, N, w, dtype);
   if (!small_shape_ok(M, N, w, dtype)) return false;
+  if (!(flags & WM_FLAG_NO_LDS_DIRECT) && w >= 8 && wide_band_in_is_faster(op, N, w)) return false;
   if (op == 2) {
     // the two LDS images must fit the default 64 KB dynamic limit; wider cases go to the wide-band family
     const int64_t NT = (N + 31) / 32;
@@ -940,7 +956,7 @@ bool small_supports(int op, int64_t M, int64_t N, int64_t w, int dtype) {
 }
 
 bool try_launch_small_p1(const Problem &p, const View &x, const View &y, const View &c, hipError_t *err) {
-  if (!small_supports(1, p.M, p.N, p.w, p.dtype)) return false;
+  if (!small_supports(1, p.M, p.N, p.w, p.dtype, p.flags)) return false;
   if (!fast_layout(x, p.dtype) || !fast_layout(y, p.dtype) || !band_contiguous(c, 2 * p.w + 1)) return false;
   if (p.dtype == WM_DTYPE_F32) {
     *err = launch_small_p1_f32(p, x, y, c);
@@ -951,7 +967,7 @@ bool try_launch_small_p1(const Problem &p, const View &x, const View &y, const V
 }
 
 bool try_launch_small_p2(const Problem &p, const View &a, const View &y, const View &c, hipError_t *err) {
-  if (!small_supports(2, p.M, p.N, p.w, p.dtype)) return false;
+  if (!small_supports(2, p.M, p.N, p.w, p.dtype, p.flags)) return false;
   if (!band_contiguous(a, 2 * p.w + 1) || !fast_layout(y, p.dtype) || !fast_layout(c, p.dtype)) return false;
   if (p.dtype == WM_DTYPE_F32) {
     *err = launch_small_in_f32<false>(p, a, y, c);
@@ -962,7 +978,7 @@ bool try_launch_small_p2(const Problem &p, const View &a, const View &y, const V
 }
 
 bool try_launch_small_p3(const Problem &p, const View &a, const View &y, const View &c, hipError_t *err) {
-  if (!small_supports(3, p.M, p.N, p.w, p.dtype)) return false;
+  if (!small_supports(3, p.M, p.N, p.w, p.dtype, p.flags)) return false;
   if (!band_contiguous(a, 2 * p.w + 1) || !fast_layout(y, p.dtype) || !fast_layout(c, p.dtype)) return false;
   if (p.dtype == WM_DTYPE_F32) {
     *err = launch_small_in_f32<true>(p, a, y, c);

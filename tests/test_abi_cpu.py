@@ -60,10 +60,18 @@ def test_kernel_choice_names():
     assert L.wm_kernel_choice(2, 96, 16384, 64, 13, 2, 1, 0) == b"narrow_p2"
     assert L.wm_kernel_choice(3, 96, 16384, 64, 8, 2, 1, 0) == b"narrow_p3"
     assert L.wm_kernel_choice(3, 96, 16384, 64, 10, 2, 1, 0) == b"narrow_p3"
-    assert L.wm_kernel_choice(3, 96, 16384, 64, 27, 2, 1, 0) == b"narrow_p3"
-    assert L.wm_kernel_choice(3, 96, 16384, 64, 30, 2, 1, 0) == b"mfma_p3"     # two workgroups per CU: slower
-    assert L.wm_kernel_choice(2, 96, 16384, 64, 30, 2, 1, 0) == b"narrow_p2"
-    assert L.wm_kernel_choice(2, 96, 16384, 64, 32, 2, 1, 0) == b"narrow_p2"  # 32 rows per wave still fit LDS
+    # from w = 16 (band-in) / 13 (transposed band-in) at N = 64 the wide-band kernels that load their
+    # tiles straight into LDS are faster; without them the narrow kernels keep their old range
+    assert L.wm_kernel_choice(2, 96, 16384, 64, 15, 2, 1, 0) == b"narrow_p2"
+    assert L.wm_kernel_choice(2, 96, 16384, 64, 16, 2, 1, 0) == b"mfma_p2"
+    assert L.wm_kernel_choice(3, 96, 16384, 64, 13, 2, 1, 0) == b"mfma_p3"
+    assert L.wm_kernel_choice(3, 96, 16384, 64, 27, 2, 1, 0) == b"mfma_p3"
+    assert L.wm_kernel_choice(3, 96, 16384, 64, 27, 2, 1, abi.NO_LDS_DIRECT) == b"narrow_p3"
+    assert L.wm_kernel_choice(3, 96, 16384, 64, 30, 2, 1, abi.NO_LDS_DIRECT) == b"mfma_p3"  # two workgroups per CU: slower
+    assert L.wm_kernel_choice(2, 96, 16384, 64, 32, 2, 1, abi.NO_LDS_DIRECT) == b"narrow_p2"  # 32 rows per wave still fit LDS
+    assert L.wm_kernel_choice(2, 96, 16384, 32, 32, 2, 1, 0) == b"narrow_p2"
+    assert L.wm_kernel_choice(3, 96, 16384, 32, 28, 2, 1, 0) == b"mfma_p3"
+    assert L.wm_kernel_choice(2, 96, 16384, 128, 12, 1, 1, 0) == b"mfma_p2"
     assert L.wm_kernel_choice(3, 96, 16384, 128, 32, 2, 1, 0) == b"mfma_p3"   # images beyond 64 KB of LDS
     assert L.wm_kernel_choice(1, 96, 16384, 64, 8, 2, 1, abi.NO_NARROW_BAND) == b"mfma_p1"
     # the band-out kernel of the narrow family reaches w = 63 while the operands fit the registers (N <= 64)
