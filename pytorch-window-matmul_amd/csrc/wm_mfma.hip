@@ -326,15 +326,26 @@ __global__ __launch_bounds__(kThreads, NT <= 2 ? 3 : 2) void mfma_p3_kernel(cons
 // ------------------------------------------------------------------------------------------
 // P1: band[b,i,c-i+w] = sum_h X[b,i,h] * Y[b,c,h]   (+0.0 where c is outside the sequence)
 // ------------------------------------------------------------------------------------------
-template <typename T, int NK, bool ALIGNED>  // NK = N / 16
-__global__ __launch_bounds__(kThreads, 2) void mfma_p1_kernel(const uint16_t *__restrict__ X,
+// RING (16-byte column groups that are not whole lines, w % 4 == 0 but w % 32 != 0): row i's 128-byte
+// lines begin at a column offset of its own, so a chunk of 64 columns on a common grid would leave
+// every row as two partial lines, completed a chunk apart, which neither plain nor non-temporal
+// stores do well (200 and 250 us against 85 us for the whole-line case at B96 M4096 N64, w = 260
+// against 256).  Here the staging area of a wavefront keeps the last two chunks (a ring of 128
+// columns per row), and after every chunk each row stores the one line of its own grid that has
+// just been completed: whole lines for every row, one chunk step late at most, plus one closing
+// step for the lines that end after the last chunk.
+template <typename T, int NK, bool ALIGNED, bool RING = false>  // NK = N / 16
+__global__ __launch_bounds__(kThreads, RING && NK <= 4 ? 3 : 2) void mfma_p1_kernel(const uint16_t *__restrict__ X,
                                                               const uint16_t *__restrict__ Y,
                                                               uint16_t *__restrict__ C, int B, int M, int w,
                                                               int nblk, int galign, int64_t xsb, int64_t xsr,
                                                               int64_t ysb, int64_t ysr, int64_t csb) {
   constexpr int N = 16 * NK;
   constexpr int SY = N + 8;   // Y chunk rows: 16 (mod 128) bytes apart in banks -> conflict-free b128 reads
-  constexpr int SS = KC + 8;  // per-wave staging rows
+  // per-wave staging rows: one chunk, padded; or a ring of two chunks, unpadded, the 16-byte piece p
+  // of row r at position p ^ (r % 16)
+  constexpr int SS = RING ? 2 * KC : KC + 8;
+  static_assert(!RING || ALIGNED, "the ring reads 16-byte pieces at line offsets that are multiples of 16 bytes");
   constexpr int YS = (KC * N / 8 + kThreads - 1) / kThreads;
   __shared__ __attribute__((aligned(16))) uint16_t y_lds[2][(KC + 1) * SY];  // row KC: sink for idle loader slots
   __shared__ __attribute__((aligned(16))) uint16_t s_lds[4][32 * SS];
@@ -358,7 +369,9 @@ __global__ __launch_bounds__(kThreads, 2) void mfma_p1_kernel(const uint16_t *__
   // Head and tail pieces of neighbouring rows meet through the seam buffer when both rows belong
   // to this wave, or to any wave of the workgroup if a workgroup barrier is certain to separate
   // the two tiles (the tail is produced 2w-1 columns after the head: at least two chunks later).
-  const bool seam_across_waves = ALIGNED && (2 * w - 1 >= 2 * KC);
+  // (ring: a row's tail line is stored (2w + d' - d) / 64 steps after the head line of the row below,
+  // d, d' < 64 the rows' line offsets in multiples of 8: at least one step from 2w - 56 >= 64 on)
+  const bool seam_across_waves = ALIGNED && (RING ? 2 * w - 56 >= KC : 2 * w - 1 >= 2 * KC);
 
   // B-operand: this wave's 32 rows of X, all of N, kept in registers
   u32x4 xop[NK];
@@ -408,7 +421,8 @@ __global__ __launch_bounds__(kThreads, 2) void mfma_p1_kernel(const uint16_t *__
   const int iw_first = i0 + wave * 32;
   int st_lo[4], st_hi[4];   // chunk-relative valid element range is [st_lo - cb, st_hi - cb]
   uint16_t *st_dst[4];      // address of dense column 8 g of the row (add cb)
-  const uint16_t *st_src[4];
+  const uint16_t *st_src[4];  // (ring: the row's staging area)
+  int st_shift[4], st_piece[4];  // ring: the row's lines begin at columns c_start + st_shift (mod 64); first piece of a line
 #pragma unroll
   for (int s = 0; s < 4; ++s) {
     const int r = (lane >> 3) + 8 * s, g = lane & 7;
@@ -416,10 +430,82 @@ __global__ __launch_bounds__(kThreads, 2) void mfma_p1_kernel(const uint16_t *__
     st_lo[s] = i - w - 8 * g;
     st_hi[s] = i < M ? i + w - 8 * g : -0x40000000;
     st_dst[s] = Cb + (int64_t)i * W + (w - i) + 8 * g;
-    st_src[s] = stage + r * SS + 8 * g;
+    st_src[s] = RING ? stage + r * SS : stage + r * SS + 8 * g;
+    // element address of (i, c_start) modulo a line: the line that contains it begins that many columns earlier
+    st_shift[s] = RING ? (int)((0 - (reinterpret_cast<uintptr_t>(Cb + (int64_t)i * W + (w - i) + c_start) >> 1)) & 63) : 0;
+    st_piece[s] = (st_shift[s] >> 3) + g;
   }
   uint16_t *stage_wr = stage + (lane & 31) * SS + 4 * (lane >> 5);
   const int y_rd_off = (lane & 31) * SY + 8 * (lane >> 5);
+
+  // The stores that follow chunk k (k = nk: the closing step of the ring).  Row-contiguous: 8 lanes
+  // cover 64 dense columns of one row, the chunk's own or, with the ring, the row's line that chunk k
+  // completed: columns cb + shift - 64 ... cb + shift - 1, which begin in the half of the ring that
+  // chunk k - 1 filled.
+  auto store_lines = [&](int k) __attribute__((always_inline)) {
+    const int cb = c_start + k * KC;
+    auto cb_of = [&](int s) { return RING ? cb + st_shift[s] - KC : cb; };
+    auto src_of = [&](int s) {
+      const int r = (lane >> 3) + 8 * s;
+      return RING ? st_src[s] + ((((st_piece[s] + 8 * ((k + 1) & 1)) & 15) ^ (r & 15)) << 3) : st_src[s];
+    };
+    if (cb - (RING ? KC : 0) >= iw_first + 31 - w && cb + KC - 1 - (RING ? 8 : 0) <= iw_first + w && iw_first + 31 < M) {
+      // every chunk of the wave's tile lies inside the band: nothing to decide, and each group of 8
+      // lanes writes one whole 128-byte line, which is what makes the streaming store pay
+#pragma unroll
+      for (int s = 0; s < 4; ++s) {
+        const u32x4 val = *reinterpret_cast<const u32x4 *>(src_of(s));
+        if (ALIGNED && (RING || galign == 64))
+          store_chunk_streaming(st_dst[s] + cb_of(s), val);
+        else
+          store_chunk<ALIGNED>(st_dst[s] + cb_of(s), val);  // (pieces of two lines: plain, see store_chunk_streaming)
+      }
+      wave_sync_lds();
+    } else {
+      // pass A: whole chunks go out; head pieces are parked in the seam buffer.
+      u32x4 v[4];
+      int tail_hi[4];  // >= 0: this slot holds a tail piece with elements 0..tail_hi, handled in pass B
+#pragma unroll
+      for (int s = 0; s < 4; ++s) {
+        const int rw = wave * 32 + (lane >> 3) + 8 * s, r = rw & 31;
+        const int e_lo = st_lo[s] - cb_of(s), e_hi = st_hi[s] - cb_of(s);
+        tail_hi[s] = -1;
+        if (e_hi >= 0 && e_lo <= 7) {
+          v[s] = *reinterpret_cast<const u32x4 *>(src_of(s));
+          uint16_t *dst = st_dst[s] + cb_of(s);
+          if (e_lo <= 0 && e_hi >= 7) {
+            store_chunk<ALIGNED>(dst, v[s]);  // (plain: lines of edge tiles are completed piecewise)
+          } else if (e_lo > 0) {  // head piece: elements e_lo..7 (W >= 17, so it reaches the chunk's end)
+            if (ALIGNED && rw > 0 && (r > 0 || seam_across_waves))
+              *reinterpret_cast<u32x4 *>(&seam[rw * 8]) = v[s];
+            else
+              store_chunk_elements(dst, v[s], e_lo, 7);
+          } else {
+            tail_hi[s] = e_hi;
+          }
+        }
+      }
+      wave_sync_lds();
+      // pass B: tail pieces pick up the head piece of the row below and leave as whole chunks.
+#pragma unroll
+      for (int s = 0; s < 4; ++s) {
+        if (tail_hi[s] >= 0) {
+          const int rw = wave * 32 + (lane >> 3) + 8 * s, r = rw & 31;
+          uint16_t *dst = st_dst[s] + cb_of(s);
+          if (ALIGNED && rw + 1 < TM && i0 + rw + 1 < M && (r < 31 || seam_across_waves)) {
+            const u32x4 head = *reinterpret_cast<const u32x4 *>(&seam[(rw + 1) * 8]);
+            const u32x4 mine_part = keep_range(v[s], 0, tail_hi[s]);
+            const u32x4 head_part = keep_range(head, tail_hi[s] + 1, 7);
+            u32x4 merged = {mine_part[0] | head_part[0], mine_part[1] | head_part[1], mine_part[2] | head_part[2],
+                            mine_part[3] | head_part[3]};
+            store_chunk<true>(dst, merged);
+          } else {
+            store_chunk_elements(dst, v[s], 0, tail_hi[s]);
+          }
+        }
+      }
+    }
+  };
 
   // One slot: request Y chunk k+PF, multiply chunk k, stage the 32 x 64 result, store it, then move
   // chunk k+1 into LDS.  The stores are issued before the wait for chunk k+1, which was requested
@@ -454,7 +540,10 @@ __global__ __launch_bounds__(kThreads, 2) void mfma_p1_kernel(const uint16_t *__
             if (c + 3 < 0 || c + 3 >= M) hi &= 0x0000ffffu;
           }
           u32x2 o = {lo, hi};
-          *reinterpret_cast<u32x2 *>(stage_wr + 32 * mt + 8 * q4) = o;
+          if (RING)
+            *reinterpret_cast<u32x2 *>(stage_wr + (((8 * buf + 4 * mt + q4) ^ (lane & 15)) << 3)) = o;
+          else
+            *reinterpret_cast<u32x2 *>(stage_wr + 32 * mt + 8 * q4) = o;
         }
       }
     };
@@ -463,63 +552,7 @@ __global__ __launch_bounds__(kThreads, 2) void mfma_p1_kernel(const uint16_t *__
     else
       multiply_and_stage(std::false_type{});
     wave_sync_lds();
-    // Row-contiguous stores: 8 lanes cover the 64 dense columns of one row.
-    if (cb >= iw_first + 31 - w && cb + KC - 1 <= iw_first + w && iw_first + 31 < M) {
-      // every chunk of the wave's tile lies inside the band: nothing to decide, and each group of 8
-      // lanes writes one whole 128-byte line, which is what makes the streaming store pay
-#pragma unroll
-      for (int s = 0; s < 4; ++s) {
-        const u32x4 val = *reinterpret_cast<const u32x4 *>(st_src[s]);
-        if (ALIGNED)
-          store_chunk_streaming(st_dst[s] + cb, val);
-        else
-          store_chunk<false>(st_dst[s] + cb, val);
-      }
-      wave_sync_lds();
-    } else {
-      // pass A: whole chunks go out; head pieces are parked in the seam buffer.
-      u32x4 v[4];
-      int tail_hi[4];  // >= 0: this slot holds a tail piece with elements 0..tail_hi, handled in pass B
-#pragma unroll
-      for (int s = 0; s < 4; ++s) {
-        const int rw = wave * 32 + (lane >> 3) + 8 * s, r = rw & 31;
-        const int e_lo = st_lo[s] - cb, e_hi = st_hi[s] - cb;
-        tail_hi[s] = -1;
-        if (e_hi >= 0 && e_lo <= 7) {
-          v[s] = *reinterpret_cast<const u32x4 *>(st_src[s]);
-          uint16_t *dst = st_dst[s] + cb;
-          if (e_lo <= 0 && e_hi >= 7) {
-            store_chunk<ALIGNED>(dst, v[s]);  // (plain: lines of edge tiles are completed piecewise)
-          } else if (e_lo > 0) {  // head piece: elements e_lo..7 (W >= 17, so it reaches the chunk's end)
-            if (ALIGNED && rw > 0 && (r > 0 || seam_across_waves))
-              *reinterpret_cast<u32x4 *>(&seam[rw * 8]) = v[s];
-            else
-              store_chunk_elements(dst, v[s], e_lo, 7);
-          } else {
-            tail_hi[s] = e_hi;
-          }
-        }
-      }
-      wave_sync_lds();
-      // pass B: tail pieces pick up the head piece of the row below and leave as whole chunks.
-#pragma unroll
-      for (int s = 0; s < 4; ++s) {
-        if (tail_hi[s] >= 0) {
-          const int rw = wave * 32 + (lane >> 3) + 8 * s, r = rw & 31;
-          uint16_t *dst = st_dst[s] + cb;
-          if (ALIGNED && rw + 1 < TM && i0 + rw + 1 < M && (r < 31 || seam_across_waves)) {
-            const u32x4 head = *reinterpret_cast<const u32x4 *>(&seam[(rw + 1) * 8]);
-            const u32x4 mine_part = keep_range(v[s], 0, tail_hi[s]);
-            const u32x4 head_part = keep_range(head, tail_hi[s] + 1, 7);
-            u32x4 merged = {mine_part[0] | head_part[0], mine_part[1] | head_part[1], mine_part[2] | head_part[2],
-                            mine_part[3] | head_part[3]};
-            store_chunk<true>(dst, merged);
-          } else {
-            store_chunk_elements(dst, v[s], 0, tail_hi[s]);
-          }
-        }
-      }
-    }
+    store_lines(k);
     __builtin_amdgcn_sched_barrier(0);
     stash(k + 1, next);
     __syncthreads();
@@ -537,6 +570,7 @@ __global__ __launch_bounds__(kThreads, 2) void mfma_p1_kernel(const uint16_t *__
     slot(k + 1, y_reg[1], y_reg[0]);
   }
   if (k < nk) slot(k, y_reg[0], y_reg[1]);
+  if (RING) store_lines(nk);  // every wavefront is past the last barrier; lines that end after the last chunk
 }
 
 // ------------------------------------------------------------------------------------------
@@ -678,10 +712,10 @@ __global__ __launch_bounds__(kThreads, 3) void mfma_p1_dma_kernel(const uint16_t
 #pragma unroll
       for (int s = 0; s < 4; ++s) {
         const u32x4 val = *reinterpret_cast<const u32x4 *>(st_src[s]);
-        if (ALIGNED)
+        if (ALIGNED && galign == 64)
           store_chunk_streaming(st_dst[s] + cb, val);
         else
-          store_chunk<false>(st_dst[s] + cb, val);
+          store_chunk<ALIGNED>(st_dst[s] + cb, val);  // (pieces of two lines: plain, see store_chunk_streaming)
       }
       wave_sync_lds();
       four_stores = true;
@@ -1112,10 +1146,20 @@ hipError_t launch_p1(const Problem &p, const View &x, const View &y, const View 
   const int nblk = (int)((p.M + TM - 1) / TM);
   const int galign = band_group(c, p.w);
   const dim3 grid(grid_size(p.B, nblk)), block(kThreads);
+  // 16-byte column groups: every row is stored as two partial lines per chunk.  While the band fits
+  // the last-level cache (256 MB) the halves meet there and plain stores do (B96 M4096 N64 w = 100,
+  // 158 MB: 62 us, against 67 us with the ring of whole lines); beyond it the ring wins: 91 against
+  // 116 us at w = 164 (259 MB), 119 against 200 us at w = 260, 327 against 747 us at w = 1028.
+  const bool ring_pays = p.B * p.M * (2 * p.w + 1) * 2 >= (int64_t)220 << 20;
 #define WM_P1(NK)                                                                                            \
-  hipLaunchKernelGGL((mfma_p1_kernel<T, NK, ALIGNED>), grid, block, 0, p.stream, (const uint16_t *)x.data,   \
-                     (const uint16_t *)y.data, (uint16_t *)c.data, (int)p.B, (int)p.M, (int)p.w, nblk, galign, \
-                     x.sb, x.sr, y.sb, y.sr, c.sb)
+  if (ALIGNED && galign != 64 && ring_pays)                                                                  \
+    hipLaunchKernelGGL((mfma_p1_kernel<T, NK, ALIGNED, ALIGNED>), grid, block, 0, p.stream,                  \
+                       (const uint16_t *)x.data, (const uint16_t *)y.data, (uint16_t *)c.data, (int)p.B,     \
+                       (int)p.M, (int)p.w, nblk, galign, x.sb, x.sr, y.sb, y.sr, c.sb);                      \
+  else                                                                                                       \
+    hipLaunchKernelGGL((mfma_p1_kernel<T, NK, ALIGNED, false>), grid, block, 0, p.stream,                    \
+                       (const uint16_t *)x.data, (const uint16_t *)y.data, (uint16_t *)c.data, (int)p.B,     \
+                       (int)p.M, (int)p.w, nblk, galign, x.sb, x.sr, y.sb, y.sr, c.sb)
   // N = 128 with whole-line band stores: Y chunks straight into LDS, three workgroups per CU (32-bit
   // byte offsets inside a batch element).  With 16-byte column groups most slots take the piecewise
   // store path, whose stores this kernel waits for: 10 % slower there than the kernel above.

@@ -98,3 +98,41 @@ def test_kernel_choice_is_unchanged_by_the_switch(device):
     for op in (1, 2, 3):
         for flags in (0, abi.NO_LDS_DIRECT):
             assert abi.lib().wm_kernel_choice(op, 8, 4096, 128, 64, abi.DTYPES[torch.bfloat16], 1, flags).decode() == f"mfma_p{op}"
+
+
+@pytest.mark.parametrize("B,M,N,w,dtype", [(26, 4099, 64, 580, torch.bfloat16), (7, 16390, 128, 516, torch.float16),
+                                           (44, 8200, 32, 172, torch.bfloat16)],
+                         ids=["N64-w580", "N128-w516", "N32-w172"])
+def test_band_out_ring_of_lines(device, B, M, N, w, dtype):
+    """A band beyond 220 MB whose column groups are 16-byte pieces but not whole lines (w % 4 == 0,
+    w % 32 != 0) is written through a ring of two chunks per row, every row in whole lines of its own
+    grid.  Every band entry is one dot product in a fixed order, so the result must equal, bit for
+    bit, that of the kernel for unaligned bands (WM_FLAG_NO_ALIGNED_BAND: 16-byte stores on a common
+    column grid), entries outside the sequence must be +0.0, and rows picked across the tensor must
+    match the CPU oracle.  The band lives at three different offsets inside a poisoned buffer: nothing
+    outside it may be written."""
+    print(f"case B{B} M{M} N{N} w{w}", flush=True)
+    W = 2 * w + 1
+    assert B * M * W * 2 >= 220 << 20 and w % 4 == 0 and w % 32 != 0
+    q, k = (seeded((B, M, N), 340 + s, dtype).to(device) for s in range(2))
+    kt = k.transpose(1, 2)
+    want = abi.window_forward(q, kt, w, abi.NO_ALIGNED_BAND)
+    store = torch.empty(B * M * W + 128, dtype=dtype, device=device)
+    for off in (0, 8, 40):
+        store.fill_(float("nan"))
+        band = store[off:off + B * M * W].view(B, M, W)
+        got = abi.window_forward(q, kt, w, 0, out=band)
+        assert torch.equal(bits(got), bits(want)), f"offset {off}"
+        assert bool(torch.isnan(store[:off]).all()) and bool(torch.isnan(store[off + B * M * W:]).all()), f"offset {off}: wrote outside the band"
+    outside = ~oracle.band_mask(M, w, device)
+    assert not bits(want)[:, outside].any(), "band entries outside the sequence are not +0.0"
+    # rows at the ends and in the middle of a few batch elements against the oracle (float32 of the rounded inputs)
+    for b in (0, B - 1):
+        for i0 in (0, M // 2 - 3, M - 40):
+            rows = slice(i0, i0 + 40)
+            lo, hi = max(i0 - w, 0), min(i0 + 40 + w, M)
+            qs = torch.zeros(1, hi - lo, N)
+            qs[0, i0 - lo:i0 - lo + 40] = q[b, rows].float().cpu()
+            ks = k[b, lo:hi].float().cpu().unsqueeze(0)
+            ref = oracle.window_matmul_forward(qs, ks.transpose(1, 2).contiguous(), w)[0, i0 - lo:i0 - lo + 40]
+            torch.testing.assert_close(want[b, rows].float().cpu(), ref, **TOL)
