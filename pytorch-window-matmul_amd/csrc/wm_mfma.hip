@@ -333,8 +333,10 @@ __global__ __launch_bounds__(kThreads, NT <= 2 ? 3 : 2) void mfma_p3_kernel(cons
 // against 256).  Here the staging area of a wavefront keeps the last two chunks (a ring of 128
 // columns per row), and after every chunk each row stores the one line of its own grid that has
 // just been completed: whole lines for every row, one chunk step late at most, plus one closing
-// step for the lines that end after the last chunk.
-template <typename T, int NK, bool ALIGNED, bool RING = false>  // NK = N / 16
+// step for the lines that end after the last chunk.  RING = 2 is the same for windows that are not a
+// multiple of 4: the rows' lines then begin at any even column offset, a 16-byte piece of a line is
+// no longer one piece of the ring, and the staging area is read in 4-byte units.
+template <typename T, int NK, bool ALIGNED, int RING = 0>  // NK = N / 16
 __global__ __launch_bounds__(kThreads, RING && NK <= 4 ? 3 : 2) void mfma_p1_kernel(const uint16_t *__restrict__ X,
                                                               const uint16_t *__restrict__ Y,
                                                               uint16_t *__restrict__ C, int B, int M, int w,
@@ -345,7 +347,8 @@ __global__ __launch_bounds__(kThreads, RING && NK <= 4 ? 3 : 2) void mfma_p1_ker
   // per-wave staging rows: one chunk, padded; or a ring of two chunks, unpadded, the 16-byte piece p
   // of row r at position p ^ (r % 16)
   constexpr int SS = RING ? 2 * KC : KC + 8;
-  static_assert(!RING || ALIGNED, "the ring reads 16-byte pieces at line offsets that are multiples of 16 bytes");
+  static_assert(!RING || ALIGNED, "the ring stores pieces that are 16-byte aligned in memory, with the seam logic");
+  constexpr int kMaxShift = RING == 2 ? 62 : 56;  // largest column offset of a row's lines
   constexpr int YS = (KC * N / 8 + kThreads - 1) / kThreads;
   __shared__ __attribute__((aligned(16))) uint16_t y_lds[2][(KC + 1) * SY];  // row KC: sink for idle loader slots
   __shared__ __attribute__((aligned(16))) uint16_t s_lds[4][32 * SS];
@@ -370,8 +373,8 @@ __global__ __launch_bounds__(kThreads, RING && NK <= 4 ? 3 : 2) void mfma_p1_ker
   // to this wave, or to any wave of the workgroup if a workgroup barrier is certain to separate
   // the two tiles (the tail is produced 2w-1 columns after the head: at least two chunks later).
   // (ring: a row's tail line is stored (2w + d' - d) / 64 steps after the head line of the row below,
-  // d, d' < 64 the rows' line offsets in multiples of 8: at least one step from 2w - 56 >= 64 on)
-  const bool seam_across_waves = ALIGNED && (RING ? 2 * w - 56 >= KC : 2 * w - 1 >= 2 * KC);
+  // d, d' <= kMaxShift the rows' line offsets: at least one step from 2w - kMaxShift >= 64 on)
+  const bool seam_across_waves = ALIGNED && (RING ? 2 * w - kMaxShift >= KC : 2 * w - 1 >= 2 * KC);
 
   // B-operand: this wave's 32 rows of X, all of N, kept in registers
   u32x4 xop[NK];
@@ -445,16 +448,26 @@ __global__ __launch_bounds__(kThreads, RING && NK <= 4 ? 3 : 2) void mfma_p1_ker
   auto store_lines = [&](int k) __attribute__((always_inline)) {
     const int cb = c_start + k * KC;
     auto cb_of = [&](int s) { return RING ? cb + st_shift[s] - KC : cb; };
-    auto src_of = [&](int s) {
+    auto piece_of = [&](int s) {  // the lane's 16 bytes of slot s
       const int r = (lane >> 3) + 8 * s;
-      return RING ? st_src[s] + ((((st_piece[s] + 8 * ((k + 1) & 1)) & 15) ^ (r & 15)) << 3) : st_src[s];
+      if (RING == 2) {
+        u32x4 v;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const int e = (KC * ((k + 1) & 1) + st_shift[s] + 8 * (lane & 7) + 2 * j) & (2 * KC - 1);
+          v[j] = *reinterpret_cast<const uint32_t *>(st_src[s] + (((e >> 3) ^ (r & 15)) << 3) + (e & 7));
+        }
+        return v;
+      }
+      if (RING) return *reinterpret_cast<const u32x4 *>(st_src[s] + ((((st_piece[s] + 8 * ((k + 1) & 1)) & 15) ^ (r & 15)) << 3));
+      return *reinterpret_cast<const u32x4 *>(st_src[s]);
     };
-    if (cb - (RING ? KC : 0) >= iw_first + 31 - w && cb + KC - 1 - (RING ? 8 : 0) <= iw_first + w && iw_first + 31 < M) {
+    if (cb - (RING ? KC : 0) >= iw_first + 31 - w && cb + (RING ? kMaxShift : KC) - 1 <= iw_first + w && iw_first + 31 < M) {
       // every chunk of the wave's tile lies inside the band: nothing to decide, and each group of 8
       // lanes writes one whole 128-byte line, which is what makes the streaming store pay
 #pragma unroll
       for (int s = 0; s < 4; ++s) {
-        const u32x4 val = *reinterpret_cast<const u32x4 *>(src_of(s));
+        const u32x4 val = piece_of(s);
         if (ALIGNED && (RING || galign == 64))
           store_chunk_streaming(st_dst[s] + cb_of(s), val);
         else
@@ -471,7 +484,7 @@ __global__ __launch_bounds__(kThreads, RING && NK <= 4 ? 3 : 2) void mfma_p1_ker
         const int e_lo = st_lo[s] - cb_of(s), e_hi = st_hi[s] - cb_of(s);
         tail_hi[s] = -1;
         if (e_hi >= 0 && e_lo <= 7) {
-          v[s] = *reinterpret_cast<const u32x4 *>(src_of(s));
+          v[s] = piece_of(s);
           uint16_t *dst = st_dst[s] + cb_of(s);
           if (e_lo <= 0 && e_hi >= 7) {
             store_chunk<ALIGNED>(dst, v[s]);  // (plain: lines of edge tiles are completed piecewise)
@@ -1151,13 +1164,20 @@ hipError_t launch_p1(const Problem &p, const View &x, const View &y, const View 
   // 158 MB: 62 us, against 67 us with the ring of whole lines); beyond it the ring wins: 91 against
   // 116 us at w = 164 (259 MB), 119 against 200 us at w = 260, 327 against 747 us at w = 1028.
   const bool ring_pays = p.B * p.M * (2 * p.w + 1) * 2 >= (int64_t)220 << 20;
+  // windows that are not a multiple of 4: the same with lines at any even column offset, which needs
+  // the band 4-byte aligned (138-150 against 205 us at B96 M4096 N64, w = 255, 257, 258)
+  const bool ring_unaligned = !(p.flags & WM_FLAG_NO_ALIGNED_BAND) && ((uintptr_t)c.data % 4) == 0;
 #define WM_P1(NK)                                                                                            \
-  if (ALIGNED && galign != 64 && ring_pays)                                                                  \
-    hipLaunchKernelGGL((mfma_p1_kernel<T, NK, ALIGNED, ALIGNED>), grid, block, 0, p.stream,                  \
+  if (!ALIGNED && ring_pays && ring_unaligned)                                                               \
+    hipLaunchKernelGGL((mfma_p1_kernel<T, NK, true, 2>), grid, block, 0, p.stream, (const uint16_t *)x.data, \
+                       (const uint16_t *)y.data, (uint16_t *)c.data, (int)p.B, (int)p.M, (int)p.w, nblk, 2,  \
+                       x.sb, x.sr, y.sb, y.sr, c.sb);                                                        \
+  else if (ALIGNED && galign != 64 && ring_pays)                                                             \
+    hipLaunchKernelGGL((mfma_p1_kernel<T, NK, ALIGNED, ALIGNED ? 1 : 0>), grid, block, 0, p.stream,          \
                        (const uint16_t *)x.data, (const uint16_t *)y.data, (uint16_t *)c.data, (int)p.B,     \
                        (int)p.M, (int)p.w, nblk, galign, x.sb, x.sr, y.sb, y.sr, c.sb);                      \
   else                                                                                                       \
-    hipLaunchKernelGGL((mfma_p1_kernel<T, NK, ALIGNED, false>), grid, block, 0, p.stream,                    \
+    hipLaunchKernelGGL((mfma_p1_kernel<T, NK, ALIGNED, 0>), grid, block, 0, p.stream,                        \
                        (const uint16_t *)x.data, (const uint16_t *)y.data, (uint16_t *)c.data, (int)p.B,     \
                        (int)p.M, (int)p.w, nblk, galign, x.sb, x.sr, y.sb, y.sr, c.sb)
   // N = 128 with whole-line band stores: Y chunks straight into LDS, three workgroups per CU (32-bit

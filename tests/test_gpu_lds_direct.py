@@ -101,24 +101,25 @@ def test_kernel_choice_is_unchanged_by_the_switch(device):
 
 
 @pytest.mark.parametrize("B,M,N,w,dtype", [(26, 4099, 64, 580, torch.bfloat16), (7, 16390, 128, 516, torch.float16),
-                                           (44, 8200, 32, 172, torch.bfloat16)],
-                         ids=["N64-w580", "N128-w516", "N32-w172"])
+                                           (44, 8200, 32, 172, torch.bfloat16), (56, 4099, 64, 255, torch.bfloat16),
+                                           (56, 4100, 64, 258, torch.float16), (7, 8200, 48, 1023, torch.bfloat16)],
+                         ids=["N64-w580", "N128-w516", "N32-w172", "N64-w255", "N64-w258", "N48-w1023"])
 def test_band_out_ring_of_lines(device, B, M, N, w, dtype):
-    """A band beyond 220 MB whose column groups are 16-byte pieces but not whole lines (w % 4 == 0,
-    w % 32 != 0) is written through a ring of two chunks per row, every row in whole lines of its own
-    grid.  Every band entry is one dot product in a fixed order, so the result must equal, bit for
+    """A band beyond 220 MB whose rows do not begin a whole number of lines apart (w % 32 != 0) is
+    written through a ring of two chunks per row, every row in whole lines of its own grid (16-byte
+    pieces of the ring when w % 4 == 0, 4-byte units otherwise).  Every band entry is one dot product in a fixed order, so the result must equal, bit for
     bit, that of the kernel for unaligned bands (WM_FLAG_NO_ALIGNED_BAND: 16-byte stores on a common
     column grid), entries outside the sequence must be +0.0, and rows picked across the tensor must
     match the CPU oracle.  The band lives at three different offsets inside a poisoned buffer: nothing
     outside it may be written."""
     print(f"case B{B} M{M} N{N} w{w}", flush=True)
     W = 2 * w + 1
-    assert B * M * W * 2 >= 220 << 20 and w % 4 == 0 and w % 32 != 0
+    assert B * M * W * 2 >= 220 << 20 and w % 32 != 0
     q, k = (seeded((B, M, N), 340 + s, dtype).to(device) for s in range(2))
     kt = k.transpose(1, 2)
     want = abi.window_forward(q, kt, w, abi.NO_ALIGNED_BAND)
     store = torch.empty(B * M * W + 128, dtype=dtype, device=device)
-    for off in (0, 8, 40):
+    for off in (0, 8, 40) if w % 4 == 0 else (0, 2, 38):
         store.fill_(float("nan"))
         band = store[off:off + B * M * W].view(B, M, W)
         got = abi.window_forward(q, kt, w, 0, out=band)
