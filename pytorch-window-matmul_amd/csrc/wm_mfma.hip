@@ -336,7 +336,11 @@ __global__ __launch_bounds__(kThreads, NT <= 2 ? 3 : 2) void mfma_p3_kernel(cons
 // step for the lines that end after the last chunk.  RING = 2 is the same for windows that are not a
 // multiple of 4: the rows' lines then begin at any even column offset, a 16-byte piece of a line is
 // no longer one piece of the ring, and the staging area is read in 4-byte units.
-template <typename T, int NK, bool ALIGNED, int RING = 0>  // NK = N / 16
+// LINES: the column groups are whole lines (galign == 64); a compile-time fact on purpose: a store
+// path chosen at run time puts the stores into a branch, after which the compiler no longer knows
+// how many memory operations are in flight and turns its next wait into a wait for all of them
+// (85 -> 130 us at config 3).
+template <typename T, int NK, bool ALIGNED, int RING = 0, bool LINES = false>  // NK = N / 16
 __global__ __launch_bounds__(kThreads, RING && NK <= 4 ? 3 : 2) void mfma_p1_kernel(const uint16_t *__restrict__ X,
                                                               const uint16_t *__restrict__ Y,
                                                               uint16_t *__restrict__ C, int B, int M, int w,
@@ -468,7 +472,7 @@ __global__ __launch_bounds__(kThreads, RING && NK <= 4 ? 3 : 2) void mfma_p1_ker
 #pragma unroll
       for (int s = 0; s < 4; ++s) {
         const u32x4 val = piece_of(s);
-        if (ALIGNED && (RING || galign == 64))
+        if (ALIGNED && (RING || LINES))
           store_chunk_streaming(st_dst[s] + cb_of(s), val);
         else
           store_chunk<ALIGNED>(st_dst[s] + cb_of(s), val);  // (pieces of two lines: plain, see store_chunk_streaming)
@@ -725,10 +729,10 @@ __global__ __launch_bounds__(kThreads, 3) void mfma_p1_dma_kernel(const uint16_t
 #pragma unroll
       for (int s = 0; s < 4; ++s) {
         const u32x4 val = *reinterpret_cast<const u32x4 *>(st_src[s]);
-        if (ALIGNED && galign == 64)
+        if (ALIGNED)  // (this kernel is launched for whole-line column groups only)
           store_chunk_streaming(st_dst[s] + cb, val);
         else
-          store_chunk<ALIGNED>(st_dst[s] + cb, val);  // (pieces of two lines: plain, see store_chunk_streaming)
+          store_chunk<false>(st_dst[s] + cb, val);
       }
       wave_sync_lds();
       four_stores = true;
@@ -1167,19 +1171,19 @@ hipError_t launch_p1(const Problem &p, const View &x, const View &y, const View 
   // windows that are not a multiple of 4: the same with lines at any even column offset, which needs
   // the band 4-byte aligned (138-150 against 205 us at B96 M4096 N64, w = 255, 257, 258)
   const bool ring_unaligned = !(p.flags & WM_FLAG_NO_ALIGNED_BAND) && ((uintptr_t)c.data % 4) == 0;
+#define WM_P1_LAUNCH(NK, AL, RING, LINES, G)                                                                 \
+  hipLaunchKernelGGL((mfma_p1_kernel<T, NK, AL, RING, LINES>), grid, block, 0, p.stream,                     \
+                     (const uint16_t *)x.data, (const uint16_t *)y.data, (uint16_t *)c.data, (int)p.B,       \
+                     (int)p.M, (int)p.w, nblk, G, x.sb, x.sr, y.sb, y.sr, c.sb)
 #define WM_P1(NK)                                                                                            \
   if (!ALIGNED && ring_pays && ring_unaligned)                                                               \
-    hipLaunchKernelGGL((mfma_p1_kernel<T, NK, true, 2>), grid, block, 0, p.stream, (const uint16_t *)x.data, \
-                       (const uint16_t *)y.data, (uint16_t *)c.data, (int)p.B, (int)p.M, (int)p.w, nblk, 2,  \
-                       x.sb, x.sr, y.sb, y.sr, c.sb);                                                        \
+    WM_P1_LAUNCH(NK, true, 2, false, 2);                                                                     \
   else if (ALIGNED && galign != 64 && ring_pays)                                                             \
-    hipLaunchKernelGGL((mfma_p1_kernel<T, NK, ALIGNED, ALIGNED ? 1 : 0>), grid, block, 0, p.stream,          \
-                       (const uint16_t *)x.data, (const uint16_t *)y.data, (uint16_t *)c.data, (int)p.B,     \
-                       (int)p.M, (int)p.w, nblk, galign, x.sb, x.sr, y.sb, y.sr, c.sb);                      \
+    WM_P1_LAUNCH(NK, ALIGNED, (ALIGNED ? 1 : 0), false, galign);                                             \
+  else if (ALIGNED && galign == 64)                                                                          \
+    WM_P1_LAUNCH(NK, ALIGNED, 0, ALIGNED, galign);                                                           \
   else                                                                                                       \
-    hipLaunchKernelGGL((mfma_p1_kernel<T, NK, ALIGNED, 0>), grid, block, 0, p.stream,                        \
-                       (const uint16_t *)x.data, (const uint16_t *)y.data, (uint16_t *)c.data, (int)p.B,     \
-                       (int)p.M, (int)p.w, nblk, galign, x.sb, x.sr, y.sb, y.sr, c.sb)
+    WM_P1_LAUNCH(NK, ALIGNED, 0, false, galign)
   // N = 128 with whole-line band stores: Y chunks straight into LDS, three workgroups per CU (32-bit
   // byte offsets inside a batch element).  With 16-byte column groups most slots take the piecewise
   // store path, whose stores this kernel waits for: 10 % slower there than the kernel above.
@@ -1203,6 +1207,7 @@ hipError_t launch_p1(const Problem &p, const View &x, const View &y, const View 
     default: WM_P1(8); break;
   }
 #undef WM_P1
+#undef WM_P1_LAUNCH
   return hipGetLastError();
 }
 
