@@ -380,7 +380,7 @@ __global__ __launch_bounds__(kThreads, 2) void attention_forward_narrow_kernel(
 
 
 // ---------------------------------------------------------------------------------------------
-// N = 64 and N = 128: key and value chunks go from memory straight into LDS
+// Key and value chunks go from memory straight into LDS
 // ---------------------------------------------------------------------------------------------
 // Same tiling and arithmetic as attention_forward_kernel.  What differs is how the wavefronts are
 // kept busy:
@@ -399,11 +399,13 @@ __global__ __launch_bounds__(kThreads, NK <= 4 ? 3 : 2) void attention_forward_d
     const uint16_t *__restrict__ Q, const uint16_t *__restrict__ K, const uint16_t *__restrict__ V,
     uint16_t *__restrict__ O, float *__restrict__ L, int B, int M, int w, int nblk, float c, int64_t qsb, int64_t qsr,
     int64_t ksb, int64_t ksr, int64_t vsb, int64_t vsr, int64_t osb, int64_t osr) {
-  constexpr int N = 16 * NK, NB = NK / 2, PPR = 2 * NK, ROWB = 2 * N;  // pieces and bytes per tile row
+  // tile rows of 128 bytes (N <= 64) or 256 bytes; the pieces of a row beyond column N are never
+  // fetched (requested out of range: zeros, no memory traffic)
+  constexpr int N = 16 * NK, NB = (NK + 1) / 2, ROWB = NK <= 4 ? 128 : 256, PPR = ROWB / 16;
   constexpr int STAGES = NK <= 4 ? 3 : 2, DEPTH = STAGES - 1;
-  constexpr int TILE = AT_KC * N;          // elements per tile
+  constexpr int TILE = AT_KC * ROWB / 2;   // elements per tile
   constexpr int LOADS = 2 * (PPR / 4);     // loads per wavefront and chunk (K and V)
-  static_assert(NK == 4 || NK == 8, "tile rows of 128 or 256 bytes");
+  static_assert(NK >= 1 && NK <= 8, "N = 16 ... 128");
   __shared__ __attribute__((aligned(1024))) uint16_t k_lds[STAGES][TILE];
   __shared__ __attribute__((aligned(1024))) uint16_t v_lds[STAGES][TILE];
 
@@ -415,9 +417,11 @@ __global__ __launch_bounds__(kThreads, NK <= 4 ? 3 : 2) void attention_forward_d
   const int qw0 = i0 + 32 * wave;     // first query of this wavefront (scalar)
   const int qi = qw0 + (lane & 31);   // this lane's query
 
-  const u32x4 k_rsrc = make_rsrc(K + (int64_t)b * ksb, (uint32_t)((M - 1) * ksr * 2 + ROWB));
-  const u32x4 v_rsrc = make_rsrc(V + (int64_t)b * vsb, (uint32_t)((M - 1) * vsr * 2 + ROWB));
-  const uint32_t k_voff = dma_lane_offset<PPR>(wave, lane, ksr), v_voff = dma_lane_offset<PPR>(wave, lane, vsr);
+  const u32x4 k_rsrc = make_rsrc(K + (int64_t)b * ksb, (uint32_t)((M - 1) * ksr * 2 + 2 * N));
+  const u32x4 v_rsrc = make_rsrc(V + (int64_t)b * vsb, (uint32_t)((M - 1) * vsr * 2 + 2 * N));
+  const bool piece_in_row = (((64 * wave + lane) % PPR) ^ swz((64 * wave + lane) / PPR)) < N / 8;
+  const uint32_t k_voff = piece_in_row ? dma_lane_offset<PPR>(wave, lane, ksr) : 0x80000000u;
+  const uint32_t v_voff = piece_in_row ? dma_lane_offset<PPR>(wave, lane, vsr) : 0x80000000u;
   const uint32_t k_step = (uint32_t)(256 / PPR * ksr * 2), v_step = (uint32_t)(256 / PPR * vsr * 2);
   const uint32_t k_chunk = (uint32_t)(AT_KC * ksr * 2), v_chunk = (uint32_t)(AT_KC * vsr * 2);
   auto request = [&](int kc, int stage) {
@@ -633,7 +637,7 @@ hipError_t launch_forward(const Problem &p, const View &q, const View &k, const 
       WM_AT((attention_forward_narrow_kernel<T, NK, 3, true>));
     else
       WM_AT((attention_forward_narrow_kernel<T, NK, 3, false>));
-  } else if constexpr (NK == 4 || NK == 8) {
+  } else {
     // the buffer loads of the LDS-direct kernel address a batch element with 32-bit byte offsets
     const int64_t lim = 0x7fffffff;
     const bool fits = (p.M + 3 * AT_KC) * k.sr * 2 < lim && (p.M + 3 * AT_KC) * v.sr * 2 < lim && k.sr > 0 && v.sr > 0;
@@ -647,11 +651,6 @@ hipError_t launch_forward(const Problem &p, const View &q, const View &k, const 
     } else {
       WM_AT((attention_forward_kernel<T, NK, false>));
     }
-  } else {
-    if (mask)
-      WM_AT((attention_forward_kernel<T, NK, true>));
-    else
-      WM_AT((attention_forward_kernel<T, NK, false>));
   }
 #undef WM_AT
   return hipGetLastError();

@@ -388,7 +388,13 @@ constexpr float kLog2e = 1.4426950408889634f;
 
 template <int NK>
 struct BwdTile {
-  static constexpr int N = 16 * NK, NB = NK / 2, PPR = 2 * NK, ROWB = 2 * N, TILE = AB_KC * N;
+  // tile rows of 128 bytes (N <= 64) or 256 bytes; pieces of a row beyond column N are never fetched
+  static constexpr int N = 16 * NK, NB = (NK + 1) / 2, ROWB = NK <= 4 ? 128 : 256, PPR = ROWB / 16, TILE = AB_KC * ROWB / 2;
+  // byte offset of the lane's piece for the loads of a chunk (dma_chunk), out of range for pieces beyond N
+  static __device__ __forceinline__ uint32_t load_offset(int wave, int lane, int64_t row_stride) {
+    const int slot = 64 * wave + lane;
+    return ((slot % PPR) ^ swz(slot / PPR)) < N / 8 ? dma_lane_offset<PPR>(wave, lane, row_stride) : 0x80000000u;
+  }
   static constexpr int STAGES = NK <= 4 ? 3 : 2, DEPTH = STAGES - 1;
   typedef s16x4 __attribute__((address_space(3))) * lds_tr_ptr;
   // byte offsets inside a tile for the two ways a tile is read (see attention_forward_dma_kernel)
@@ -462,9 +468,9 @@ __global__ __launch_bounds__(kThreads, NK <= 4 ? 3 : 2) void attention_backward_
   const bool q_ok = qi < M;
   const float c = scale * kLog2e;
 
-  const u32x4 k_rsrc = make_rsrc(K + (int64_t)b * ksb, (uint32_t)((M - 1) * ksr * 2 + ROWB));
-  const u32x4 v_rsrc = make_rsrc(V + (int64_t)b * vsb, (uint32_t)((M - 1) * vsr * 2 + ROWB));
-  const uint32_t k_voff = dma_lane_offset<PPR>(wave, lane, ksr), v_voff = dma_lane_offset<PPR>(wave, lane, vsr);
+  const u32x4 k_rsrc = make_rsrc(K + (int64_t)b * ksb, (uint32_t)((M - 1) * ksr * 2 + 2 * N));
+  const u32x4 v_rsrc = make_rsrc(V + (int64_t)b * vsb, (uint32_t)((M - 1) * vsr * 2 + 2 * N));
+  const uint32_t k_voff = TL::load_offset(wave, lane, ksr), v_voff = TL::load_offset(wave, lane, vsr);
   const uint32_t k_step = (uint32_t)(256 / PPR * ksr * 2), v_step = (uint32_t)(256 / PPR * vsr * 2);
   const uint32_t k_chunk = (uint32_t)(AB_KC * ksr * 2), v_chunk = (uint32_t)(AB_KC * vsr * 2);
   auto request = [&](int kc, int stage) {
@@ -614,12 +620,12 @@ __global__ __launch_bounds__(kThreads, NK <= 4 ? 2 : 1) void attention_backward_
   const bool k_ok = kj < M;
   const float c = scale * kLog2e;
 
-  const u32x4 q_rsrc = make_rsrc(Q + (int64_t)b * qsb, (uint32_t)((M - 1) * qsr * 2 + ROWB));
-  const u32x4 g_rsrc = make_rsrc(dO + (int64_t)b * gsb, (uint32_t)((M - 1) * gsr * 2 + ROWB));
+  const u32x4 q_rsrc = make_rsrc(Q + (int64_t)b * qsb, (uint32_t)((M - 1) * qsr * 2 + 2 * N));
+  const u32x4 g_rsrc = make_rsrc(dO + (int64_t)b * gsb, (uint32_t)((M - 1) * gsr * 2 + 2 * N));
   // waves 0 and 2 fetch D, waves 1 and 3 the log-sum-exp (twice the same 256 bytes each: every
   // wavefront then has the same number of loads in flight, which is what the waits count)
   const u32x4 s_rsrc = make_rsrc(D + ((int64_t)(wave & 1) * B + b) * M, (uint32_t)(M * 4));
-  const uint32_t q_voff = dma_lane_offset<PPR>(wave, lane, qsr), g_voff = dma_lane_offset<PPR>(wave, lane, gsr);
+  const uint32_t q_voff = TL::load_offset(wave, lane, qsr), g_voff = TL::load_offset(wave, lane, gsr);
   const uint32_t q_step = (uint32_t)(256 / PPR * qsr * 2), g_step = (uint32_t)(256 / PPR * gsr * 2);
   const uint32_t q_chunk = (uint32_t)(AB_KC * qsr * 2), g_chunk = (uint32_t)(AB_KC * gsr * 2);
   auto request = [&](int qc, int stage) {
@@ -763,7 +769,7 @@ hipError_t launch_backward(const Problem &p, const View &q, const View &k, const
   const dim3 grid((unsigned)(groups * 8 * nblk)), block(kThreads);
   typedef const uint16_t *in_t;
   typedef uint16_t *out_t;
-  if constexpr (NK == 4 || NK == 8) {
+  {
     // the LDS-direct kernels address a batch element with 32-bit byte offsets
     const int64_t lim = 0x7fffffff;
     bool fits = !(p.flags & WM_FLAG_NO_LDS_DIRECT) && (p.M + 3 * AB_KC) * 4 < lim;

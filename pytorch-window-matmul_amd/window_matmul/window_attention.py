@@ -23,15 +23,10 @@ def _chain_is_faster(window_size: int, width: int) -> bool:
     """Windows at which a training step is faster through the separate ops than through the fused
     kernels, whose recomputing backward costs the same at every narrow window.  Measured on bf16
     tensors of 100 M elements with M = 16384 (chain / fused, ms per step): N = 32: 0.32 / 0.33 at
-    w = 4, 0.35 / 0.32 at w = 8; N = 64: 0.58 / 0.66 at w = 12, 0.72 / 0.67 at w = 14; N = 128:
-    0.72 / 0.79 at w = 32, 0.86 / 0.84 at w = 40; N = 96 (as every width that is not 64 or 128, on
-    the fused kernels that stage their chunks through registers): 1.06 / 1.19 at w = 48, 1.21 / 1.16
-    at w = 64."""
-    if width <= 32:
-        return window_size <= 4
-    if width <= 64:
-        return window_size <= 13
-    return window_size <= (36 if width == 128 else 56)
+    w = 4, 0.34 / 0.34 at w = 8; N = 64: 0.58 / 0.66 at w = 12, 0.72 / 0.67 at w = 14; N = 96:
+    0.81 / 0.86 at w = 32, 0.96 / 0.92 at w = 40; N = 128: 0.72 / 0.79 at w = 32, 0.86 / 0.84 at
+    w = 40."""
+    return window_size <= (4 if width <= 32 else 13 if width <= 64 else 36)
 
 
 class WindowAttentionFunc(torch.autograd.Function):
