@@ -60,6 +60,33 @@ torch::Tensor band_friendly(const torch::Tensor &t) {
   return aligned16(c) || c.numel() == 0 ? c : c.clone(at::MemoryFormat::Contiguous);
 }
 
+// Head widths that the tuned kernels do not take -- N not a multiple of 16 for 16-bit storage, of 8
+// for float32 -- are padded with zero columns to the next such width (up to 128): zero columns add
+// nothing to a dot product and produce result columns that are cut off again, and two or three
+// passes over the (B,M,N) tensors cost far less than the strided kernels, which take such shapes
+// otherwise (float64 and N > 128 still do).
+int64_t padded_width(const torch::Tensor &t) {
+  const int64_t N = t.size(2);
+  int64_t unit;
+  switch (t.scalar_type()) {
+    case at::kHalf:
+    case at::kBFloat16: unit = 16; break;
+    case at::kFloat: unit = 8; break;
+    default: return N;
+  }
+  const int64_t Np = (N + unit - 1) / unit * unit;
+  return N > 0 && Np <= 128 ? Np : N;
+}
+torch::Tensor pad_columns(const torch::Tensor &t, int64_t Np) {
+  if (t.size(2) == Np) return t;
+  auto padded = torch::zeros({t.size(0), t.size(1), Np}, t.options());
+  padded.narrow(2, 0, t.size(2)).copy_(t);
+  return padded;
+}
+torch::Tensor cut_columns(const torch::Tensor &t, int64_t N) {
+  return t.size(2) == N ? t : t.narrow(2, 0, N).contiguous();
+}
+
 // K comes as (B,N,M).  The kernels want key rows contiguous, which is what a
 // transposed view of a row-major (B,M,N) tensor already is; anything else is
 // copied into that layout once (the reference always copies: cuda:236).
@@ -111,9 +138,9 @@ torch::Tensor window_matmul_forward(torch::Tensor src, torch::Tensor other, int6
   check_window_inputs(src, other);
   const int dtype = abi_dtype(src, "window_matmul_fw_cuda");
   at::hip::HIPGuardMasqueradingAsCUDA guard(src.device());
-  const int64_t B = src.size(0), M = src.size(1), N = src.size(2);
-  auto q = vector_friendly(src);
-  auto krows = key_rows(other);  // (B,M,N) view or copy
+  const int64_t B = src.size(0), M = src.size(1), N = padded_width(src);
+  auto q = vector_friendly(pad_columns(src, N));
+  auto krows = pad_columns(key_rows(other), N);  // (B,M,N) view or copy
   auto kt = krows.transpose(1, 2);
   auto out = torch::empty({B, M, 2 * window_size + 1}, src.options());
   wm_operand oq = operand(q), ok = operand(kt), oa = operand(out);
@@ -134,20 +161,23 @@ std::tuple<c10::optional<torch::Tensor>, c10::optional<torch::Tensor>> window_ma
   check_grad(grad_output, src, {B, M, 2 * window_size + 1});
   const int dtype = abi_dtype(src, "window_matmul_bw_cuda");
   at::hip::HIPGuardMasqueradingAsCUDA guard(src.device());
-  auto q = vector_friendly(src);
-  auto kt = key_rows(other).transpose(1, 2);
+  const int64_t Np = padded_width(src);
+  auto q = vector_friendly(pad_columns(src, Np));
+  auto kt = pad_columns(key_rows(other), Np).transpose(1, 2);
   auto ga = band_friendly(grad_output);
   c10::optional<torch::Tensor> grad_q, grad_k;
-  if (need_src) grad_q = torch::empty({B, M, N}, src.options());
+  if (need_src) grad_q = torch::empty({B, M, Np}, src.options());
   // grad_k is produced row-major per key row and handed back in the (B,N,M)
   // orientation of `other` as a transposed view, like the reference (cuda:318).
-  if (need_other) grad_k = torch::empty({B, M, N}, src.options()).transpose(1, 2);
+  if (need_other) grad_k = torch::empty({B, M, Np}, src.options()).transpose(1, 2);
   wm_operand oq = operand(q), ok = operand(kt), oga = operand(ga), ogq{}, ogk{};
   if (need_src) ogq = operand(*grad_q);
   if (need_other) ogk = operand(*grad_k);
   raise_on_error(wm_window_matmul_backward(&oq, &ok, &oga, need_src ? &ogq : nullptr, need_other ? &ogk : nullptr, B,
-                                           M, N, window_size, dtype, 0, current_stream(src)),
+                                           M, Np, window_size, dtype, 0, current_stream(src)),
                  "window_matmul_backward");
+  if (need_src) grad_q = cut_columns(*grad_q, N);
+  if (need_other && Np != N) grad_k = grad_k->narrow(1, 0, N);
   return std::make_tuple(grad_q, grad_k);
 }
 
@@ -158,13 +188,14 @@ torch::Tensor unwindow_matmul_forward(torch::Tensor src, torch::Tensor other, in
   const int dtype = abi_dtype(src, "unwindow_matmul_fw_cuda");
   at::hip::HIPGuardMasqueradingAsCUDA guard(src.device());
   const int64_t B = other.size(0), M = other.size(1), N = other.size(2);
+  const int64_t Np = padded_width(other);
   auto a = band_friendly(src);
-  auto v = vector_friendly(other);
-  auto out = torch::empty({B, M, N}, src.options());
+  auto v = vector_friendly(pad_columns(other, Np));
+  auto out = torch::empty({B, M, Np}, src.options());
   wm_operand oa = operand(a), ov = operand(v), oo = operand(out);
-  raise_on_error(wm_unwindow_matmul_forward(&oa, &ov, &oo, B, M, N, window_size, dtype, 0, current_stream(src)),
+  raise_on_error(wm_unwindow_matmul_forward(&oa, &ov, &oo, B, M, Np, window_size, dtype, 0, current_stream(src)),
                  "unwindow_matmul_forward");
-  return out;
+  return cut_columns(out, N);
 }
 
 // reference: unwindow_matmul_backward -> unwindow_matmul_bw_cuda (window_matmul.cpp:93-98, cuda:360-416)
@@ -177,18 +208,20 @@ std::tuple<c10::optional<torch::Tensor>, c10::optional<torch::Tensor>> unwindow_
   check_grad(grad_output, src, {B, M, N});
   const int dtype = abi_dtype(src, "unwindow_matmul_bw_cuda");
   at::hip::HIPGuardMasqueradingAsCUDA guard(src.device());
+  const int64_t Np = padded_width(other);
   auto a = band_friendly(src);
-  auto v = vector_friendly(other);
-  auto go = vector_friendly(grad_output);
+  auto v = vector_friendly(pad_columns(other, Np));
+  auto go = vector_friendly(pad_columns(grad_output, Np));
   c10::optional<torch::Tensor> grad_a, grad_v;
   if (need_src) grad_a = torch::empty({B, M, 2 * window_size + 1}, src.options());
-  if (need_other) grad_v = torch::empty({B, M, N}, src.options());
+  if (need_other) grad_v = torch::empty({B, M, Np}, src.options());
   wm_operand oa = operand(a), ov = operand(v), ogo = operand(go), oga{}, ogv{};
   if (need_src) oga = operand(*grad_a);
   if (need_other) ogv = operand(*grad_v);
   raise_on_error(wm_unwindow_matmul_backward(&oa, &ov, &ogo, need_src ? &oga : nullptr, need_other ? &ogv : nullptr, B,
-                                             M, N, window_size, dtype, 0, current_stream(src)),
+                                             M, Np, window_size, dtype, 0, current_stream(src)),
                  "unwindow_matmul_backward");
+  if (need_other) grad_v = cut_columns(*grad_v, N);
   return std::make_tuple(grad_a, grad_v);
 }
 

@@ -254,3 +254,37 @@ def test_views_at_a_misaligned_storage_offset(device, dtype):
     if dtype != torch.float32:
         fused = window_attention(q, k, v, w, 0.125)
         assert torch.equal(window_attention(shifted(q), shifted(k), shifted(v), w, 0.125), fused)
+
+
+@pytest.mark.parametrize("dtype,N", [(torch.bfloat16, 3), (torch.bfloat16, 40), (torch.float16, 72), (torch.float16, 100),
+                                      (torch.float32, 3), (torch.float32, 20), (torch.float32, 50), (torch.float32, 121)],
+                         ids=lambda x: str(x).replace("torch.", ""))
+@pytest.mark.parametrize("w", [2, 9, 40])
+def test_head_widths_between_the_tuned_ones(device, dtype, N, w):
+    """A head width that is not a multiple of 16 (16-bit storage) or 8 (float32) is padded with zero
+    columns inside the extension and runs on the tuned kernels; results, shapes, contiguity and all
+    four gradients are those of the operation on the unpadded tensors (CPU oracle)."""
+    from window_matmul import unwindow_matmul, window_matmul
+
+    B, M = 3, 150
+    tol = dict(rtol=1e-3, atol=1e-3) if dtype == torch.float32 else dict(rtol=2e-2, atol=2e-2)
+    q, k, v = (seeded((B, M, N), 400 + s, dtype) for s in range(3))
+    a = seeded((B, M, 2 * w + 1), 410, dtype, 0.25)
+    g_att, g_out = seeded((B, M, 2 * w + 1), 411, dtype, 0.25), seeded((B, M, N), 412, dtype)
+    dq, dk, dv, da = (t.clone().to(device).requires_grad_(True) for t in (q, k, v, a))
+    att = window_matmul(dq, dk.transpose(1, 2), w)
+    out = unwindow_matmul(da, dv, w)
+    assert att.shape == (B, M, 2 * w + 1) and out.shape == (B, M, N) and out.is_contiguous()
+    att.backward(g_att.to(device))
+    out.backward(g_out.to(device))
+    f = lambda t: t.float()  # noqa: E731
+    ktc = f(k).transpose(1, 2).contiguous()
+    torch.testing.assert_close(f(att).cpu(), oracle.window_matmul_forward(f(q), ktc, w), **tol)
+    torch.testing.assert_close(f(out).cpu(), oracle.unwindow_matmul_forward(f(a), f(v), w), **tol)
+    want_q, want_k = oracle.window_matmul_backward(f(q), ktc, w, f(g_att))
+    want_a, want_v = oracle.unwindow_matmul_backward(f(a), f(v), w, f(g_out))
+    assert dq.grad.shape == q.shape and dk.grad.shape == k.shape and dv.grad.shape == v.shape
+    torch.testing.assert_close(f(dq.grad).cpu(), want_q, **tol)
+    torch.testing.assert_close(f(dk.grad).cpu(), want_k.transpose(1, 2), **tol)
+    torch.testing.assert_close(f(da.grad).cpu(), want_a, **tol)
+    torch.testing.assert_close(f(dv.grad).cpu(), want_v, **tol)
