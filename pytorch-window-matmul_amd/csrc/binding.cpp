@@ -12,6 +12,9 @@
 // (reference window_matmul.cpp:15).
 #include <torch/extension.h>
 
+#include <algorithm>
+#include <vector>
+
 #include <ATen/hip/impl/HIPGuardImplMasqueradingAsCUDA.h>
 #include <ATen/hip/impl/HIPStreamMasqueradingAsCUDA.h>
 
@@ -87,6 +90,16 @@ torch::Tensor cut_columns(const torch::Tensor &t, int64_t N) {
   return t.size(2) == N ? t : t.narrow(2, 0, N).contiguous();
 }
 
+// Head widths beyond 128 (the widest the tuned kernels take) are worked on in slices of 128 columns:
+// results with N columns are independent per slice, bands are the sum over the slices.  The slices
+// of a band are computed and summed in float32 whatever the storage type (a 16-bit partial band
+// would be rounded at the magnitude of the partial sums, which shows where the slices cancel) and
+// the sum is rounded once.  float64 has no tuned kernels and is not sliced.
+constexpr int64_t kMaxWidth = 128;
+bool sliced_width(const torch::Tensor &t) {
+  return t.size(2) > kMaxWidth && (t.scalar_type() == at::kHalf || t.scalar_type() == at::kBFloat16 || t.scalar_type() == at::kFloat);
+}
+
 // K comes as (B,N,M).  The kernels want key rows contiguous, which is what a
 // transposed view of a row-major (B,M,N) tensor already is; anything else is
 // copied into that layout once (the reference always copies: cuda:236).
@@ -138,6 +151,15 @@ torch::Tensor window_matmul_forward(torch::Tensor src, torch::Tensor other, int6
   check_window_inputs(src, other);
   const int dtype = abi_dtype(src, "window_matmul_fw_cuda");
   at::hip::HIPGuardMasqueradingAsCUDA guard(src.device());
+  if (sliced_width(src)) {
+    torch::Tensor band;
+    for (int64_t h = 0; h < src.size(2); h += kMaxWidth) {
+      const int64_t n = std::min(kMaxWidth, src.size(2) - h);
+      auto part = window_matmul_forward(src.narrow(2, h, n).to(at::kFloat), other.narrow(1, h, n).to(at::kFloat), window_size);
+      if (h == 0) band = part; else band.add_(part);
+    }
+    return band.to(src.scalar_type());
+  }
   const int64_t B = src.size(0), M = src.size(1), N = padded_width(src);
   auto q = vector_friendly(pad_columns(src, N));
   auto krows = pad_columns(key_rows(other), N);  // (B,M,N) view or copy
@@ -161,6 +183,19 @@ std::tuple<c10::optional<torch::Tensor>, c10::optional<torch::Tensor>> window_ma
   check_grad(grad_output, src, {B, M, 2 * window_size + 1});
   const int dtype = abi_dtype(src, "window_matmul_bw_cuda");
   at::hip::HIPGuardMasqueradingAsCUDA guard(src.device());
+  if (sliced_width(src)) {
+    std::vector<torch::Tensor> gq, gk;
+    for (int64_t h = 0; h < N; h += kMaxWidth) {
+      const int64_t n = std::min(kMaxWidth, N - h);
+      auto part = window_matmul_backward(src.narrow(2, h, n), other.narrow(1, h, n), window_size, grad_output, need_src, need_other);
+      if (need_src) gq.push_back(*std::get<0>(part));
+      if (need_other) gk.push_back(*std::get<1>(part));
+    }
+    c10::optional<torch::Tensor> grad_q, grad_k;
+    if (need_src) grad_q = torch::cat(gq, 2);
+    if (need_other) grad_k = torch::cat(gk, 1);
+    return std::make_tuple(grad_q, grad_k);
+  }
   const int64_t Np = padded_width(src);
   auto q = vector_friendly(pad_columns(src, Np));
   auto kt = pad_columns(key_rows(other), Np).transpose(1, 2);
@@ -188,6 +223,12 @@ torch::Tensor unwindow_matmul_forward(torch::Tensor src, torch::Tensor other, in
   const int dtype = abi_dtype(src, "unwindow_matmul_fw_cuda");
   at::hip::HIPGuardMasqueradingAsCUDA guard(src.device());
   const int64_t B = other.size(0), M = other.size(1), N = other.size(2);
+  if (sliced_width(other)) {
+    std::vector<torch::Tensor> parts;
+    for (int64_t h = 0; h < N; h += kMaxWidth)
+      parts.push_back(unwindow_matmul_forward(src, other.narrow(2, h, std::min(kMaxWidth, N - h)), window_size));
+    return torch::cat(parts, 2);
+  }
   const int64_t Np = padded_width(other);
   auto a = band_friendly(src);
   auto v = vector_friendly(pad_columns(other, Np));
@@ -208,6 +249,22 @@ std::tuple<c10::optional<torch::Tensor>, c10::optional<torch::Tensor>> unwindow_
   check_grad(grad_output, src, {B, M, N});
   const int dtype = abi_dtype(src, "unwindow_matmul_bw_cuda");
   at::hip::HIPGuardMasqueradingAsCUDA guard(src.device());
+  if (sliced_width(other)) {
+    c10::optional<torch::Tensor> grad_a, grad_v;
+    std::vector<torch::Tensor> gv;
+    for (int64_t h = 0; h < N; h += kMaxWidth) {
+      const int64_t n = std::min(kMaxWidth, N - h);
+      if (need_other)
+        gv.push_back(*std::get<1>(unwindow_matmul_backward(src, other.narrow(2, h, n), window_size, grad_output.narrow(2, h, n), false, true)));
+      if (need_src) {  // grad_a = band of grad_output against other: in float32, as in window_matmul_forward
+        auto part = window_matmul_forward(grad_output.narrow(2, h, n).to(at::kFloat), other.narrow(2, h, n).transpose(1, 2).to(at::kFloat), window_size);
+        if (h == 0) grad_a = part; else grad_a->add_(part);
+      }
+    }
+    if (need_src) grad_a = grad_a->to(src.scalar_type());
+    if (need_other) grad_v = torch::cat(gv, 2);
+    return std::make_tuple(grad_a, grad_v);
+  }
   const int64_t Np = padded_width(other);
   auto a = band_friendly(src);
   auto v = vector_friendly(pad_columns(other, Np));

@@ -257,13 +257,15 @@ def test_views_at_a_misaligned_storage_offset(device, dtype):
 
 
 @pytest.mark.parametrize("dtype,N", [(torch.bfloat16, 3), (torch.bfloat16, 40), (torch.float16, 72), (torch.float16, 100),
-                                      (torch.float32, 3), (torch.float32, 20), (torch.float32, 50), (torch.float32, 121)],
+                                      (torch.float32, 3), (torch.float32, 20), (torch.float32, 50), (torch.float32, 121),
+                                      (torch.bfloat16, 160), (torch.float16, 256), (torch.bfloat16, 136), (torch.float32, 200)],
                          ids=lambda x: str(x).replace("torch.", ""))
 @pytest.mark.parametrize("w", [2, 9, 40])
 def test_head_widths_between_the_tuned_ones(device, dtype, N, w):
     """A head width that is not a multiple of 16 (16-bit storage) or 8 (float32) is padded with zero
-    columns inside the extension and runs on the tuned kernels; results, shapes, contiguity and all
-    four gradients are those of the operation on the unpadded tensors (CPU oracle)."""
+    columns inside the extension, one beyond 128 is worked on in slices of 128 columns, and both run
+    on the tuned kernels; results, shapes, contiguity and all four gradients are those of the
+    operation on the whole tensors (CPU oracle)."""
     from window_matmul import unwindow_matmul, window_matmul
 
     B, M = 3, 150
