@@ -137,3 +137,30 @@ def test_band_out_ring_of_lines(device, B, M, N, w, dtype):
             ks = k[b, lo:hi].float().cpu().unsqueeze(0)
             ref = oracle.window_matmul_forward(qs, ks.transpose(1, 2).contiguous(), w)[0, i0 - lo:i0 - lo + 40]
             torch.testing.assert_close(want[b, rows].float().cpu(), ref, **TOL)
+
+
+@pytest.mark.parametrize("w", [40, 41, 64])
+def test_band_at_an_odd_element_offset(device, w):
+    """A band whose first element sits at an odd element offset is only 2-byte aligned: neither the
+    16-byte pieces of the LDS-direct kernels nor the whole-line stores apply, the products take the
+    kernels for unaligned bands and give the numbers of the aligned call."""
+    B, M, N, dtype = 3, 700, 64, torch.bfloat16
+    W = 2 * w + 1
+    q, k, v, go = (seeded((B, M, N), 350 + s, dtype).to(device) for s in range(4))
+    a = seeded((B, M, W), 360, dtype, 0.25).to(device)
+    store = torch.full((B * M * W + 8,), float("nan"), dtype=dtype, device=device)
+    odd = store[1:1 + B * M * W].view(B, M, W)
+    assert odd.data_ptr() % 4 == 2
+    want_att = abi.window_forward(q, k.transpose(1, 2), w)
+    got_att = abi.window_forward(q, k.transpose(1, 2), w, out=odd)
+    assert torch.equal(bits(got_att), bits(want_att)) and bool(torch.isnan(store[0])) and bool(torch.isnan(store[1 + B * M * W:]).all())
+    odd.copy_(a)
+    torch.testing.assert_close(abi.unwindow_forward(odd, v, w).float(), abi.unwindow_forward(a, v, w).float(), **TOL)
+    g_a, g_v = abi.unwindow_backward(odd, v, w, go)
+    w_a, w_v = abi.unwindow_backward(a, v, w, go)
+    assert torch.equal(bits(g_a), bits(w_a))
+    torch.testing.assert_close(g_v.float(), w_v.float(), **TOL)
+    g_q, g_k = abi.window_backward(q, k.transpose(1, 2), w, odd)
+    w_q, w_k = abi.window_backward(q, k.transpose(1, 2), w, a)
+    torch.testing.assert_close(g_q.float(), w_q.float(), **TOL)
+    torch.testing.assert_close(g_k.float(), w_k.float(), **TOL)
