@@ -249,11 +249,13 @@ class Bench:
                 fused = {"fwd_ms": round(fwd, 4), "fwd_TFLOPs": round(2 * self.unit / fwd / 1e9, 1),
                          "fwd_mfma_frac": round(2 * self.unit / fwd / 1e9 / MFMA_PEAK_TFLOPS, 4),
                          "fwd_hbm_frac": round((4 * B * M * N * es + 4 * B * M) / fwd / 1e6 / HBM_PEAK_GBS, 4)}
-                if cfg["backward"]:
-                    bwd = time_gpu(lambda: abi.attention_backward(q, k, v, fo, flse, go, w, 1.0), iters, 3)
-                    fused.update({"bwd_ms": round(bwd, 4), "bwd_TFLOPs": round(4 * self.unit / bwd / 1e9, 1),
-                                  "bwd_mfma_frac": round(4 * self.unit / bwd / 1e9 / MFMA_PEAK_TFLOPS, 4),
-                                  "step_mfma_frac": round(6 * self.unit / (fwd + bwd) / 1e9 / MFMA_PEAK_TFLOPS, 4)})
+                # (a forward-only workload gets the backward of a training step as well: its band is so
+                # narrow that the step is bound by the eight tensors it reads and writes, q k v o dO dq dk dv)
+                bwd = time_gpu(lambda: abi.attention_backward(q, k, v, fo, flse, go, w, 1.0), iters, 3)
+                fused.update({"bwd_ms": round(bwd, 4), "bwd_TFLOPs": round(4 * self.unit / bwd / 1e9, 1),
+                              "bwd_mfma_frac": round(4 * self.unit / bwd / 1e9 / MFMA_PEAK_TFLOPS, 4),
+                              "bwd_hbm_frac": round((8 * B * M * N * es + 4 * B * M) / bwd / 1e6 / HBM_PEAK_GBS, 4),
+                              "step_mfma_frac": round(6 * self.unit / (fwd + bwd) / 1e9 / MFMA_PEAK_TFLOPS, 4)})
                 out["fused_attention"] = fused
                 del fo, flse
             # device-to-device copy of the band as the achievable-bandwidth yardstick

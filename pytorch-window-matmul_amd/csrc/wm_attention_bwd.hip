@@ -17,6 +17,8 @@
 // stationary side (lane % 32) and 16 rows of the streamed side, so P and dS come out of the
 // arithmetic already arranged as B operands of the products that consume them, and the streamed
 // tiles are read from LDS both by rows (first products) and transposed (second products).
+// Narrow windows of heads up to 64 wide take a third kernel that does the work of both at once
+// (attention_backward_narrow_kernel below).
 #include "wm_mfma_common.hpp"
 
 #include <type_traits>
@@ -759,6 +761,269 @@ __global__ __launch_bounds__(kThreads, NK <= 4 ? 2 : 1) void attention_backward_
   if (dV != nullptr) store_wave_rows<T, NB>(stage_rows, dv, 1.0f, dV + (int64_t)b * dvsb, dvsr, kw0, M, N, lane);
 }
 
+// ---------------------------------------------------------------------------------------------
+// Narrow windows (w <= 16 (NKB - 1), N <= 64): one kernel for all three gradients
+// ---------------------------------------------------------------------------------------------
+// With a band of at most 65 entries the two kernels above read q, k, v and dO twice and exchange D
+// through memory.  Here a workgroup owns 128 rows both as keys and as queries; the rows it needs
+// from its neighbours (w on either side) come with the tiles:
+//   1. Q and dO rows [i0 - w, i0 + 127 + w] go straight into two LDS tiles (rows further out, up to
+//      the tile's 16 (NKB - 1) on either side, are not fetched); D = dO . O and the log-sum-exp of
+//      those rows go into a small LDS array; the wavefront's own k and v rows into registers.
+//   2. As keys: S, dP against the 32 NKB query rows a wavefront's keys can reach, dV^T += dO^T P,
+//      dK^T += Q^T dS; dK and dV leave through LDS as whole lines.
+//   3. K and V rows replace Q and dO in the two tiles, the wavefront's own q and dO rows go into
+//      registers; as queries: S^T, dP^T, dQ^T += K^T dS^T; dQ leaves the same way.
+// Memory sees q, k, v, dO, O once each (plus the halo, which the neighbouring workgroup has
+// usually just brought into the L2) and dQ, dK, dV once: nothing else bounds this kernel.
+template <typename T, int NK, int NKB>
+__global__ __launch_bounds__(kThreads, NK >= 3 && NKB == 3 ? 2 : 3) void attention_backward_narrow_kernel(
+    const uint16_t *__restrict__ Q, const uint16_t *__restrict__ K, const uint16_t *__restrict__ V,
+    const uint16_t *__restrict__ O, const uint16_t *__restrict__ dO, const float *__restrict__ L,
+    uint16_t *__restrict__ dQ, uint16_t *__restrict__ dK, uint16_t *__restrict__ dV, int B, int M, int w, int nblk,
+    float scale, int64_t qsb, int64_t qsr, int64_t ksb, int64_t ksr, int64_t vsb, int64_t vsr, int64_t osb, int64_t osr,
+    int64_t gsb, int64_t gsr, int64_t dqsb, int64_t dqsr, int64_t dksb, int64_t dksr, int64_t dvsb, int64_t dvsr) {
+  static_assert(NK <= 4, "rows of 128 bytes: two tiles and the staging must fit 64 KB of LDS");
+  constexpr int N = 16 * NK, NB = (NK + 1) / 2;
+  constexpr int PADW = 16 * (NKB - 1);     // tile rows before the first and after the last own row
+  constexpr int ROWS = AB_TM + 2 * PADW;   // rows of a tile
+  typedef LdsTile<ROWS, 8> TL;
+  constexpr int LOADS = TL::LOADS;
+  __shared__ __attribute__((aligned(1024))) uint16_t tile_a[TL::ELEMS];  // Q, then K
+  __shared__ __attribute__((aligned(1024))) uint16_t tile_b[TL::ELEMS];  // dO, then V
+  __shared__ __attribute__((aligned(16))) float stat[2][ROWS];           // [0] D, [1] log-sum-exp in log2 units
+  static_assert(4 * RowStage<NB>::ELEMS <= TL::ELEMS, "the four staging areas must fit one tile");
+
+  int b, blk;
+  if (!decode_block(nblk, B, &b, &blk)) return;
+  const int tid = threadIdx.x, lane = tid & 63, half = lane >> 5;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int i0 = blk * AB_TM;
+  const int t0 = i0 - PADW;         // sequence row of tile row 0 (negative in the first workgroup)
+  const int rw0 = i0 + 32 * wave;   // first own row of this wavefront (scalar)
+  const int ri = rw0 + (lane & 31);
+  const bool r_ok = ri < M;
+  const float c = scale * kLog2e;
+  const int need_lo = max(i0 - w, 0), need_hi = min(i0 + AB_TM - 1 + w, M - 1);  // rows anybody reads
+
+  // one tile from a tensor: tile row r = sequence row t0 + r; rows nobody reads and pieces beyond
+  // column N are requested out of range (zeros, no traffic)
+  const int piece = TL::load_piece(wave, lane);
+  auto request = [&](const uint16_t *base, int64_t sr, const uint16_t *tile) __attribute__((always_inline)) {
+    const u32x4 rsrc = make_rsrc(base, (uint32_t)((M - 1) * sr * 2 + 2 * N));
+    const uint32_t lds = lds_address(tile) + 1024 * wave;
+#pragma unroll
+    for (int j = 0; j < LOADS; ++j) {
+      const int row = t0 + TL::load_row(wave, lane, j);
+      const bool wanted = row >= need_lo && row <= need_hi && piece < N / 8;
+      dma_piece(rsrc, lds + 4096 * j, wanted ? (uint32_t)(row * sr * 2 + piece * 16) : 0x80000000u, 0);
+    }
+  };
+  request(Q + (int64_t)b * qsb, qsr, tile_a);
+  request(dO + (int64_t)b * gsb, gsr, tile_b);
+
+  const uint32_t row_at = TL::row_at(lane), tr_at = TL::tr_at(lane);
+  const float ninf = -__builtin_huge_valf();
+  const int r32 = lane & 31;
+  const bool want_kv = dK != nullptr || dV != nullptr;
+  // a group of 32 tile rows that starts at row `first` (a multiple of 8) as B operand: row lane % 32,
+  // pieces 2 ks + lane / 32
+  auto own_rows = [&](const uint16_t *tile, int first, uint32_t at, int ks) __attribute__((always_inline)) {
+    return *reinterpret_cast<const u32x4 *>(reinterpret_cast<const char *>(tile) + first * TL::ROWB + (at ^ (32 * ks)));
+  };
+
+  // For D = dO . O the rows of O come in operand layout (lane pair per row) and meet the rows of dO
+  // in the tile: the wavefront's own 32 rows, and in the first and last wavefront the rows before
+  // and after the workgroup's own.
+  const int own_first = PADW + 32 * wave;                            // tile row of the wavefront's first own row
+  const int halo_first = wave == 0 ? 0 : PADW + AB_TM;               // (waves 0 and 3 only)
+  const int h32 = r32 < PADW ? r32 : 0;                              // lanes beyond the halo repeat its first row
+  const uint32_t halo_at = TL::row_at(32 * half + h32);
+  u32x4 o_own[NK], o_halo[NK];
+  float l_own, l_halo = 0.0f;
+  {
+    const int row = t0 + own_first + r32;
+    const bool ok = row >= need_lo && row <= need_hi;
+    const uint16_t *orow = O + (int64_t)b * osb + (int64_t)row * osr + 8 * half;
+#pragma unroll
+    for (int ks = 0; ks < NK; ++ks) o_own[ks] = load_row_chunk(orow + 16 * ks, O, ok);
+    l_own = ok ? L[(int64_t)b * M + row] * kLog2e : 0.0f;
+  }
+  if (wave == 0 || wave == 3) {
+    const int row = t0 + halo_first + h32;
+    const bool ok = row >= need_lo && row <= need_hi;
+    const uint16_t *orow = O + (int64_t)b * osb + (int64_t)row * osr + 8 * half;
+#pragma unroll
+    for (int ks = 0; ks < NK; ++ks) o_halo[ks] = load_row_chunk(orow + 16 * ks, O, ok);
+    l_halo = ok ? L[(int64_t)b * M + row] * kLog2e : 0.0f;
+  }
+  // own rows as keys: B operands of the first two products
+  u32x4 kf[NK], vf[NK];
+  if (want_kv) {
+    const uint16_t *kr = K + (int64_t)b * ksb + (int64_t)ri * ksr + 8 * half;
+    const uint16_t *vr = V + (int64_t)b * vsb + (int64_t)ri * vsr + 8 * half;
+#pragma unroll
+    for (int ks = 0; ks < NK; ++ks) {
+      kf[ks] = load_row_chunk(kr + 16 * ks, K, r_ok);
+      vf[ks] = load_row_chunk(vr + 16 * ks, V, r_ok);
+    }
+  }
+  wait_vmcnt<0>();
+  __syncthreads();
+
+  {
+    float d = 0.0f;
+#pragma unroll
+    for (int ks = 0; ks < NK; ++ks) d += dot8<T>(own_rows(tile_b, own_first, row_at, ks), o_own[ks]);
+    d = halves_sum(d);
+    if (half == 0) stat[0][own_first + r32] = d, stat[1][own_first + r32] = l_own;
+  }
+  if (wave == 0 || wave == 3) {
+    float d = 0.0f;
+#pragma unroll
+    for (int ks = 0; ks < NK; ++ks) d += dot8<T>(own_rows(tile_b, halo_first, halo_at, ks), o_halo[ks]);
+    d = halves_sum(d);
+    if (half == 0 && r32 < PADW) stat[0][halo_first + r32] = d, stat[1][halo_first + r32] = l_halo;
+  }
+  __syncthreads();
+
+  f32x16 dk[NB], dv[NB];
+  if (want_kv) {
+#pragma unroll
+    for (int hb = 0; hb < NB; ++hb)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) dk[hb][v] = 0.0f, dv[hb][v] = 0.0f;
+#pragma unroll
+    for (int j = 0; j < NKB; ++j) {
+      const int rb = wave + j;          // 32-row block of the tiles
+      const int r0 = t0 + 32 * rb;      // its first sequence row
+      if (r0 + 31 < rw0 - w || r0 > rw0 + 31 + w || r0 >= M || r0 + 31 < 0) continue;  // scalar
+      f32x16 s, dp;
+#pragma unroll
+      for (int v = 0; v < 16; ++v) s[v] = 0.0f, dp[v] = 0.0f;
+      u32x4 qa[NK], ga[NK];
+#pragma unroll
+      for (int ks = 0; ks < NK; ++ks) qa[ks] = TL::rows(tile_a, row_at, rb, ks), ga[ks] = TL::rows(tile_b, row_at, rb, ks);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int ks = 0; ks < NK; ++ks) {
+        s = Mma<T>::run(qa[ks], kf[ks], s);
+        dp = Mma<T>::run(ga[ks], vf[ks], dp);
+      }
+      {
+        // accumulator v of this lane: query r0 + 4 half + 8 (v / 4) + v % 4, key ri
+        const int d0 = r0 + 4 * half - ri;  // query - key at offset 0; valid offsets: first..last
+        const int first = max(-w - d0, -(r0 + 4 * half)), last = min(w - d0, M - 1 - r0 - 4 * half);
+        const int origin = last < first ? 0x100000 : first;
+        const unsigned span = last < first ? 0u : (unsigned)(last - first);
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          const int ofs = 8 * (v / 4) + v % 4;
+          s[v] = (unsigned)(ofs - origin) <= span ? s[v] : ninf;
+        }
+      }
+      // by halves of the block (16 query rows each): the operands of the second products and the row
+      // statistics of a half are read when its turn comes, which keeps three workgroups on a CU
+#pragma unroll
+      for (int t = 0; t < 2; ++t) {
+        u32x4 gc[NB], qc[NB];
+#pragma unroll
+        for (int hb = 0; hb < NB; ++hb)
+          gc[hb] = TL::cols(tile_b, tr_at, 32 * rb + 16 * t, hb), qc[hb] = TL::cols(tile_a, tr_at, 32 * rb + 16 * t, hb);
+        float p[8], ds[8];
+#pragma unroll
+        for (int g = 0; g < 2; ++g) {
+          const f32x4 dl = *reinterpret_cast<const f32x4 *>(&stat[0][32 * rb + 16 * t + 8 * g + 4 * half]);
+          const f32x4 l2 = *reinterpret_cast<const f32x4 *>(&stat[1][32 * rb + 16 * t + 8 * g + 4 * half]);
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            const int v = 8 * t + 4 * g + r;
+            p[4 * g + r] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[v], c, -l2[r]));
+            ds[4 * g + r] = p[4 * g + r] * (dp[v] - dl[r]);
+          }
+        }
+        const u32x4 pf = pack8<T>(p), dsf = pack8<T>(ds);
+#pragma unroll
+        for (int hb = 0; hb < NB; ++hb) {
+          dv[hb] = Mma<T>::run(gc[hb], pf, dv[hb]);
+          dk[hb] = Mma<T>::run(qc[hb], dsf, dk[hb]);
+        }
+      }
+    }
+  }
+  // own rows as queries: B operands of the other side, taken from the tiles before they go
+  u32x4 qf[NK], gf[NK];
+  float delta = 0.0f, lse2 = 0.0f;
+  if (dQ != nullptr) {
+#pragma unroll
+    for (int ks = 0; ks < NK; ++ks) qf[ks] = own_rows(tile_a, own_first, row_at, ks), gf[ks] = own_rows(tile_b, own_first, row_at, ks);
+    delta = stat[0][own_first + r32], lse2 = stat[1][own_first + r32];
+  }
+  __syncthreads();  // nobody reads the tiles any more
+  // K replaces Q while dK and dV leave through the other tile; V follows when those rows are out
+  if (dQ != nullptr) request(K + (int64_t)b * ksb, ksr, tile_a);
+  uint16_t *stage_rows = tile_b + wave * RowStage<NB>::ELEMS;
+  if (dK != nullptr) store_wave_rows<T, NB>(stage_rows, dk, scale, dK + (int64_t)b * dksb, dksr, rw0, M, N, lane);
+  if (dV != nullptr) store_wave_rows<T, NB>(stage_rows, dv, 1.0f, dV + (int64_t)b * dvsb, dvsr, rw0, M, N, lane);
+  if (dQ == nullptr) return;
+  __syncthreads();
+  request(V + (int64_t)b * vsb, vsr, tile_b);
+  f32x16 dq[NB];
+#pragma unroll
+  for (int hb = 0; hb < NB; ++hb)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) dq[hb][v] = 0.0f;
+  wait_vmcnt<0>();
+  __syncthreads();
+#pragma unroll
+  for (int j = 0; j < NKB; ++j) {
+    const int rb = wave + j;
+    const int c0 = t0 + 32 * rb;  // first key of the block
+    if (c0 + 31 < rw0 - w || c0 > rw0 + 31 + w || c0 >= M || c0 + 31 < 0) continue;  // scalar
+    f32x16 s, dp;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) s[v] = 0.0f, dp[v] = 0.0f;
+    u32x4 ka[NK], va[NK];
+#pragma unroll
+    for (int ks = 0; ks < NK; ++ks) ka[ks] = TL::rows(tile_a, row_at, rb, ks), va[ks] = TL::rows(tile_b, row_at, rb, ks);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int ks = 0; ks < NK; ++ks) {
+      s = Mma<T>::run(ka[ks], qf[ks], s);
+      dp = Mma<T>::run(va[ks], gf[ks], dp);
+    }
+    u32x4 kc[2][NB];
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int hb = 0; hb < NB; ++hb) kc[t][hb] = TL::cols(tile_a, tr_at, 32 * rb + 16 * t, hb);
+    __builtin_amdgcn_sched_barrier(0);
+    {
+      // accumulator v of this lane: key c0 + 4 half + 8 (v / 4) + v % 4, query ri
+      const int d0 = c0 + 4 * half - ri;
+      const int first = max(-w - d0, -(c0 + 4 * half)), last = min(w - d0, M - 1 - c0 - 4 * half);
+      const int origin = last < first ? 0x100000 : first;
+      const unsigned span = last < first ? 0u : (unsigned)(last - first);
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int ofs = 8 * (v / 4) + v % 4;
+        s[v] = (unsigned)(ofs - origin) <= span ? s[v] : ninf;
+      }
+    }
+    float ds[16];
+#pragma unroll
+    for (int v = 0; v < 16; ++v) ds[v] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[v], c, -lse2)) * (dp[v] - delta);
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      const u32x4 dsf = pack8<T>(ds + 8 * t);
+#pragma unroll
+      for (int hb = 0; hb < NB; ++hb) dq[hb] = Mma<T>::run(kc[t][hb], dsf, dq[hb]);
+    }
+  }
+  __syncthreads();
+  store_wave_rows<T, NB>(tile_a + wave * RowStage<NB>::ELEMS, dq, scale, dQ + (int64_t)b * dqsb, dqsr, rw0, M, N, lane);
+}
+
 template <typename T, int NK>
 hipError_t launch_backward(const Problem &p, const View &q, const View &k, const View &v, const View &o,
                            const View &go, const float *lse, float *delta, const View &gq, const View &gk,
@@ -774,6 +1039,22 @@ hipError_t launch_backward(const Problem &p, const View &q, const View &k, const
     const int64_t lim = 0x7fffffff;
     bool fits = !(p.flags & WM_FLAG_NO_LDS_DIRECT) && (p.M + 3 * AB_KC) * 4 < lim;
     for (const View *t : {&q, &k, &v, &go}) fits = fits && t->sr > 0 && (p.M + 3 * AB_KC) * t->sr * 2 < lim;
+    if constexpr (NK <= 4) {
+      // narrow windows: one kernel for all three gradients (two row blocks per wavefront up to w = 16, three up to 32)
+      if (fits && p.w <= 32 && !(p.flags & WM_FLAG_NO_NARROW_BAND)) {
+#define WM_ABN(NKB)                                                                                                   \
+  hipLaunchKernelGGL((attention_backward_narrow_kernel<T, NK, NKB>), grid, block, 0, p.stream, (in_t)q.data,          \
+                     (in_t)k.data, (in_t)v.data, (in_t)o.data, (in_t)go.data, lse, (out_t)gq.data, (out_t)gk.data,    \
+                     (out_t)gv.data, (int)p.B, (int)p.M, (int)p.w, nblk, (float)scale, q.sb, q.sr, k.sb, k.sr, v.sb,  \
+                     v.sr, o.sb, o.sr, go.sb, go.sr, gq.sb, gq.sr, gk.sb, gk.sr, gv.sb, gv.sr)
+        if (p.w <= 16)
+          WM_ABN(2);
+        else
+          WM_ABN(3);
+#undef WM_ABN
+        return hipGetLastError();
+      }
+    }
     if (fits) {
       if (gq.data != nullptr)
         hipLaunchKernelGGL((attention_backward_query_dma_kernel<T, NK>), grid, block, 0, p.stream, (in_t)q.data,

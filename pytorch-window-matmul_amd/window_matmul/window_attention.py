@@ -21,12 +21,14 @@ from .window_matmul import unwindow_matmul, window_matmul
 
 def _chain_is_faster(window_size: int, width: int) -> bool:
     """Windows at which a training step is faster through the separate ops than through the fused
-    kernels, whose recomputing backward costs the same at every narrow window.  Measured on bf16
-    tensors of 100 M elements with M = 16384 (chain / fused, ms per step): N = 32: 0.32 / 0.33 at
-    w = 4, 0.34 / 0.34 at w = 8; N = 64: 0.58 / 0.66 at w = 12, 0.72 / 0.67 at w = 14; N = 96:
-    0.81 / 0.86 at w = 32, 0.96 / 0.92 at w = 40; N = 128: 0.72 / 0.79 at w = 32, 0.86 / 0.84 at
-    w = 40."""
-    return window_size <= (4 if width <= 32 else 13 if width <= 64 else 36)
+    kernels.  Up to N = 64 the fused backward is one kernel at windows up to 32 and the chain only wins
+    at the very narrowest windows of the narrow heads; above N = 64 the recomputing two-kernel backward
+    costs the same at every narrow window.  Measured on bf16 tensors of 100 M elements with M = 16384
+    (chain / fused, ms per step): N = 16: 0.67 / 0.69 at w = 2, 0.72 / 0.72 at w = 3; N = 32: 0.48 /
+    0.48 at w = 2, 0.50 / 0.48 at w = 3; N = 48: 0.51 / 0.46 at w = 1; N = 64: 0.47 / 0.47 at w = 1,
+    0.48 / 0.45 at w = 2, 0.52 / 0.44 at w = 8, 0.88 / 0.52 at w = 32; N = 96: 0.81 / 0.86 at w = 32,
+    0.96 / 0.92 at w = 40; N = 128: 0.72 / 0.79 at w = 32, 0.86 / 0.84 at w = 40."""
+    return window_size <= (2 if width <= 32 else 0 if width <= 64 else 36)
 
 
 class WindowAttentionFunc(torch.autograd.Function):

@@ -260,20 +260,55 @@ def _graph_nodes(t):
 
 
 def test_narrow_window_training_goes_through_the_separate_ops(device):
-    """Same values either way; the choice only shows in which autograd nodes produced the result."""
+    """Same values either way; the choice only shows in which autograd nodes produced the result.
+    Heads up to 64 wide have a one-kernel backward at narrow windows and stay fused (but for the very
+    narrowest windows of heads up to 32 wide); wider heads train through the separate ops up to w = 36."""
     from window_matmul import window_attention
 
-    q, k, v, go = (seeded((2, 200, 64), s, torch.bfloat16).to(device) for s in (131, 132, 133, 134))
-    with torch.no_grad():
-        want = window_attention(q, k, v, 8)          # fused one-pass forward
-    qq, kk, vv = (t.clone().requires_grad_(True) for t in (q, k, v))
-    out = window_attention(qq, kk, vv, 8)             # separate ops (w <= 14 and gradients wanted)
-    assert "UnwindowMatmulFuncBackward" in _graph_nodes(out)
-    torch.testing.assert_close(out.float(), want.float(), **TOL)
-    out.backward(go)
-    want_g = ao.window_attention_backward(q.cpu(), k.cpu(), v.cpu(), 8, go.cpu(), 1.0 / math.sqrt(64))
-    for x, y in zip((qq.grad, kk.grad, vv.grad), want_g):
-        close(x, y)
-    assert "UnwindowMatmulFuncBackward" in _graph_nodes(window_attention(qq, kk, vv, 12))
-    for w in (16, 20):  # the fused kernels win there
-        assert "WindowAttentionFuncBackward" in _graph_nodes(window_attention(qq, kk, vv, w))
+    for N, w_chain, w_fused in ((96, (8, 36), (40,)), (32, (1, 2), (3, 8, 20)), (64, (), (1, 8, 12, 16, 20))):
+        q, k, v, go = (seeded((2, 200, N), s, torch.bfloat16).to(device) for s in (131, 132, 133, 134))
+        for w in w_chain + w_fused:
+            with torch.no_grad():
+                want = window_attention(q, k, v, w)      # fused forward (one pass up to w = 16 / 32)
+            qq, kk, vv = (t.clone().requires_grad_(True) for t in (q, k, v))
+            out = window_attention(qq, kk, vv, w)
+            nodes = _graph_nodes(out)
+            assert ("UnwindowMatmulFuncBackward" in nodes) == (w in w_chain), (N, w)
+            assert ("WindowAttentionFuncBackward" in nodes) == (w in w_fused), (N, w)
+            torch.testing.assert_close(out.float(), want.float(), **TOL)
+            out.backward(go)
+            want_g = ao.window_attention_backward(q.cpu(), k.cpu(), v.cpu(), w, go.cpu(), 1.0 / math.sqrt(N))
+            for x, y in zip((qq.grad, kk.grad, vv.grad), want_g):
+                close(x, y)
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=lambda d: str(d).split(".")[-1])
+@pytest.mark.parametrize("case", [(3, 700, 64, 3), (2, 130, 64, 16), (2, 1000, 64, 17), (5, 300, 64, 32), (4, 257, 48, 8),
+                                  (3, 400, 32, 31), (6, 129, 16, 5), (2, 9, 64, 12), (1, 128, 64, 1), (2, 255, 32, 16)],
+                         ids=lambda c: "B%d_M%d_N%d_w%d" % c)
+def test_one_kernel_and_two_kernel_backward_agree(device, case, dtype):
+    """Heads up to 64 wide, windows up to 32: one kernel computes all three gradients (a workgroup owns
+    128 rows as keys and as queries); WM_FLAG_NO_NARROW_BAND forces the two-kernel backward.  Both
+    against the oracle, both ways of asking for part of the gradients, strided (head-major) operands,
+    and twice for the same bits."""
+    B, M, N, w = case
+    scale = 1.0 / math.sqrt(N)
+    big = [seeded((M, B * N), s, dtype) for s in (141, 142, 143, 144)]
+    q, k, v, go = (t.view(M, B, N).transpose(0, 1) for t in big)  # (B, M, N) views, row stride B * N
+    for mask in (False, True):
+        want = ao.window_attention_backward(q, k, v, w, go, scale, mask)
+        qd, kd, vd, gd = (t.to(device).view(M, B, N).transpose(0, 1) for t in big)
+        assert not qd.is_contiguous() or B == 1
+        o, lse = abi.attention_forward(qd, kd, vd, w, scale, mask)
+        one = abi.attention_backward(qd, kd, vd, o, lse, gd, w, scale)
+        two = abi.attention_backward(qd, kd, vd, o, lse, gd, w, scale, flags=abi.NO_NARROW_BAND)
+        for x, y, z in zip(one, want, two):
+            close(x, y)
+            close(z, y)
+            torch.testing.assert_close(x.float(), z.float(), rtol=2e-2, atol=2e-2)
+        for part in ((True, False, False), (False, True, True), (False, True, False)):
+            some = abi.attention_backward(qd, kd, vd, o, lse, gd, w, scale, want=part)
+            for wanted, x, y in zip(part, some, one):
+                assert (x is None) == (not wanted)
+                if wanted:
+                    assert torch.equal(x, y)
