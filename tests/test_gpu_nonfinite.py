@@ -112,3 +112,32 @@ def test_fused_attention_poisoned_value_row(device, w, dtype):
     same = rows_equal(clean, dirty)
     assert bool(same[dist > reach(w)].all())
     assert bool(torch.isnan(dirty[0, :, 7].cpu().float())[dist <= w].all())
+
+
+@pytest.mark.parametrize("which", ["v", "grad_o"])
+@pytest.mark.parametrize("w", [8, 32, 64, 256])
+def test_fused_attention_backward_poisoned_row(device, w, which):
+    """The fused backward (one kernel up to w = 32 at this head width, two kernels above) under the same
+    rule: a NaN in one row of v or of the upstream gradient changes no gradient row farther than
+    REACH(w) from it, and the rows the chain would poison are non-finite here too."""
+    dtype = torch.bfloat16
+    q, k, v, go = (seeded((1, M, N), 95 + s, dtype).to(device) for s in range(4))
+    scale = 1.0 / math.sqrt(N)
+    o, lse = abi.attention_forward(q, k, v, w, scale)
+    clean = abi.attention_backward(q, k, v, o, lse, go, w, scale)
+    vp, gp = v.clone(), go.clone()
+    (vp if which == "v" else gp)[0, ROW, 7] = float("nan")
+    dirty = abi.attention_backward(q, k, vp, o, lse, gp, w, scale)
+    dist = (torch.arange(M) - ROW).abs()
+    for name, c, d in zip(("grad_q", "grad_k", "grad_v"), clean, dirty):
+        same = rows_equal(c, d)
+        assert bool(same[dist > reach(w)].all()), f"{name}: a row more than {reach(w)} rows from the poisoned one changed"
+    gq, gk, gv = dirty
+    if which == "v":
+        # dP[i, ROW] = grad_o_i . v_ROW is NaN for every query i in the window of key ROW: grad_q_i and grad_k_ROW
+        assert bool(torch.isnan(gq[0].float()).any(dim=-1).cpu()[dist <= w].all())
+        assert bool(torch.isnan(gk[0, ROW].float()).any())
+    else:
+        # grad_v_c takes P[ROW, c] * grad_o_ROW for every key c in the window of query ROW
+        assert bool(torch.isnan(gv[0, :, 7].float()).cpu()[dist <= w].all())
+        assert bool(torch.isnan(gq[0, ROW].float()).any())
