@@ -34,7 +34,7 @@
 extern "C" {
 #endif
 
-#define WM_ABI_VERSION 3
+#define WM_ABI_VERSION 4
 
 typedef enum wm_dtype {
   WM_DTYPE_F32 = 0,
@@ -195,6 +195,16 @@ int wm_window_attention_backward_static(const wm_operand *q, const wm_operand *k
                                         const wm_operand *grad_q, const wm_operand *grad_k,
                                         const wm_operand *grad_v, int64_t B, int64_t M, int64_t N, int64_t w,
                                         double scale, int dtype, unsigned flags, void *stream);
+
+/* Keys that arrive as a (B, N, M) tensor with unit stride along M (the layout of the reference's
+ * `other` argument when it is contiguous) copied into key rows, a contiguous (B, M, N) buffer
+ * `rows`, which is what the kernels above consume in place as k with strides {M*N, 1, N}.  It
+ * replaces the copy the reference makes on entry (`B.transpose(-1, -2).contiguous()`, reference
+ * cuda/window_matmul_cuda.cu:236, 285) and runs at memory speed (one read and one write of the
+ * tensor).  Callers that hold key rows already (key.transpose(-1, -2) of a row-major tensor) skip it.
+ * WM_ERR_UNSUPPORTED, nothing launched, unless k has unit column stride, rows is 16-byte aligned
+ * and N is a multiple of 16 bytes (any M, any row stride). */
+int wm_key_rows(const wm_operand *k, void *rows, int64_t B, int64_t N, int64_t M, int dtype, void *stream);
 
 /* 1 if the fused kernels exist for this shape, dtype and scale (layout aside), else 0. */
 int wm_window_attention_supported(int64_t M, int64_t N, int64_t w, int dtype, double scale);

@@ -100,11 +100,6 @@ bool sliced_width(const torch::Tensor &t) {
   return t.size(2) > kMaxWidth && (t.scalar_type() == at::kHalf || t.scalar_type() == at::kBFloat16 || t.scalar_type() == at::kFloat);
 }
 
-// K comes as (B,N,M).  The kernels want key rows contiguous, which is what a
-// transposed view of a row-major (B,M,N) tensor already is; anything else is
-// copied into that layout once (the reference always copies: cuda:236).
-torch::Tensor key_rows(const torch::Tensor &k) { return vector_friendly(k.transpose(1, 2)); }
-
 wm_operand operand(const torch::Tensor &t) {
   return wm_operand{t.data_ptr(), t.stride(0), t.stride(1), t.stride(2)};
 }
@@ -116,6 +111,27 @@ void raise_on_error(int status, const char *op) {
 void *current_stream(const torch::Tensor &t) {
   return c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(t.device().index()).stream();
 }
+
+// K comes as (B,N,M).  The kernels want key rows contiguous, which is what a
+// transposed view of a row-major (B,M,N) tensor already is; anything else is
+// copied into that layout once (the reference always copies: cuda:236).
+// A tensor that is laid out as (B,N,M) with unit stride along M goes through the library's own
+// transpose (one read and one write at memory speed; a general strided copy reaches a quarter of that).
+torch::Tensor key_rows(const torch::Tensor &k) {
+  auto view = k.transpose(1, 2);
+  if (view.stride(2) == 1 || k.stride(2) != 1 || k.numel() == 0 || !k.is_cuda()) return vector_friendly(view);
+  const int64_t es = k.element_size();
+  if (es != 2 && es != 4 && es != 8) return vector_friendly(view);
+  auto rows = torch::empty({k.size(0), k.size(2), k.size(1)}, k.options());
+  const wm_operand src{k.data_ptr(), k.stride(0), k.stride(1), k.stride(2)};
+  const int dtype = es == 2 ? WM_DTYPE_BF16 : es == 4 ? WM_DTYPE_F32 : WM_DTYPE_F64;  // only the element size matters
+  const int status = wm_key_rows(&src, rows.data_ptr(), k.size(0), k.size(1), k.size(2), dtype,
+                                 current_stream(k));
+  if (status == WM_ERR_UNSUPPORTED) return vector_friendly(view);  // odd alignment: the general copy
+  raise_on_error(status, "key rows");
+  return rows;
+}
+
 
 void check_window_inputs(const torch::Tensor &src, const torch::Tensor &other) {
   check_gpu(src, "A");

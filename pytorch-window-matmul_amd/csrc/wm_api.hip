@@ -220,6 +220,17 @@ int wm_window_attention_backward_static(const wm_operand *q, const wm_operand *k
                                       flags, stream);
 }
 
+int wm_key_rows(const wm_operand *k, void *rows, int64_t B, int64_t N, int64_t M, int dtype, void *stream) {
+  if (int st = check_common(B, M, N, 0, dtype, 0)) return st;
+  if (missing(k) || rows == nullptr) return WM_ERR_NULL_POINTER;
+  if (k->stride_c != 1) return WM_ERR_UNSUPPORTED;
+  hipError_t err = hipSuccess;
+  if (!try_launch_transpose(k->data, rows, B, N, M, k->stride_b, k->stride_r, (int)dtype_size(dtype),
+                            static_cast<hipStream_t>(stream), &err))
+    return WM_ERR_UNSUPPORTED;
+  return to_status(err);
+}
+
 int wm_window_attention_supported(int64_t M, int64_t N, int64_t w, int dtype, double scale) {
   return attention_supports(M, N, w, dtype, scale) ? 1 : 0;
 }

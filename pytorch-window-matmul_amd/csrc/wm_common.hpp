@@ -85,6 +85,12 @@ bool try_launch_attention_backward(const Problem &p, const View &q, const View &
                                    const View &go, const float *lse, float *delta, const View &gq, const View &gk,
                                    const View &gv, double scale, hipError_t *err);
 
+// Batched transpose of the last two dimensions (wm_transpose.hip): src (B,R,C) with unit column stride and
+// batch / row strides ssb / ssr (elements), dst contiguous (B,C,R).  Returns false, nothing launched,
+// unless dst is 16-byte aligned, R is a multiple of 16 bytes and elem_size is 2, 4 or 8.
+bool try_launch_transpose(const void *src, void *dst, int64_t B, int64_t R, int64_t C, int64_t ssb, int64_t ssr,
+                          int elem_size, hipStream_t stream, hipError_t *err);
+
 inline size_t dtype_size(int dtype) {
   switch (dtype) {
     case WM_DTYPE_F32: return 4;

@@ -68,6 +68,7 @@ def lib():
         L.wm_window_attention_backward_static.argtypes = [P, P, P, P, vp, P, P, P, P, i64, i64, i64, i64,
                                                           ctypes.c_double, ctypes.c_int, u32, vp]
         L.wm_window_attention_supported.argtypes = [i64, i64, i64, ctypes.c_int, ctypes.c_double]
+        L.wm_key_rows.argtypes = [P, vp, i64, i64, i64, ctypes.c_int, vp]
         _LIB = L
     return _LIB
 
@@ -96,6 +97,14 @@ def window_forward(q, k, w, flags=0, out=None):
     _check(lib().wm_window_matmul_forward(op(q), op(k), op(a), B, M, N, w, DTYPES[q.dtype], flags, _stream()),
            "wm_window_matmul_forward")
     return a
+
+
+def key_rows(k):
+    """wm_key_rows: k (B,N,M) with unit stride along M -> contiguous key rows (B,M,N)."""
+    B, N, M = k.shape
+    rows = torch.empty(B, M, N, dtype=k.dtype, device=k.device)
+    _check(lib().wm_key_rows(op(k), ctypes.c_void_p(rows.data_ptr()), B, N, M, DTYPES[k.dtype], _stream()), "wm_key_rows")
+    return rows
 
 
 def window_backward(q, k, w, ga, flags=0, want_q=True, want_k=True):

@@ -18,10 +18,10 @@ def test_library_exports_every_declared_symbol():
             "wm_unwindow_matmul_backward", "wm_band_softmax_forward", "wm_band_softmax_backward",
             "wm_band_softmax_kernel_choice", "wm_window_attention_forward", "wm_window_attention_backward",
             "wm_window_attention_supported", "wm_window_attention_backward_static",
-            "wm_kernel_choice", "wm_status_string", "wm_abi_version"} <= set(names)
+            "wm_kernel_choice", "wm_key_rows", "wm_status_string", "wm_abi_version"} <= set(names)
     for name in names:
         assert hasattr(L, name), name
-    assert L.wm_abi_version() == 3
+    assert L.wm_abi_version() == 4
 
 
 def test_argument_validation_happens_on_the_host():

@@ -3,6 +3,7 @@ their autograd Functions), in the manner of the reference's own tests: the custo
 against an independent torch formulation, outputs and input gradients
 (reference tests/test_window_matmul.py:53-84, tests/test_unwindow_matmul.py:40-79,
 tests/test_attention.py:90-140)."""
+import ctypes
 import itertools
 import math
 
@@ -290,3 +291,43 @@ def test_head_widths_between_the_tuned_ones(device, dtype, N, w):
     torch.testing.assert_close(f(dk.grad).cpu(), want_k.transpose(1, 2), **tol)
     torch.testing.assert_close(f(da.grad).cpu(), want_a, **tol)
     torch.testing.assert_close(f(dv.grad).cpu(), want_v, **tol)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32, torch.float64],
+                         ids=lambda d: str(d).split(".")[-1])
+def test_key_rows_from_contiguous_transposed_keys(device, dtype):
+    """Keys given as a contiguous (B,N,M) tensor (reference window_matmul.py:30-40 takes exactly that
+    shape) are copied into key rows by the library's own transpose: bit-exact against torch's copy at
+    ragged and tile-sized shapes, with a row stride, and the ops on top of it give the same bits as with
+    keys that were row-major all along.  Layouts it does not take report WM_ERR_UNSUPPORTED."""
+    import wm_ctypes as abi
+    from window_matmul import window_matmul
+
+    for B, N, M in ((3, 64, 300), (2, 128, 64), (5, 16, 1), (1, 80, 4097), (2, 8, 129), (7, 48, 1000), (2, 64, 3001)):
+        kt = seeded((B, N, M), 201, dtype).to(device)
+        assert torch.equal(abi.key_rows(kt), kt.transpose(1, 2).contiguous())
+        for off in (8, 3):  # rows that start on a 16-byte boundary, and rows that do not
+            view = seeded((B, N, M + 24), 202, dtype).to(device)[:, :, off:off + M]
+            assert torch.equal(abi.key_rows(view), view.transpose(1, 2).contiguous())
+    # through the Python API: same bits as with row-major keys, forward and both gradients
+    B, M, N, w = 3, 333, 64, 21
+    q = seeded((B, M, N), 203, dtype).to(device).requires_grad_(True)
+    k_rows = seeded((B, M, N), 204, dtype).to(device)
+    kt = k_rows.transpose(1, 2).contiguous().requires_grad_(True)      # contiguous (B,N,M)
+    kv = k_rows.clone().requires_grad_(True)
+    ga = seeded((B, M, 2 * w + 1), 205, dtype).to(device)
+    a1 = window_matmul(q, kt, w)
+    a1.backward(ga)
+    g1 = (q.grad.clone(), kt.grad.clone())
+    q.grad = None
+    a2 = window_matmul(q, kv.transpose(1, 2), w)
+    a2.backward(ga)
+    assert torch.equal(a1, a2) and torch.equal(g1[0], q.grad) and torch.equal(g1[1], kv.grad.transpose(1, 2))
+    # not taken: a head width whose rows cannot be 16-byte pieces, keys whose unit stride is not along M
+    L = abi.lib()
+    thin = seeded((2, 3, 64), 207, dtype).to(device)
+    out = torch.empty(2, 64, 3, dtype=dtype, device=device)
+    assert L.wm_key_rows(abi.op(thin), ctypes.c_void_p(out.data_ptr()), 2, 3, 64, abi.DTYPES[dtype], None) == 7
+    rows = seeded((2, 64, 64), 208, dtype).to(device).transpose(1, 2)
+    out = torch.empty(2, 64, 64, dtype=dtype, device=device)
+    assert L.wm_key_rows(abi.op(rows), ctypes.c_void_p(out.data_ptr()), 2, 64, 64, abi.DTYPES[dtype], None) == 7
