@@ -383,9 +383,10 @@ __global__ __launch_bounds__(kThreads, NK <= 4 ? 2 : 1) void attention_backward_
 // (wm_attention.hip): swizzled tiles filled by buffer loads with the lds modifier, requested DEPTH
 // chunks ahead and counted by the kernel itself; scalar control flow; one branch-free loop for the
 // chunks that lie wholly inside a wavefront's band and a general one for the chunks at its edges.
-// The workspace holds two float32 values per row: D = sum_h dO * O at [b * M + i] and the row's
-// log-sum-exp in log2 units at [B * M + b * M + i]; the query kernel writes both, the key kernel
-// streams both.  dS is formed without the factor `scale`, which multiplies the finished dQ and dK.
+// The workspace holds two float32 values per row: -D = -sum_h dO * O at [b * M + i] (negated: the dP
+// accumulators of the key kernel start from it) and the row's log-sum-exp in log2 units at
+// [B * M + b * M + i]; the query kernel writes both, the key kernel streams both.  dS is formed
+// without the factor `scale`, which multiplies the finished dQ and dK.
 constexpr float kLog2e = 1.4426950408889634f;
 
 template <int NK>
@@ -441,7 +442,7 @@ __global__ __launch_bounds__(kThreads) void attention_backward_stats_kernel(
     delta += dot8<T>(load_row_chunk(gr + 16 * ks, dO, q_ok), load_row_chunk(orow + 16 * ks, O, q_ok));
   delta = halves_sum(delta);
   if (q_ok && half == 0) {
-    D[(int64_t)b * M + qi] = delta;
+    D[(int64_t)b * M + qi] = -delta;
     D[((int64_t)B + b) * M + qi] = L[(int64_t)b * M + qi] * kLog2e;
   }
 }
@@ -501,7 +502,7 @@ __global__ __launch_bounds__(kThreads, NK <= 4 ? 3 : 2) void attention_backward_
   delta = halves_sum(delta);
   const float l2 = (q_ok ? L[(int64_t)b * M + qi] : 0.0f) * kLog2e;
   if (q_ok && half == 0) {
-    D[(int64_t)b * M + qi] = delta;
+    D[(int64_t)b * M + qi] = -delta;  // the key kernel's dP accumulators start from it
     D[((int64_t)B + b) * M + qi] = l2;
   }
 
@@ -610,7 +611,7 @@ __global__ __launch_bounds__(kThreads, NK <= 4 ? 2 : 1) void attention_backward_
   constexpr int LOADS = 2 * (PPR / 4) + 1;  // loads per wavefront and chunk: Q, dO and one row statistic
   __shared__ __attribute__((aligned(1024))) uint16_t q_lds[STAGES][TILE];
   __shared__ __attribute__((aligned(1024))) uint16_t g_lds[STAGES][TILE];
-  __shared__ __attribute__((aligned(256))) float stat_lds[STAGES][2][AB_KC];  // [0] D, [1] log-sum-exp (log2 units)
+  __shared__ __attribute__((aligned(256))) float stat_lds[STAGES][2][AB_KC];  // [0] -D, [1] log-sum-exp (log2 units)
 
   int b, blk;
   if (!decode_block(nblk, B, &b, &blk)) return;
@@ -667,14 +668,16 @@ __global__ __launch_bounds__(kThreads, NK <= 4 ? 2 : 1) void attention_backward_
     constexpr bool EDGE = decltype(edge)::value;
     f32x16 s, dp;
 #pragma unroll
-    for (int v = 0; v < 16; ++v) s[v] = 0.0f, dp[v] = 0.0f;
+    for (int v = 0; v < 16; ++v) s[v] = 0.0f;
     u32x4 qa[NK], ga[NK];
-    f32x4 dl[4], l2[4];
+    f32x4 l2[4];
 #pragma unroll
     for (int ks = 0; ks < NK; ++ks) qa[ks] = TL::rows(qt, row_at, qb, ks), ga[ks] = TL::rows(gt, row_at, qb, ks);
 #pragma unroll
     for (int g = 0; g < 4; ++g) {
-      dl[g] = *reinterpret_cast<const f32x4 *>(st + 32 * qb + 8 * g + 4 * half);
+      // the dP accumulator starts from -D of its sixteen queries: dP - D comes out of the matrix pipe
+      const f32x4 nd = *reinterpret_cast<const f32x4 *>(st + 32 * qb + 8 * g + 4 * half);
+      dp[4 * g] = nd[0], dp[4 * g + 1] = nd[1], dp[4 * g + 2] = nd[2], dp[4 * g + 3] = nd[3];
       l2[g] = *reinterpret_cast<const f32x4 *>(st + AB_KC + 32 * qb + 8 * g + 4 * half);
     }
     __builtin_amdgcn_sched_barrier(0);
@@ -708,7 +711,7 @@ __global__ __launch_bounds__(kThreads, NK <= 4 ? 2 : 1) void attention_backward_
       for (int r = 0; r < 4; ++r) {
         const int v = 4 * g + r;
         p[v] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[v], c, -l2[g][r]));
-        ds[v] = p[v] * (dp[v] - dl[g][r]);
+        ds[v] = p[v] * dp[v];
       }
 #pragma unroll
     for (int t = 0; t < 2; ++t) {
