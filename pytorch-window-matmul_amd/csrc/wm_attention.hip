@@ -395,19 +395,19 @@ __global__ __launch_bounds__(kThreads, 2) void attention_forward_narrow_kernel(
 //     the exponentials of one block run on the vector ALU while the matrix pipe multiplies the
 //     other block's probabilities with V.
 template <typename T, int NK, bool MASK>
-__global__ __launch_bounds__(kThreads, NK <= 4 ? 3 : 2) void attention_forward_dma_kernel(
+__global__ __launch_bounds__(kThreads, NK <= 4 ? 4 : 2) void attention_forward_dma_kernel(
     const uint16_t *__restrict__ Q, const uint16_t *__restrict__ K, const uint16_t *__restrict__ V,
     uint16_t *__restrict__ O, float *__restrict__ L, int B, int M, int w, int nblk, float c, int64_t qsb, int64_t qsr,
     int64_t ksb, int64_t ksr, int64_t vsb, int64_t vsr, int64_t osb, int64_t osr) {
   // tile rows of 128 bytes (N <= 64) or 256 bytes; the pieces of a row beyond column N are never
   // fetched (requested out of range: zeros, no memory traffic)
   constexpr int N = 16 * NK, NB = (NK + 1) / 2, ROWB = NK <= 4 ? 128 : 256, PPR = ROWB / 16;
-  constexpr int STAGES = NK <= 4 ? 3 : 2, DEPTH = STAGES - 1;
+  constexpr int STAGES = 2, DEPTH = STAGES - 1;
   constexpr int TILE = AT_KC * ROWB / 2;   // elements per tile
   constexpr int LOADS = 2 * (PPR / 4);     // loads per wavefront and chunk (K and V)
   static_assert(NK >= 1 && NK <= 8, "N = 16 ... 128");
-  __shared__ __attribute__((aligned(1024))) uint16_t k_lds[STAGES][TILE];
-  __shared__ __attribute__((aligned(1024))) uint16_t v_lds[STAGES][TILE];
+  __shared__ __attribute__((aligned(1024))) uint16_t kv_lds[2 * STAGES][TILE];  // key tiles, then value tiles
+  uint16_t (*const k_lds)[TILE] = kv_lds, (*const v_lds)[TILE] = kv_lds + STAGES;
 
   int b, blk;
   if (!decode_block(nblk, B, &b, &blk)) return;
@@ -587,30 +587,24 @@ __global__ __launch_bounds__(kThreads, NK <= 4 ? 3 : 2) void attention_forward_d
   for (; kc <= kc_hi; ++kc) edge_chunk(kc);
 
   float l = across_halves_sum(l_part);
+  float alpha = 1.0f;  // what the accumulated O still has to be scaled by (folded into the division by l)
   if (!MASK) {
-    // Band entries outside the sequence: score 0 each, no value row (scalar test first).
-    if (qw0 < w || qw0 + 31 + w > M - 1) {
-      const int n_out = max(0, w - qi) + max(0, qi + w - (M - 1));
-      if (n_out > 0) {
-        const float m_new = fmaxf(m_used, 0.0f);
-        const float alpha = __builtin_amdgcn_exp2f(m_used - m_new);
-        l = l * alpha + (float)n_out * __builtin_amdgcn_exp2f(-m_new);
-        m_used = m_new;
-#pragma unroll
-        for (int hb = 0; hb < NB; ++hb)
-#pragma unroll
-          for (int v = 0; v < 16; ++v) o[hb][v] *= alpha;
-      }
-    }
+    // Band entries outside the sequence: score 0 each, no value row.  Branch-free: a row without such
+    // entries keeps its maximum, alpha = 1 and adds 0 to the sum.
+    const int n_out = max(0, w - qi) + max(0, qi + w - (M - 1));
+    const float m_new = n_out > 0 ? fmaxf(m_used, 0.0f) : m_used;
+    alpha = __builtin_amdgcn_exp2f(m_used - m_new);
+    l = l * alpha + (float)n_out * __builtin_amdgcn_exp2f(-m_new);
+    m_used = m_new;
   }
   if (qi >= M) l = 1.0f;  // rows past the end: keep the arithmetic finite, nothing is stored
-  const float inv = 1.0f / l;
+  const float inv = alpha / l;
   if (L != nullptr && half == 0 && qi < M) L[(int64_t)b * M + qi] = (m_used + __builtin_amdgcn_logf(l)) * kLn2F;
   // The chunks requested past the last one must have landed before their tiles are reused, and
-  // every wavefront must be done with the last chunk: then the key tiles stage the result rows.
+  // every wavefront must be done with the last chunk: then the tiles stage the result rows.
   wait_vmcnt<0>();
   __builtin_amdgcn_s_barrier();
-  static_assert(4 * RowStage<NB>::ELEMS <= STAGES * TILE, "the four staging areas must fit the key tiles");
+  static_assert(4 * RowStage<NB>::ELEMS <= 2 * STAGES * TILE, "the four staging areas must fit the tiles");
   store_wave_rows<T, NB>(&k_lds[0][0] + wave * RowStage<NB>::ELEMS, o, inv, O + (int64_t)b * osb, osr, qw0, M, N, lane);
 }
 
