@@ -817,11 +817,17 @@ __global__ __launch_bounds__(kThreads, 3) void mfma_p1_dma_kernel(const uint16_t
 #ifndef WM_P3_DMA_KC
 #define WM_P3_DMA_KC 64
 #endif
+#ifndef WM_P3_SHALLOW_BELOW
+#define WM_P3_SHALLOW_BELOW 56
+#endif
+constexpr int kShallowChunksBelow = WM_P3_SHALLOW_BELOW;  // window sizes below this take the 32-row chunks
 #ifndef WM_P3_DMA_STAGES
 #define WM_P3_DMA_STAGES 2
 #endif
 template <typename T, int NK, int KCH, int STAGES>
-__global__ __launch_bounds__(kThreads, (160 * 1024 / (STAGES * KCH * (2 * TM + (NK <= 4 ? 128 : 256))) >= 3 ? 3 : 2)) void mfma_p3_dma_kernel(
+__global__ __launch_bounds__(kThreads, (160 * 1024 / (STAGES * KCH * (2 * TM + (NK <= 4 ? 128 : 256))) >= 4
+                                           ? 4
+                                           : 160 * 1024 / (STAGES * KCH * (2 * TM + (NK <= 4 ? 128 : 256))) >= 3 ? 3 : 2)) void mfma_p3_dma_kernel(
     const uint16_t *__restrict__ A, const uint16_t *__restrict__ Y, uint16_t *__restrict__ C, int B, int M, int w,
     int nblk, int galign, int64_t asb, int64_t ysb, int64_t ysr, int64_t csb, int64_t csr) {
   constexpr int N = 16 * NK, NT = (NK + 1) / 2, CH = KCH, DEPTH = STAGES - 1;
@@ -1132,14 +1138,25 @@ hipError_t launch_p3(const Problem &p, const View &a, const View &y, const View 
   if (const int g = lds_direct_group<ALIGNED>(p, a, y)) {
     const dim3 grid_g(grid_size(p.B, (p.M + g - 1 + TM - 1) / TM));
     const int nblk_g = (int)((p.M + g - 1 + TM - 1) / TM);
-#define WM_P3_DMA(NK)                                                                                          \
+#define WM_P3_DMA(NK, KCH, STAGES)                                                                             \
   case NK:                                                                                                     \
-    hipLaunchKernelGGL((mfma_p3_dma_kernel<T, NK, WM_P3_DMA_KC, WM_P3_DMA_STAGES>), grid_g, block, 0, p.stream, \
+    hipLaunchKernelGGL((mfma_p3_dma_kernel<T, NK, KCH, STAGES>), grid_g, block, 0, p.stream,                   \
                        (const uint16_t *)a.data, (const uint16_t *)y.data, (uint16_t *)c.data, (int)p.B,       \
                        (int)p.M, (int)p.w, nblk_g, g, a.sb, y.sb, y.sr, c.sb, c.sr);                           \
     break;
-    switch (p.N / 16) {
-      WM_P3_DMA(1) WM_P3_DMA(2) WM_P3_DMA(3) WM_P3_DMA(4) WM_P3_DMA(5) WM_P3_DMA(6) WM_P3_DMA(7) WM_P3_DMA(8)
+    // A band of a few chunks only (the windows just above the narrow-band kernels' range): chunks of
+    // 32 rows, three deep, fit four workgroups on a CU up to N = 64 and overfetch less at the band's
+    // edges (B96 M16384 N64: 119 against 143 us at w = 33, 136 against 150 at w = 48, level from w = 56
+    // to 128, 7 % slower at w = 200; B192 N32: 171 against 204 us at w = 33).
+    if (p.N <= 64 && p.w < kShallowChunksBelow) {
+      switch (p.N / 16) { WM_P3_DMA(1, 32, 3) WM_P3_DMA(2, 32, 3) WM_P3_DMA(3, 32, 3) WM_P3_DMA(4, 32, 3) }
+    } else {
+      switch (p.N / 16) {
+        WM_P3_DMA(1, WM_P3_DMA_KC, WM_P3_DMA_STAGES) WM_P3_DMA(2, WM_P3_DMA_KC, WM_P3_DMA_STAGES)
+        WM_P3_DMA(3, WM_P3_DMA_KC, WM_P3_DMA_STAGES) WM_P3_DMA(4, WM_P3_DMA_KC, WM_P3_DMA_STAGES)
+        WM_P3_DMA(5, WM_P3_DMA_KC, WM_P3_DMA_STAGES) WM_P3_DMA(6, WM_P3_DMA_KC, WM_P3_DMA_STAGES)
+        WM_P3_DMA(7, WM_P3_DMA_KC, WM_P3_DMA_STAGES) WM_P3_DMA(8, WM_P3_DMA_KC, WM_P3_DMA_STAGES)
+      }
     }
 #undef WM_P3_DMA
     return hipGetLastError();
