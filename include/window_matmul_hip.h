@@ -59,7 +59,7 @@ typedef enum wm_status {
 /* Kernel selection.  0 lets the library choose per (shape, dtype, layout). */
 #define WM_FLAG_FORCE_STRIDED 0x1u   /* always use the strided fallback kernels (A/B testing) */
 #define WM_FLAG_NO_ALIGNED_BAND 0x2u /* MFMA kernels: never use the 16-byte aligned band variant */
-#define WM_FLAG_NO_NARROW_BAND 0x4u  /* never use the narrow-band kernels (MFMA, w <= 63; vector ALU, w <= 14; fused attention, w <= 32) */
+#define WM_FLAG_NO_NARROW_BAND 0x4u  /* never use the narrow-band kernels (MFMA, w <= 63; vector ALU, w <= 14; fused attention, w <= 64) */
 #define WM_FLAG_NO_LDS_DIRECT 0x8u   /* never use the kernels that load chunks straight into LDS (fused attention; band-out product at N = 128) */
 
 /* Rank-3 operand: element (b, r, c) lives at data + b*stride_b + r*stride_r + c*stride_c. */
@@ -165,7 +165,7 @@ int wm_window_attention_forward(const wm_operand *q, const wm_operand *k, const 
  * needs no argument here.  Any of grad_q, grad_k, grad_v may be NULL to skip that gradient
  * (grad_q NULL shortens the first kernel to the delta pass, grad_k and grad_v both NULL drop the
  * second).  Up to two kernels are enqueued on the stream; no atomics, so results are
- * reproducible run to run.  With N <= 64 and w <= 32 one kernel computes all three gradients and
+ * reproducible run to run.  With N <= 64 and w <= 48 (64 from N = 48) one kernel computes all three gradients and
  * delta is not touched (it must still be passed: which kernels run is the library's choice;
  * WM_FLAG_NO_NARROW_BAND selects the two-kernel form).  Same support rule and WM_ERR_UNSUPPORTED
  * behaviour as the forward.

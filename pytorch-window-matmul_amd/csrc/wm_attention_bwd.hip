@@ -780,7 +780,7 @@ __global__ __launch_bounds__(kThreads, NK <= 4 ? 2 : 1) void attention_backward_
 // Memory sees q, k, v, dO, O once each (plus the halo, which the neighbouring workgroup has
 // usually just brought into the L2) and dQ, dK, dV once: nothing else bounds this kernel.
 template <typename T, int NK, int NKB>
-__global__ __launch_bounds__(kThreads, NK >= 3 && NKB == 3 ? 2 : 3) void attention_backward_narrow_kernel(
+__global__ __launch_bounds__(kThreads, NKB >= 4 || (NK >= 3 && NKB == 3) ? 2 : 3) void attention_backward_narrow_kernel(
     const uint16_t *__restrict__ Q, const uint16_t *__restrict__ K, const uint16_t *__restrict__ V,
     const uint16_t *__restrict__ O, const uint16_t *__restrict__ dO, const float *__restrict__ L,
     uint16_t *__restrict__ dQ, uint16_t *__restrict__ dK, uint16_t *__restrict__ dV, int B, int M, int w, int nblk,
@@ -792,9 +792,17 @@ __global__ __launch_bounds__(kThreads, NK >= 3 && NKB == 3 ? 2 : 3) void attenti
   constexpr int ROWS = AB_TM + 2 * PADW;   // rows of a tile
   typedef LdsTile<ROWS, 8> TL;
   constexpr int LOADS = TL::LOADS;
-  __shared__ __attribute__((aligned(1024))) uint16_t tile_a[TL::ELEMS];  // Q, then K
-  __shared__ __attribute__((aligned(1024))) uint16_t tile_b[TL::ELEMS];  // dO, then V
-  __shared__ __attribute__((aligned(16))) float stat[2][ROWS];           // [0] D, [1] log-sum-exp in log2 units
+  // Two tiles (Q then K; dO then V) and the row statistics ([0] D, [1] log-sum-exp in log2 units).  With
+  // five row blocks per wavefront they take 66 KB, more than a kernel can declare: that instantiation
+  // gets them as dynamic LDS, which the launcher asks for (narrow_lds_bytes).
+  constexpr bool DYN = NKB >= 5;
+  __shared__ __attribute__((aligned(1024))) uint16_t tiles_declared[DYN ? 8 : 2 * TL::ELEMS];
+  __shared__ __attribute__((aligned(16))) float stat_declared[DYN ? 4 : 2 * ROWS];
+  extern __shared__ __attribute__((aligned(1024))) unsigned char narrow_dynamic_lds[];
+  uint16_t *const tile_a = DYN ? reinterpret_cast<uint16_t *>(narrow_dynamic_lds) : tiles_declared;
+  uint16_t *const tile_b = tile_a + TL::ELEMS;
+  float(*const stat)[ROWS] = reinterpret_cast<float(*)[ROWS]>(
+      DYN ? reinterpret_cast<float *>(narrow_dynamic_lds + 4 * TL::ELEMS) : stat_declared);
   static_assert(4 * RowStage<NB>::ELEMS <= TL::ELEMS, "the four staging areas must fit one tile");
 
   int b, blk;
@@ -836,11 +844,15 @@ __global__ __launch_bounds__(kThreads, NK >= 3 && NKB == 3 ? 2 : 3) void attenti
   };
 
   // For D = dO . O the rows of O come in operand layout (lane pair per row) and meet the rows of dO
-  // in the tile: the wavefront's own 32 rows, and in the first and last wavefront the rows before
+  // in the tile: the wavefront's own 32 rows, and in the first and last wavefronts the rows before
   // and after the workgroup's own.
   const int own_first = PADW + 32 * wave;                            // tile row of the wavefront's first own row
-  const int halo_first = wave == 0 ? 0 : PADW + AB_TM;               // (waves 0 and 3 only)
-  const int h32 = r32 < PADW ? r32 : 0;                              // lanes beyond the halo repeat its first row
+  constexpr int HP = (PADW + 31) / 32;                               // wavefronts per side of the halo (32 rows each)
+  const bool halo_wave = wave < HP || wave >= 4 - HP;                // scalar
+  const int hp = wave < HP ? wave : wave - (4 - HP);
+  const int halo_first = (wave < HP ? 0 : PADW + AB_TM) + 32 * hp;   // first halo row of this wavefront
+  const int halo_rows = min(32, PADW - 32 * hp);
+  const int h32 = r32 < halo_rows ? r32 : 0;                         // lanes beyond the halo repeat its first row
   const uint32_t halo_at = TL::row_at(32 * half + h32);
   u32x4 o_own[NK], o_halo[NK];
   float l_own, l_halo = 0.0f;
@@ -852,7 +864,7 @@ __global__ __launch_bounds__(kThreads, NK >= 3 && NKB == 3 ? 2 : 3) void attenti
     for (int ks = 0; ks < NK; ++ks) o_own[ks] = load_row_chunk(orow + 16 * ks, O, ok);
     l_own = ok ? L[(int64_t)b * M + row] * kLog2e : 0.0f;
   }
-  if (wave == 0 || wave == 3) {
+  if (halo_wave) {
     const int row = t0 + halo_first + h32;
     const bool ok = row >= need_lo && row <= need_hi;
     const uint16_t *orow = O + (int64_t)b * osb + (int64_t)row * osr + 8 * half;
@@ -881,12 +893,12 @@ __global__ __launch_bounds__(kThreads, NK >= 3 && NKB == 3 ? 2 : 3) void attenti
     d = halves_sum(d);
     if (half == 0) stat[0][own_first + r32] = d, stat[1][own_first + r32] = l_own;
   }
-  if (wave == 0 || wave == 3) {
+  if (halo_wave) {
     float d = 0.0f;
 #pragma unroll
     for (int ks = 0; ks < NK; ++ks) d += dot8<T>(own_rows(tile_b, halo_first, halo_at, ks), o_halo[ks]);
     d = halves_sum(d);
-    if (half == 0 && r32 < PADW) stat[0][halo_first + r32] = d, stat[1][halo_first + r32] = l_halo;
+    if (half == 0 && r32 < halo_rows) stat[0][halo_first + r32] = d, stat[1][halo_first + r32] = l_halo;
   }
   __syncthreads();
 
@@ -1043,19 +1055,37 @@ hipError_t launch_backward(const Problem &p, const View &q, const View &k, const
     bool fits = !(p.flags & WM_FLAG_NO_LDS_DIRECT) && (p.M + 3 * AB_KC) * 4 < lim;
     for (const View *t : {&q, &k, &v, &go}) fits = fits && t->sr > 0 && (p.M + 3 * AB_KC) * t->sr * 2 < lim;
     if constexpr (NK <= 4) {
-      // narrow windows: one kernel for all three gradients (two row blocks per wavefront up to w = 16, three up to 32)
-      if (fits && p.w <= 32 && !(p.flags & WM_FLAG_NO_NARROW_BAND)) {
-#define WM_ABN(NKB)                                                                                                   \
-  hipLaunchKernelGGL((attention_backward_narrow_kernel<T, NK, NKB>), grid, block, 0, p.stream, (in_t)q.data,          \
+      // narrow windows: one kernel for all three gradients (two row blocks per wavefront up to w = 16, three up
+      // to 32, four up to 48, five up to 64 where it still pays: B96 M16384 N64 w = 64: 490 against 555 us for
+      // the two kernels, N = 48: 552 against 592, N = 32: 633 against 603)
+      if (fits && (p.w <= 48 || (p.w <= 64 && NK >= 3)) && !(p.flags & WM_FLAG_NO_NARROW_BAND)) {
+#define WM_ABN(NKB, LDS_BYTES)                                                                                        \
+  hipLaunchKernelGGL((attention_backward_narrow_kernel<T, NK, NKB>), grid, block, LDS_BYTES, p.stream, (in_t)q.data,  \
                      (in_t)k.data, (in_t)v.data, (in_t)o.data, (in_t)go.data, lse, (out_t)gq.data, (out_t)gk.data,    \
                      (out_t)gv.data, (int)p.B, (int)p.M, (int)p.w, nblk, (float)scale, q.sb, q.sr, k.sb, k.sr, v.sb,  \
                      v.sr, o.sb, o.sr, go.sb, go.sr, gq.sb, gq.sr, gk.sb, gk.sr, gv.sb, gv.sr)
-        if (p.w <= 16)
-          WM_ABN(2);
-        else
-          WM_ABN(3);
+        if (p.w <= 16) {
+          WM_ABN(2, 0);
+          return hipGetLastError();
+        } else if (p.w <= 32) {
+          WM_ABN(3, 0);
+          return hipGetLastError();
+        } else if (p.w <= 48) {
+          WM_ABN(4, 0);
+          return hipGetLastError();
+        } else {
+          // 66 KB of LDS: above what a kernel gets without asking (the call changes an attribute of the
+          // function, it allocates nothing); if the runtime refuses, the two kernels below take over
+          constexpr int rows = AB_TM + 2 * 64, bytes = 2 * rows * 128 + 2 * rows * 4;
+          const auto kernel = attention_backward_narrow_kernel<T, NK, 5>;
+          if (hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                  bytes) == hipSuccess) {
+            WM_ABN(5, bytes);
+            return hipGetLastError();
+          }
+          (void)hipGetLastError();
+        }
 #undef WM_ABN
-        return hipGetLastError();
       }
     }
     if (fits) {

@@ -284,11 +284,13 @@ def test_narrow_window_training_goes_through_the_separate_ops(device):
 
 @pytest.mark.parametrize("dtype", DTYPES, ids=lambda d: str(d).split(".")[-1])
 @pytest.mark.parametrize("case", [(3, 700, 64, 3), (2, 130, 64, 16), (2, 1000, 64, 17), (5, 300, 64, 32), (4, 257, 48, 8),
-                                  (3, 400, 32, 31), (6, 129, 16, 5), (2, 9, 64, 12), (1, 128, 64, 1), (2, 255, 32, 16)],
+                                  (3, 400, 32, 31), (6, 129, 16, 5), (2, 9, 64, 12), (1, 128, 64, 1), (2, 255, 32, 16),
+                                  (3, 500, 64, 33), (2, 129, 32, 48), (2, 640, 64, 49), (3, 257, 48, 64), (2, 40, 64, 64),
+                                  (2, 300, 16, 41)],
                          ids=lambda c: "B%d_M%d_N%d_w%d" % c)
 def test_one_kernel_and_two_kernel_backward_agree(device, case, dtype):
-    """Heads up to 64 wide, windows up to 32: one kernel computes all three gradients (a workgroup owns
-    128 rows as keys and as queries); WM_FLAG_NO_NARROW_BAND forces the two-kernel backward.  Both
+    """Heads up to 64 wide, windows up to 48 (64 from N = 48): one kernel computes all three gradients (a
+    workgroup owns 128 rows as keys and as queries); WM_FLAG_NO_NARROW_BAND forces the two-kernel backward.  Both
     against the oracle, both ways of asking for part of the gradients, strided (head-major) operands,
     and twice for the same bits."""
     B, M, N, w = case
