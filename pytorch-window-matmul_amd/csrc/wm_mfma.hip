@@ -818,7 +818,7 @@ __global__ __launch_bounds__(kThreads, 3) void mfma_p1_dma_kernel(const uint16_t
 #define WM_P3_DMA_KC 64
 #endif
 #ifndef WM_P3_SHALLOW_BELOW
-#define WM_P3_SHALLOW_BELOW 56
+#define WM_P3_SHALLOW_BELOW 136
 #endif
 constexpr int kShallowChunksBelow = WM_P3_SHALLOW_BELOW;  // window sizes below this take the 32-row chunks
 #ifndef WM_P3_DMA_STAGES
@@ -1144,10 +1144,10 @@ hipError_t launch_p3(const Problem &p, const View &a, const View &y, const View 
                        (const uint16_t *)a.data, (const uint16_t *)y.data, (uint16_t *)c.data, (int)p.B,       \
                        (int)p.M, (int)p.w, nblk_g, g, a.sb, y.sb, y.sr, c.sb, c.sr);                           \
     break;
-    // A band of a few chunks only (the windows just above the narrow-band kernels' range): chunks of
-    // 32 rows, three deep, fit four workgroups on a CU up to N = 64 and overfetch less at the band's
-    // edges (B96 M16384 N64: 119 against 143 us at w = 33, 136 against 150 at w = 48, level from w = 56
-    // to 128, 7 % slower at w = 200; B192 N32: 171 against 204 us at w = 33).
+    // A band of a few chunks only: chunks of 32 rows, three deep, fit four workgroups on a CU up to
+    // N = 64 and overfetch less at the band's edges (B96 M16384 N64, 32- against 64-row chunks: 119
+    // against 140 us at w = 33, 130 against 145 at w = 48, 175 against 188 at w = 96, 206 against 216
+    // at w = 128, 349 against 329 at w = 200).
     if (p.N <= 64 && p.w < kShallowChunksBelow) {
       switch (p.N / 16) { WM_P3_DMA(1, 32, 3) WM_P3_DMA(2, 32, 3) WM_P3_DMA(3, 32, 3) WM_P3_DMA(4, 32, 3) }
     } else {
