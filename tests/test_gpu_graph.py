@@ -26,7 +26,8 @@ def fused(native, q, k, v, go, w, scale):
 
 
 @pytest.mark.parametrize("which", ["separate_ops", "fused_attention"])
-@pytest.mark.parametrize("shape", [(3, 300, 64, 40), (2, 500, 64, 8)], ids=["wide", "narrow"])
+@pytest.mark.parametrize("shape", [(3, 300, 64, 40), (2, 500, 64, 8), (2, 400, 64, 64), (2, 400, 64, 100)],
+                         ids=["w40", "w8", "w64_dynamic_lds", "w100_two_kernels"])
 def test_replay_matches_eager(device, which, shape):
     import window_matmul_kernel as native
 
