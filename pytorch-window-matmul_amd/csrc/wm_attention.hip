@@ -209,24 +209,18 @@ __global__ __launch_bounds__(kThreads, NK <= 4 ? 4 : 2) void attention_forward_k
   }
 
   float l = across_halves_sum(l_part);
+  float alpha = 1.0f;  // what the accumulated O still has to be scaled by (folded into the division by l)
   if (!MASK) {
-    // Band entries outside the sequence: score 0 each, no value row (wave-uniform test first).
-    if (qw0 < w || qw0 + 31 + w > M - 1) {
-      const int n_out = max(0, w - qi) + max(0, qi + w - (M - 1));
-      if (n_out > 0) {
-        const float m_new = fmaxf(m_used, 0.0f);
-        const float alpha = __builtin_amdgcn_exp2f(m_used - m_new);
-        l = l * alpha + (float)n_out * __builtin_amdgcn_exp2f(-m_new);
-        m_used = m_new;
-#pragma unroll
-        for (int hb = 0; hb < NB; ++hb)
-#pragma unroll
-          for (int v = 0; v < 16; ++v) o[hb][v] *= alpha;
-      }
-    }
+    // Band entries outside the sequence: score 0 each, no value row.  Branch-free, see
+    // attention_forward_dma_kernel.
+    const int n_out = max(0, w - qi) + max(0, qi + w - (M - 1));
+    const float m_new = n_out > 0 ? fmaxf(m_used, 0.0f) : m_used;
+    alpha = __builtin_amdgcn_exp2f(m_used - m_new);
+    l = l * alpha + (float)n_out * __builtin_amdgcn_exp2f(-m_new);
+    m_used = m_new;
   }
   if (qi >= M) l = 1.0f;  // rows past the end: keep the arithmetic finite, nothing is stored
-  const float inv = 1.0f / l;
+  const float inv = alpha / l;
   if (L != nullptr && half == 0 && qi < M) L[(int64_t)b * M + qi] = (m_used + __builtin_amdgcn_logf(l)) * kLn2F;
   // every wave is past the last barrier: the value buffers are free and stage the result rows
   static_assert(4 * RowStage<NB>::ELEMS <= 2 * AT_KC * VS, "the four staging areas must fit the value buffers");
