@@ -108,3 +108,21 @@ def test_band_softmax_and_attention_on_a_large_band(device):
     _close(o[B - 1:], o1, "attention output")
     for name, x, y in zip(("grad_q", "grad_k", "grad_v"), (gq, gk, gv), g1):
         _close(x[B - 1:], y, name)
+
+
+@pytest.mark.parametrize("shape", [(1, 4_000_037, 64, 8), (2, 1_500_000, 48, 64)], ids=lambda s: "B%d_M%d_N%d_w%d" % s)
+def test_one_kernel_attention_backward_on_a_long_sequence(device, shape):
+    """The one-kernel backward of the fused attention addresses a batch element with 32-bit byte offsets
+    (up to 2^31 bytes per tensor): at sequences of millions of rows it must give what the two-kernel
+    form gives, also in the last rows, where the offsets are largest."""
+    B, M, N, w = shape
+    g = torch.Generator(device=device).manual_seed(1)
+    q, k, v, go = (torch.randn(B, M, N, device=device, generator=g).to(torch.bfloat16) for _ in range(4))
+    scale = N ** -0.5
+    o, lse = abi.attention_forward(q, k, v, w, scale)
+    one = abi.attention_backward(q, k, v, o, lse, go, w, scale)
+    two = abi.attention_backward(q, k, v, o, lse, go, w, scale, flags=abi.NO_NARROW_BAND)
+    for x, y in zip(one, two):
+        assert bool(torch.isfinite(x).all())
+        torch.testing.assert_close(x[:, -1000:].float(), y[:, -1000:].float(), rtol=2e-2, atol=2e-2)
+        torch.testing.assert_close(x[:, ::997].float(), y[:, ::997].float(), rtol=2e-2, atol=2e-2)
