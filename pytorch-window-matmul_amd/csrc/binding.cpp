@@ -67,7 +67,7 @@ torch::Tensor band_friendly(const torch::Tensor &t) {
 // for float32 -- are padded with zero columns to the next such width (up to 128): zero columns add
 // nothing to a dot product and produce result columns that are cut off again, and two or three
 // passes over the (B,M,N) tensors cost far less than the strided kernels, which take such shapes
-// otherwise (float64 and N > 128 still do).
+// otherwise.  float64 needs none of this: its kernels take every head width.
 int64_t padded_width(const torch::Tensor &t) {
   const int64_t N = t.size(2);
   int64_t unit;
@@ -94,7 +94,7 @@ torch::Tensor cut_columns(const torch::Tensor &t, int64_t N) {
 // results with N columns are independent per slice, bands are the sum over the slices.  The slices
 // of a band are computed and summed in float32 whatever the storage type (a 16-bit partial band
 // would be rounded at the magnitude of the partial sums, which shows where the slices cancel) and
-// the sum is rounded once.  float64 has no tuned kernels and is not sliced.
+// the sum is rounded once.  float64 is not sliced: its kernels take every head width.
 constexpr int64_t kMaxWidth = 128;
 bool sliced_width(const torch::Tensor &t) {
   return t.size(2) > kMaxWidth && (t.scalar_type() == at::kHalf || t.scalar_type() == at::kBFloat16 || t.scalar_type() == at::kFloat);

@@ -49,7 +49,9 @@ def test_argument_validation_happens_on_the_host():
 def test_kernel_choice_names():
     L = abi.lib()
     assert L.wm_kernel_choice(1, 2, 128, 64, 4, 0, 1, abi.FORCE_STRIDED) == b"strided_p1"
-    assert L.wm_kernel_choice(3, 2, 128, 64, 4, 3, 1, 0) == b"strided_p3"  # float64 has no MFMA path
+    assert L.wm_kernel_choice(3, 2, 128, 64, 4, 3, 1, 0) == b"f64_tile_p3"  # float64: register-blocked tiles
+    assert L.wm_kernel_choice(1, 2, 128, 7, 0, 3, 0, 0) == b"f64_tile_p1"   # every layout and head width
+    assert L.wm_kernel_choice(2, 2, 128, 64, 4, 3, 1, abi.FORCE_STRIDED) == b"strided_p2"
     assert L.wm_kernel_choice(9, 2, 128, 64, 4, 0, 1, 0) == b"invalid"
     # per family: float32 MFMA, 16-bit wide band, 16-bit narrow band (P1 any w <= 32, P2 and P3 for w % 4 == 0)
     assert L.wm_kernel_choice(1, 7, 3001, 80, 1500, 0, 1, 0) == b"f32_mfma_p1"

@@ -2,8 +2,8 @@
 
 The reference's CPU path only ever multiplies rows that lie inside the window (reference
 cpu/window_matmul_cpu.cpp:39-43, 129-141), so an Inf in row c of k, v, q or grad_o reaches the
-outputs of rows |i - c| <= w and nothing else.  The matrix-instruction kernels multiply whole
-tiles in which entries outside the band are exact zeros, and 0 * Inf = NaN: there the value can
+outputs of rows |i - c| <= w and nothing else.  The matrix-instruction kernels (and the float64
+tile kernels) multiply whole tiles in which entries outside the band are exact zeros, and 0 * Inf = NaN: there the value can
 also reach rows of the same tile that are outside the window.  This file pins that behaviour as a
 contract, against the CPU oracle run on the same poisoned inputs:
 
@@ -26,7 +26,7 @@ pytestmark = pytest.mark.gpu
 
 M, N, ROW = 2048, 64, 1000
 WINDOWS = [3, 8, 24, 64, 256]
-DTYPES = [torch.bfloat16, torch.float16, torch.float32]
+DTYPES = [torch.bfloat16, torch.float16, torch.float32, torch.float64]
 
 
 def reach(w):
@@ -34,7 +34,7 @@ def reach(w):
 
 
 def bits(t):
-    return t.contiguous().view({2: torch.int16, 4: torch.int32}[t.element_size()])
+    return t.contiguous().view({2: torch.int16, 4: torch.int32, 8: torch.int64}[t.element_size()])
 
 
 def rows_equal(a, b):
