@@ -16,7 +16,8 @@
  *   - Every operand is a rank-3 view described by a base pointer and ELEMENT
  *     strides for (batch, row, column); any strides are accepted.  The fast
  *     kernels need unit column stride and 16-byte aligned rows; other layouts
- *     run on the slower strided kernels, with identical results.
+ *     (and float64 in every layout) run on a slower family of tiled kernels that
+ *     reads element by element through the strides, with the same results.
  *   - Outputs need not be zeroed: every element is written, and band entries
  *     that fall outside the sequence are written as +0.0.
  *   - Band convention: column j of band row i addresses source row c = i+j-w,
@@ -57,7 +58,7 @@ typedef enum wm_status {
 } wm_status;
 
 /* Kernel selection.  0 lets the library choose per (shape, dtype, layout). */
-#define WM_FLAG_FORCE_STRIDED 0x1u   /* always use the strided fallback kernels (A/B testing) */
+#define WM_FLAG_FORCE_STRIDED 0x1u   /* always use the one-thread-per-output kernels (A/B testing) */
 #define WM_FLAG_NO_ALIGNED_BAND 0x2u /* MFMA kernels: never use the 16-byte aligned band variant */
 #define WM_FLAG_NO_NARROW_BAND 0x4u  /* never use the narrow-band kernels (MFMA, w <= 63; vector ALU, w <= 14; fused attention, w <= 64) */
 #define WM_FLAG_NO_LDS_DIRECT 0x8u   /* never use the kernels that load chunks straight into LDS (fused attention; band-out product at N = 128) */

@@ -48,7 +48,7 @@ torch::Tensor vector_friendly(const torch::Tensor &t) {
   const bool ok = t.stride(2) == 1 && (t.stride(1) * es) % 16 == 0 && (t.stride(0) * es) % 16 == 0 && aligned16(t);
   if (ok || t.numel() == 0) return t;
   if (t.is_contiguous()) {
-    // rows that cannot be aligned (N * element size not a multiple of 16): the strided kernels take
+    // rows that cannot be aligned (N * element size not a multiple of 16): the tile kernels take
     // the tensor as it is; alignable rows behind a misaligned pointer (a view at a storage offset)
     // move into a fresh allocation so that the tuned kernels apply
     return (t.size(2) * es) % 16 == 0 ? t.clone(at::MemoryFormat::Contiguous) : t;
@@ -66,8 +66,8 @@ torch::Tensor band_friendly(const torch::Tensor &t) {
 // Head widths that the tuned kernels do not take -- N not a multiple of 16 for 16-bit storage, of 8
 // for float32 -- are padded with zero columns to the next such width (up to 128): zero columns add
 // nothing to a dot product and produce result columns that are cut off again, and two or three
-// passes over the (B,M,N) tensors cost far less than the strided kernels, which take such shapes
-// otherwise.  float64 needs none of this: its kernels take every head width.
+// passes over the (B,M,N) tensors cost less than the element-by-element tile kernels, which take such
+// shapes otherwise.  float64 needs none of this: its kernels take every head width.
 int64_t padded_width(const torch::Tensor &t) {
   const int64_t N = t.size(2);
   int64_t unit;

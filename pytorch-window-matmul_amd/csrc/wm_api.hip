@@ -54,13 +54,13 @@ typedef hipError_t (*strided_fn)(const Problem &, const View &, const View &, co
 
 // Kernel choice per primitive: vector-ALU kernels (the narrowest windows), else narrow-band MFMA
 // family, else wide-band MFMA family (all 16-bit storage except the float32 vector kernels), else
-// the float32 MFMA family, else the float64 tile family (every layout), else strided.
+// the float32 MFMA family, else the tile family (float64; every layout and head width), else strided.
 // The tiled families launch one workgroup per (batch element, block of at least 16 rows), with the
 // batch count rounded up to a multiple of 8; a grid beyond 2^31 - 1 workgroups does not exist, so
 // such extents run on the strided kernels, whose grid strides over the work.
 bool tiled_grid_fits(int64_t B, int64_t M) { return ((B + 7) / 8) * 8 * ((M + 15) / 16) <= 0x7fffffff; }
 
-int run_primitive(mfma_fn narrow, mfma_fn vector, mfma_fn fast, mfma_fn f32, mfma_fn f64, strided_fn slow,
+int run_primitive(mfma_fn narrow, mfma_fn vector, mfma_fn fast, mfma_fn f32, mfma_fn tile, strided_fn slow,
                   const Problem &p, const View &a, const View &y, const View &c) {
   hipError_t err = hipSuccess;
   if (!(p.flags & WM_FLAG_FORCE_STRIDED) && tiled_grid_fits(p.B, p.M)) {
@@ -68,22 +68,22 @@ int run_primitive(mfma_fn narrow, mfma_fn vector, mfma_fn fast, mfma_fn f32, mfm
     if (narrow && !(p.flags & WM_FLAG_NO_NARROW_BAND) && narrow(p, a, y, c, &err)) return to_status(err);
     if (fast(p, a, y, c, &err)) return to_status(err);
     if (f32(p, a, y, c, &err)) return to_status(err);
-    if (f64(p, a, y, c, &err)) return to_status(err);
+    if (tile(p, a, y, c, &err)) return to_status(err);
   }
   return to_status(slow(p, a, y, c));
 }
 
 int p1(const Problem &p, const View &x, const View &y, const View &c) {
   return run_primitive(try_launch_small_p1, try_launch_vector_p1, try_launch_mfma_p1, try_launch_f32_p1,
-                       try_launch_f64_p1, launch_strided_p1, p, x, y, c);
+                       try_launch_tile_p1, launch_strided_p1, p, x, y, c);
 }
 int p2(const Problem &p, const View &a, const View &y, const View &c) {
   return run_primitive(try_launch_small_p2, try_launch_vector_p2, try_launch_mfma_p2, try_launch_f32_p2,
-                       try_launch_f64_p2, launch_strided_p2, p, a, y, c);
+                       try_launch_tile_p2, launch_strided_p2, p, a, y, c);
 }
 int p3(const Problem &p, const View &a, const View &y, const View &c) {
   return run_primitive(try_launch_small_p3, try_launch_vector_p3, try_launch_mfma_p3, try_launch_f32_p3,
-                       try_launch_f64_p3, launch_strided_p3, p, a, y, c);
+                       try_launch_tile_p3, launch_strided_p3, p, a, y, c);
 }
 
 }  // namespace
@@ -264,8 +264,8 @@ const char *wm_kernel_choice(int op, int64_t B, int64_t M, int64_t N, int64_t w,
       return names[op - 1];
     }
   }
-  if (!(flags & WM_FLAG_FORCE_STRIDED) && tiled_grid_fits(B, M) && f64_supports(op, M, N, w, dtype)) {
-    static const char *names[] = {"f64_tile_p1", "f64_tile_p2", "f64_tile_p3"};  // takes every layout
+  if (!(flags & WM_FLAG_FORCE_STRIDED) && tiled_grid_fits(B, M) && tile_supports(op, M, N, w, dtype)) {
+    static const char *names[] = {"tile_p1", "tile_p2", "tile_p3"};  // takes every layout
     return names[op - 1];
   }
   static const char *names[] = {"strided_p1", "strided_p2", "strided_p3"};

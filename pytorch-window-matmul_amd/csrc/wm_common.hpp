@@ -62,11 +62,12 @@ bool try_launch_f32_p1(const Problem &p, const View &x, const View &y, const Vie
 bool try_launch_f32_p2(const Problem &p, const View &a, const View &y, const View &c, hipError_t *err);
 bool try_launch_f32_p3(const Problem &p, const View &a, const View &y, const View &c, hipError_t *err);
 bool f32_supports(int op, int64_t M, int64_t N, int64_t w, int dtype);
-// float64 family: 64 x 64 tiles on the vector ALU, any strides, any N and w.
-bool try_launch_f64_p1(const Problem &p, const View &x, const View &y, const View &c, hipError_t *err);
-bool try_launch_f64_p2(const Problem &p, const View &a, const View &y, const View &c, hipError_t *err);
-bool try_launch_f64_p3(const Problem &p, const View &a, const View &y, const View &c, hipError_t *err);
-bool f64_supports(int op, int64_t M, int64_t N, int64_t w, int dtype);
+// Tile family: float64, and whatever the families above decline in 16-bit and float32 storage;
+// 64 x 64 tiles on the 16x16x4 matrix instructions, any strides, any N and w.
+bool try_launch_tile_p1(const Problem &p, const View &x, const View &y, const View &c, hipError_t *err);
+bool try_launch_tile_p2(const Problem &p, const View &a, const View &y, const View &c, hipError_t *err);
+bool try_launch_tile_p3(const Problem &p, const View &a, const View &y, const View &c, hipError_t *err);
+bool tile_supports(int op, int64_t M, int64_t N, int64_t w, int dtype);
 // Pure predicate behind the wide-band 16-bit functions above (shape/dtype only).
 bool mfma_supports(int op, int64_t B, int64_t M, int64_t N, int64_t w, int dtype);
 

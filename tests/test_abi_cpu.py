@@ -49,8 +49,10 @@ def test_argument_validation_happens_on_the_host():
 def test_kernel_choice_names():
     L = abi.lib()
     assert L.wm_kernel_choice(1, 2, 128, 64, 4, 0, 1, abi.FORCE_STRIDED) == b"strided_p1"
-    assert L.wm_kernel_choice(3, 2, 128, 64, 4, 3, 1, 0) == b"f64_tile_p3"  # float64: register-blocked tiles
-    assert L.wm_kernel_choice(1, 2, 128, 7, 0, 3, 0, 0) == b"f64_tile_p1"   # every layout and head width
+    assert L.wm_kernel_choice(3, 2, 128, 64, 4, 3, 1, 0) == b"tile_p3"  # float64: tiles on the float64 matrix instruction
+    assert L.wm_kernel_choice(1, 2, 128, 7, 0, 3, 0, 0) == b"tile_p1"   # every layout and head width
+    assert L.wm_kernel_choice(2, 2, 128, 7, 4, 2, 1, 0) == b"tile_p2"   # bf16 at a head width no tuned kernel takes
+    assert L.wm_kernel_choice(1, 2, 128, 64, 4, 0, 0, 0) == b"tile_p1"  # float32 in a layout no tuned kernel takes
     assert L.wm_kernel_choice(2, 2, 128, 64, 4, 3, 1, abi.FORCE_STRIDED) == b"strided_p2"
     assert L.wm_kernel_choice(9, 2, 128, 64, 4, 0, 1, 0) == b"invalid"
     # per family: float32 MFMA, 16-bit wide band, 16-bit narrow band (P1 any w <= 32, P2 and P3 for w % 4 == 0)
@@ -88,7 +90,7 @@ def test_kernel_choice_names():
     assert L.wm_kernel_choice(1, 96, 16384, 64, 7, 1, 1, 0) == b"narrow_p1"
     assert L.wm_kernel_choice(1, 96, 16384, 64, 2, 2, 1, 0) == b"narrow_p1"
     assert L.wm_kernel_choice(1, 96, 16384, 64, 3, 2, 1, 0) == b"narrow_p1"
-    assert L.wm_kernel_choice(2, 96, 16384, 64, 7, 2, 1, abi.NO_NARROW_BAND) == b"strided_p2"
+    assert L.wm_kernel_choice(2, 96, 16384, 64, 7, 2, 1, abi.NO_NARROW_BAND) == b"tile_p2"   # below the wide-band kernels' w = 8
     # float32: band-in products on the vector ALU up to w = 14, the float32 MFMA kernels beyond; the
     # band-out product on the narrow-band MFMA kernel up to w = 31 when N is a multiple of 16 up to 64
     assert L.wm_kernel_choice(2, 96, 16384, 64, 3, 0, 1, 0) == b"vector_p2"
@@ -106,8 +108,8 @@ def test_kernel_choice_names():
     assert L.wm_kernel_choice(2, 96, 16384, 16, 28, 0, 1, 0) == b"narrow_p2"
     assert L.wm_kernel_choice(2, 96, 16384, 64, 29, 0, 1, 0) == b"f32_mfma_p2"
     assert L.wm_kernel_choice(1, 96, 16384, 64, 8, 0, 1, abi.NO_NARROW_BAND) == b"f32_mfma_p1"
-    assert L.wm_kernel_choice(1, 2, 128, 3, 4, 0, 1, 0) == b"strided_p1"  # N not a multiple of 8
-    assert L.wm_kernel_choice(1, 2, 128, 64, 4, 2, 0, 0) == b"strided_p1"  # layout not vector friendly
+    assert L.wm_kernel_choice(1, 2, 128, 3, 4, 0, 1, 0) == b"tile_p1"  # N not a multiple of 8
+    assert L.wm_kernel_choice(1, 2, 128, 64, 4, 2, 0, 0) == b"tile_p1"  # layout not vector friendly
 
 
 def test_python_surface_matches_reference():
