@@ -23,7 +23,7 @@ the count but its time is inside the step).  Next to it:
                  (N = 128, w = 512, float16) and the float32 band that covers the sequence.
 
 Usage: python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c2|c4|c5] [--no-cpu] [--no-others]
-       python bench.py --kernels-only [--shape B M N w] [--dtype bf16|fp16|fp32] [--family auto|wide|staged|strided]
+       python bench.py --kernels-only [--shape B M N w] [--dtype bf16|fp16|fp32|fp64] [--family auto|wide|staged|strided]
 """
 import argparse
 import hashlib
@@ -42,6 +42,7 @@ for _p in (REPO, PKG):
 HBM_PEAK_GBS = 8000.0      # MI355X published HBM3E bandwidth
 MFMA_PEAK_TFLOPS = 2500.0  # dense bf16 / fp16 matrix peak
 FP32_PEAK_TFLOPS = 157.3   # float32 matrix peak
+FP64_PEAK_TFLOPS = 78.6    # float64 matrix peak
 
 WORKLOADS = {
     "c3": dict(B=96, M=4096, N=64, w=256, dtype="bf16", qk_scale=0.125, backward=True,
@@ -138,7 +139,7 @@ def cpu_baseline(cfg, seconds_budget=20.0):
 
     torch.set_num_threads(1)
     M, N, w = cfg["M"], cfg["N"], cfg["w"]
-    rnd = {"bf16": torch.bfloat16, "fp16": torch.float16, "fp32": torch.float32}[cfg["dtype"]]
+    rnd = {"bf16": torch.bfloat16, "fp16": torch.float16, "fp32": torch.float32, "fp64": torch.float64}[cfg["dtype"]]
 
     def run(impl, budget):
         g = torch.Generator().manual_seed(0)
@@ -193,8 +194,9 @@ class Bench:
 
         self.cfg, self.abi, self.torch, self.fam = cfg, abi, torch, family
         self.B, self.M, self.N, self.w = cfg["B"], cfg["M"], cfg["N"], cfg["w"]
-        self.dtype = {"bf16": torch.bfloat16, "fp16": torch.float16, "fp32": torch.float32}[cfg["dtype"]]
-        self.es = 4 if self.dtype == torch.float32 else 2
+        self.dtype = {"bf16": torch.bfloat16, "fp16": torch.float16, "fp32": torch.float32,
+                      "fp64": torch.float64}[cfg["dtype"]]
+        self.es = torch.empty((), dtype=self.dtype).element_size()
         self.dev = torch.device("cuda:0")
         self.g = torch.Generator().manual_seed(0)
         self.q, self.k = self.synth(cfg["qk_scale"]), self.synth(cfg["qk_scale"])
@@ -243,7 +245,8 @@ class Bench:
                               iters, 3)
             out["band_softmax"] = {"fwd_ms": round(bs_fwd, 4), "fwd_GBps": round(2 * band_bytes / bs_fwd / 1e6, 1),
                                    "bwd_ms": round(bs_bwd, 4), "bwd_GBps": round(3 * band_bytes / bs_bwd / 1e6, 1)}
-            if es == 2:  # the fused kernels are 16-bit only; float32 runs the chain of separate ops
+            # the fused kernels are 16-bit only (N a multiple of 16 up to 128); other shapes run the chain of separate ops
+            if es == 2 and abi.lib().wm_window_attention_supported(M, N, w, abi.DTYPES[self.dtype], 1.0):
                 fo, flse = abi.attention_forward(q, k, v, w, 1.0)
                 fwd = time_gpu(lambda: abi.attention_forward(q, k, v, w, 1.0), iters, 3)
                 fused = {"fwd_ms": round(fwd, 4), "fwd_TFLOPs": round(2 * self.unit / fwd / 1e9, 1),
@@ -265,9 +268,10 @@ class Bench:
             out["copy_bytes_each_way"] = att.numel() * es
         dom = max(per_kernel, key=lambda n: per_kernel[n]["ms"])
         out["slowest_kernel"] = dom
-        if self.dtype == torch.float32:
-            out["bound"] = "mfma (float32 matrix peak %.1f TFLOP/s)" % FP32_PEAK_TFLOPS
-            out["slowest_kernel_frac"] = round(per_kernel[dom]["TFLOPs"] / FP32_PEAK_TFLOPS, 4)
+        if self.dtype in (torch.float32, torch.float64):
+            name, peak = ("float32", FP32_PEAK_TFLOPS) if self.dtype == torch.float32 else ("float64", FP64_PEAK_TFLOPS)
+            out["bound"] = "mfma (%s matrix peak %.1f TFLOP/s)" % (name, peak)
+            out["slowest_kernel_frac"] = round(per_kernel[dom]["TFLOPs"] / peak, 4)
         else:
             out["bound"] = "hbm"
             out["slowest_kernel_frac"] = per_kernel[dom]["hbm_frac"]
@@ -282,7 +286,7 @@ def main():
     ap.add_argument("--workload", default="c3", choices=sorted(WORKLOADS))
     ap.add_argument("--shape", type=int, nargs=4, metavar=("B", "M", "N", "w"),
                     help="time this shape instead of a named workload (forward + backward)")
-    ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp16", "fp32"],
+    ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp16", "fp32", "fp64"],
                     help="storage type for --shape")
     ap.add_argument("--family", default="auto", choices=["auto", "wide", "staged", "strided"],
                     help="kernel family for the per-kernel timings: the library's choice, the wide-band MFMA "
