@@ -51,6 +51,8 @@ BATCH_CASES = [
     pytest.param(9, 1 << 22, 64, 4, torch.float32, 0, id="rows-vector-f32-w4"),   # q, k, v 2.4 G elements
     pytest.param(9, 1 << 22, 64, 20, torch.float32, 0, id="rows-mfma-f32-w20"),
     pytest.param(5, 1 << 22, 128, 2, torch.float16, abi.FORCE_STRIDED, id="rows-strided-w2"),
+    pytest.param(3, 1 << 20, 20, 512, torch.bfloat16, 0, id="band-tile-bf16-n20"),  # head width no tuned kernel takes
+    pytest.param(3, 1 << 20, 16, 400, torch.float64, 0, id="band-tile-f64-w400"),   # band 2.5 G elements, 20 GB
 ]
 
 
