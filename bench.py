@@ -100,13 +100,27 @@ def profiled_traffic(kernel_label):
     return value, digest
 
 
-def time_gpu(fn, iters, warmup):
+def time_gpu(fn, iters, warmup, settle_ms=0.0):
     """Median duration of one launch, each launch bracketed by its own pair of HIP events on the
-    current stream (so that the gap between dependent launches is not counted as kernel time)."""
+    current stream (so that the gap between dependent launches is not counted as kernel time).
+    The untimed launches before it go on until `settle_ms` of GPU time have passed: after a pause
+    (host-side input generation between workloads) the first 10 ms of a run of launches are a clock
+    transient, 300 rising to 400 and settling at 310 us per launch for the band-out product at
+    B16 M32768 N128 w512, and a median over 10 launches taken inside it is not the kernel's rate."""
     import torch
 
     for _ in range(warmup):
         fn()
+    if settle_ms > 0:
+        start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
+        for _ in range(1000):  # bounded: a launch that takes no time cannot spin here
+            for _ in range(4):
+                fn()
+            stop.record()
+            stop.synchronize()
+            if start.elapsed_time(stop) >= settle_ms:
+                break
     pairs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(iters)]
     torch.cuda.synchronize()
     for start, stop in pairs:
@@ -206,8 +220,10 @@ class Bench:
     def synth(self, scale=1.0):
         return (self.torch.randn(self.B, self.M, self.N, generator=self.g) * scale).to(self.dtype).to(self.dev)
 
-    def kernels(self, iters):
-        """Per-kernel timing through the C ABI (one launch per call), same tensors, same stream."""
+    def kernels(self, iters, settle_ms=30.0):
+        """Per-kernel timing through the C ABI (one launch per call), same tensors, same stream.
+        `settle_ms` of untimed launches precede every timing (0 for profiler passes, which want
+        few launches and say how many they saw)."""
         torch, abi, cfg, w, fam = self.torch, self.abi, self.cfg, self.w, self.fam
         B, M, N, es = self.B, self.M, self.N, self.es
         out = {}
@@ -232,29 +248,29 @@ class Bench:
             kb = kernel_bytes(B, M, N, w, es)
             per_kernel = {}
             for name, fn in launches.items():
-                ms = time_gpu(fn, iters, 3)
+                ms = time_gpu(fn, iters, 3, settle_ms)
                 per_kernel[name] = {"ms": round(ms, 4), "GBps": round(kb / ms / 1e6, 1),
                                     "hbm_frac": round(kb / ms / 1e6 / HBM_PEAK_GBS, 4),
                                     "TFLOPs": round(self.unit / ms / 1e9, 1)}
             out["kernels"], out["algorithmic_bytes_per_launch"] = per_kernel, kb
-            out["softmax_fwd_ms"] = round(time_gpu(lambda: torch.softmax(att, dim=-1), iters, 3), 4)
+            out["softmax_fwd_ms"] = round(time_gpu(lambda: torch.softmax(att, dim=-1), iters, 3, settle_ms), 4)
             band_bytes = att.numel() * es
             sm_out = torch.empty_like(att)
-            bs_fwd = time_gpu(lambda: abi.band_softmax_forward(att, 1.0, out=sm_out), iters, 3)
+            bs_fwd = time_gpu(lambda: abi.band_softmax_forward(att, 1.0, out=sm_out), iters, 3, settle_ms)
             bs_bwd = time_gpu(lambda: abi.band_softmax_backward(probs, ga if ga is not None else att, 1.0, out=sm_out),
-                              iters, 3)
+                              iters, 3, settle_ms)
             out["band_softmax"] = {"fwd_ms": round(bs_fwd, 4), "fwd_GBps": round(2 * band_bytes / bs_fwd / 1e6, 1),
                                    "bwd_ms": round(bs_bwd, 4), "bwd_GBps": round(3 * band_bytes / bs_bwd / 1e6, 1)}
             # the fused kernels are 16-bit only (N a multiple of 16 up to 128); other shapes run the chain of separate ops
             if es == 2 and abi.lib().wm_window_attention_supported(M, N, w, abi.DTYPES[self.dtype], 1.0):
                 fo, flse = abi.attention_forward(q, k, v, w, 1.0)
-                fwd = time_gpu(lambda: abi.attention_forward(q, k, v, w, 1.0), iters, 3)
+                fwd = time_gpu(lambda: abi.attention_forward(q, k, v, w, 1.0), iters, 3, settle_ms)
                 fused = {"fwd_ms": round(fwd, 4), "fwd_TFLOPs": round(2 * self.unit / fwd / 1e9, 1),
                          "fwd_mfma_frac": round(2 * self.unit / fwd / 1e9 / MFMA_PEAK_TFLOPS, 4),
                          "fwd_hbm_frac": round((4 * B * M * N * es + 4 * B * M) / fwd / 1e6 / HBM_PEAK_GBS, 4)}
                 # (a forward-only workload gets the backward of a training step as well: its band is so
                 # narrow that the step is bound by the eight tensors it reads and writes, q k v o dO dq dk dv)
-                bwd = time_gpu(lambda: abi.attention_backward(q, k, v, fo, flse, go, w, 1.0), iters, 3)
+                bwd = time_gpu(lambda: abi.attention_backward(q, k, v, fo, flse, go, w, 1.0), iters, 3, settle_ms)
                 fused.update({"bwd_ms": round(bwd, 4), "bwd_TFLOPs": round(4 * self.unit / bwd / 1e9, 1),
                               "bwd_mfma_frac": round(4 * self.unit / bwd / 1e9 / MFMA_PEAK_TFLOPS, 4),
                               "bwd_hbm_frac": round((8 * B * M * N * es + 4 * B * M) / bwd / 1e6 / HBM_PEAK_GBS, 4),
@@ -263,7 +279,7 @@ class Bench:
                 del fo, flse
             # device-to-device copy of the band as the achievable-bandwidth yardstick
             scratch = torch.empty_like(att)
-            copy_ms = time_gpu(lambda: scratch.copy_(att), iters, 3)
+            copy_ms = time_gpu(lambda: scratch.copy_(att), iters, 3, settle_ms)
             out["copy_yardstick_GBps"] = round(2 * att.numel() * es / copy_ms / 1e6, 1)
             out["copy_bytes_each_way"] = att.numel() * es
         dom = max(per_kernel, key=lambda n: per_kernel[n]["ms"])
@@ -321,7 +337,7 @@ def main():
     B, M, N, w = bench.B, bench.M, bench.N, bench.w
 
     if args.kernels_only:
-        k = bench.kernels(iters)
+        k = bench.kernels(iters, settle_ms=0.0)
         print(json.dumps({"workload": cfg["label"], "family": args.family, "kernels": k["kernels"],
                           "fused_attention": k.get("fused_attention"), "band_softmax": k["band_softmax"],
                           "copy_yardstick_GBps": k["copy_yardstick_GBps"],
