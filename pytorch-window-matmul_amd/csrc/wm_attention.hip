@@ -606,9 +606,8 @@ template <typename T, int NK>
 hipError_t launch_forward(const Problem &p, const View &q, const View &k, const View &v, const View &o, float *lse,
                           double scale, int mask) {
   const int nblk = (int)((p.M + AT_TM - 1) / AT_TM);
-  const int64_t groups = (p.B + 7) / 8;
-  if (groups * 8 * nblk > 0x7fffffff) return hipErrorInvalidValue;
-  const dim3 grid((unsigned)(groups * 8 * nblk)), block(kThreads);
+  if (tiled_grid(p.B, nblk) > 0x7fffffff) return hipErrorInvalidValue;
+  const dim3 grid((unsigned)tiled_grid(p.B, nblk)), block(kThreads);
   const float c = (float)(scale * 1.4426950408889634);
 #define WM_AT(KERNEL)                                                                                              \
   hipLaunchKernelGGL(KERNEL, grid, block, 0, p.stream, (const uint16_t *)q.data, (const uint16_t *)k.data,         \

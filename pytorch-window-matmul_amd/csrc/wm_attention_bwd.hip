@@ -1044,9 +1044,8 @@ hipError_t launch_backward(const Problem &p, const View &q, const View &k, const
                            const View &go, const float *lse, float *delta, const View &gq, const View &gk,
                            const View &gv, double scale) {
   const int nblk = (int)((p.M + AB_TM - 1) / AB_TM);
-  const int64_t groups = (p.B + 7) / 8;
-  if (groups * 8 * nblk > 0x7fffffff) return hipErrorInvalidValue;
-  const dim3 grid((unsigned)(groups * 8 * nblk)), block(kThreads);
+  if (tiled_grid(p.B, nblk) > 0x7fffffff) return hipErrorInvalidValue;
+  const dim3 grid((unsigned)tiled_grid(p.B, nblk)), block(kThreads);
   typedef const uint16_t *in_t;
   typedef uint16_t *out_t;
   {

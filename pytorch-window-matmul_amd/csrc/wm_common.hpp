@@ -34,6 +34,12 @@ struct Problem {
   hipStream_t stream;
 };
 
+// Workgroups of a tiled launch over B batch elements of nblk blocks each (the decode_block of the
+// kernels maps them back): whole elements for every full group of 8, the rest of the tiles in eight
+// equal ranges.  No surplus workgroups: the dispatcher places workgroups in order, and ones that
+// return at once still shift the others onto fewer CUs.
+inline int64_t tiled_grid(int64_t B, int64_t nblk) { return 8 * ((B >> 3) * nblk + ((B & 7) * nblk + 7) / 8); }
+
 // Launchers return hipSuccess or the launch error.  The strided family accepts
 // any dtype and layout; the MFMA family reports whether it took the problem.
 hipError_t launch_strided_p1(const Problem &p, const View &x, const View &y, const View &c);

@@ -1070,7 +1070,7 @@ bool band_aligned(const View &v, int64_t w, unsigned flags) {
 // skew per row (2w elements) keeps them aligned, 16-byte chunks otherwise.
 int band_group(const View &v, int64_t w) { return (w % 32 == 0 && ((uintptr_t)v.data % 128) == 0) ? 64 : 8; }
 
-unsigned grid_size(int64_t B, int64_t nblk) { return (unsigned)(((B + 7) / 8) * 8 * nblk); }
+unsigned grid_size(int64_t B, int64_t nblk) { return (unsigned)tiled_grid(B, nblk); }
 
 // Shapes the kernels that load their tiles straight into LDS accept (band-in products): 32-bit byte
 // offsets inside a batch element of the band and of Y (chunks past the end included), and band rows

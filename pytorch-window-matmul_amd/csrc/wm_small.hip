@@ -716,7 +716,7 @@ bool small_p1_shape_ok(int64_t M, int64_t N, int64_t w, int dtype) {
   return M >= 1 && M <= (1 << 30) && w >= 1 && w <= (N <= 64 ? WM_SMALL_P1_MAX_W : SMALL_MAX_W);
 }
 
-unsigned small_grid(int64_t B, int64_t nblk) { return (unsigned)(((B + 7) / 8) * 8 * nblk); }
+unsigned small_grid(int64_t B, int64_t nblk) { return (unsigned)tiled_grid(B, nblk); }
 
 template <typename T>
 hipError_t launch_small_p1(const Problem &p, const View &x, const View &y, const View &c) {

@@ -296,7 +296,7 @@ size_t vector_out_lds(int64_t w, int64_t N, int dtype) {
   return (size_t)((2 * vector_out_rows(N, dtype) + 2 * w) * (N + vec)) * (16 / vec);
 }
 
-unsigned vector_grid(int64_t B, int64_t nblk) { return (unsigned)(((B + 7) / 8) * 8 * nblk); }
+unsigned vector_grid(int64_t B, int64_t nblk) { return (unsigned)tiled_grid(B, nblk); }
 
 template <typename T, bool TRANSPOSED>
 hipError_t launch_vector(const Problem &p, const View &a, const View &y, const View &c) {
