@@ -144,3 +144,34 @@ def test_runs_on_a_side_stream(device):
         got = abi.window_forward(q, k.transpose(1, 2), w)
     s.synchronize()
     assert torch.equal(got, want)
+
+
+@pytest.mark.parametrize("B", [7, 8, 9, 12, 17, 23])
+@pytest.mark.parametrize("dtype,N,w", [(torch.bfloat16, 64, 64), (torch.bfloat16, 64, 8), (torch.float16, 128, 2),
+                                       (torch.float32, 80, 40), (torch.float32, 32, 16), (torch.float32, 64, 3)],
+                         ids=["wide", "narrow", "vector", "f32-mfma", "f32-narrow", "f32-vector"])
+def test_batch_counts_around_multiples_of_eight(device, B, dtype, N, w):
+    """Workgroups are dealt to the 8 XCDs by batch element for full groups of 8 and by ranges of tiles
+    for the elements left over: every (batch element, block) must be computed exactly once, whatever B."""
+    M = 300
+    print(f"case B={B} {dtype} N={N} w={w}", flush=True)
+    q, k, v, a, ga, go = (t.to(device) for t in make(B, M, N, w, dtype, seed=40))
+    kt = k.transpose(1, 2)
+    tol = dict(rtol=1e-3, atol=1e-3) if dtype == torch.float32 else dict(rtol=2e-2, atol=2e-2)
+    got, want = [], []
+    for flags, res in ((0, got), (abi.FORCE_STRIDED, want)):
+        res.append(abi.window_forward(q, kt, w, flags))
+        res.extend(abi.window_backward(q, kt, w, ga, flags))
+        res.append(abi.unwindow_forward(a, v, w, flags))
+        res.extend(abi.unwindow_backward(a, v, w, go, flags))
+    for x, y in zip(got, want):
+        torch.testing.assert_close(x.float(), y.float(), **tol)
+    if dtype != torch.float32:
+        scale = N ** -0.5
+        o, lse = abi.attention_forward(q, k, v, w, scale)
+        grads = abi.attention_backward(q, k, v, o, lse, go, w, scale)
+        o1, lse1 = abi.attention_forward(q[B - 1:], k[B - 1:], v[B - 1:], w, scale)
+        g1 = abi.attention_backward(q[B - 1:], k[B - 1:], v[B - 1:], o1, lse1, go[B - 1:], w, scale)
+        assert torch.equal(o[B - 1:], o1) and torch.equal(lse[B - 1:], lse1)
+        for x, y in zip(grads, g1):
+            assert torch.equal(x[B - 1:], y)
