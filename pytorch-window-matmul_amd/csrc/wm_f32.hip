@@ -397,11 +397,15 @@ __global__ __launch_bounds__(kThreads, NK8 <= 8 ? 4 : 2) void f32_band_out_kerne
 #pragma unroll
     for (int v = 0; v < 16; ++v) acc[v] = 0.f;
     const float *yl = y_lds[buf] + col * SY + 4 * half;
+    // a chunk that lies wholly outside the sequence (a quarter of them when the band covers the
+    // sequence) holds zeros only: nothing to multiply, the stores below write the zeros
+    if (cb + KC > 0 && cb < M) {
 #pragma unroll
-    for (int u = 0; u < NK8; ++u) {
-      const f32x4 aop = *reinterpret_cast<const f32x4 *>(yl + 8 * u);
+      for (int u = 0; u < NK8; ++u) {
+        const f32x4 aop = *reinterpret_cast<const f32x4 *>(yl + 8 * u);
 #pragma unroll
-      for (int j = 0; j < 4; ++j) acc = mma(aop[j], xop[u][j], acc);
+        for (int j = 0; j < 4; ++j) acc = mma(aop[j], xop[u][j], acc);
+      }
     }
     // acc[v]: dense column c = cb + 8 (v / 4) + 4 half + v % 4, row i; band column j = c - i + w
     wave_sync_lds();  // the pieces of the previous chunk have been read
