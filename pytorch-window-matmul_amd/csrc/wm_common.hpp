@@ -40,6 +40,27 @@ struct Problem {
 // return at once still shift the others onto fewer CUs.
 inline int64_t tiled_grid(int64_t B, int64_t nblk) { return 8 * ((B >> 3) * nblk + ((B & 7) * nblk + 7) / 8); }
 
+// Workgroup -> (batch, block).  Workgroups are dealt round-robin to the 8 XCDs, each with its
+// own L2: XCD x runs ids x, x + 8, ...  Every full group of 8 batch elements gives one element to
+// each XCD, so that neighbouring blocks of an element find the rows they share (the +-w halo) in
+// that L2; the B % 8 elements left over are cut into 8 contiguous ranges of tiles, one per XCD
+// (a whole element per XCD would leave one XCD idle at B = 7).  The launch uses tiled_grid():
+// at most 7 workgroups at the end of the grid have no tile and return at once.
+__device__ __forceinline__ bool decode_block(int nblk, int B, int *b, int *blk) {
+  const int id = blockIdx.x, xcd = id & 7, slot = id >> 3;
+  const int full = (B >> 3) * nblk;  // slots of the full groups
+  if (slot < full) {
+    *b = (slot / nblk) * 8 + xcd;
+    *blk = slot % nblk;
+    return true;
+  }
+  const int64_t tiles = (int64_t)(B & 7) * nblk, per = (tiles + 7) / 8, t = xcd * per + (slot - full);
+  if (slot - full >= per || t >= tiles) return false;
+  *b = (B & ~7) + (int)(t / nblk);
+  *blk = (int)(t % nblk);
+  return true;
+}
+
 // Launchers return hipSuccess or the launch error.  The strided family accepts
 // any dtype and layout; the MFMA family reports whether it took the problem.
 hipError_t launch_strided_p1(const Problem &p, const View &x, const View &y, const View &c);

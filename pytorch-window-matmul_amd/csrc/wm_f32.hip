@@ -66,27 +66,6 @@ __device__ __forceinline__ void wave_sync_lds() {
 __device__ __forceinline__ f32x16 mma(float a, float b, f32x16 c) {
   return __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, 0, 0, 0);
 }
-// Workgroup -> (batch, block).  Workgroups are dealt round-robin to the 8 XCDs, each with its
-// own L2: XCD x runs ids x, x + 8, ...  Every full group of 8 batch elements gives one element to
-// each XCD, so that neighbouring blocks of an element find the rows they share (the +-w halo) in
-// that L2; the B % 8 elements left over are cut into 8 contiguous ranges of tiles, one per XCD
-// (a whole element per XCD would leave one XCD idle at B = 7).  The launch uses tiled_grid():
-// at most 7 workgroups at the end of the grid have no tile and return at once.
-__device__ __forceinline__ bool decode_block(int nblk, int B, int *b, int *blk) {
-  const int id = blockIdx.x, xcd = id & 7, slot = id >> 3;
-  const int full = (B >> 3) * nblk;  // slots of the full groups
-  if (slot < full) {
-    *b = (slot / nblk) * 8 + xcd;
-    *blk = slot % nblk;
-    return true;
-  }
-  const int64_t tiles = (int64_t)(B & 7) * nblk, per = (tiles + 7) / 8, t = xcd * per + (slot - full);
-  if (slot - full >= per || t >= tiles) return false;
-  *b = (B & ~7) + (int)(t / nblk);
-  *blk = (int)(t % nblk);
-  return true;
-}
-
 // ------------------------------------------------------------------------------------------
 // P2: C[b,i,h] = sum_c T[i][c] Y[b,c,h]          P3: C[b,c,h] = sum_r T[r][c] Y[b,r,h]
 // acc(m = h, n = output row): A operand Y[k][h] (4-byte LDS reads along h), B operand T.

@@ -419,27 +419,6 @@ __device__ __forceinline__ u32x4 keep_rows_tr(u32x4 v, int r_first, int lo, int 
   return r;
 }
 
-// Workgroup -> (batch, block).  Workgroups are dealt round-robin to the 8 XCDs, each with its
-// own L2: XCD x runs ids x, x + 8, ...  Every full group of 8 batch elements gives one element to
-// each XCD, so that neighbouring blocks of an element find the rows they share (the +-w halo) in
-// that L2; the B % 8 elements left over are cut into 8 contiguous ranges of tiles, one per XCD
-// (a whole element per XCD would leave one XCD idle at B = 7).  The launch uses tiled_grid():
-// at most 7 workgroups at the end of the grid have no tile and return at once.
-__device__ __forceinline__ bool decode_block(int nblk, int B, int *b, int *blk) {
-  const int id = blockIdx.x, xcd = id & 7, slot = id >> 3;
-  const int full = (B >> 3) * nblk;  // slots of the full groups
-  if (slot < full) {
-    *b = (slot / nblk) * 8 + xcd;
-    *blk = slot % nblk;
-    return true;
-  }
-  const int64_t tiles = (int64_t)(B & 7) * nblk, per = (tiles + 7) / 8, t = xcd * per + (slot - full);
-  if (slot - full >= per || t >= tiles) return false;
-  *b = (B & ~7) + (int)(t / nblk);
-  *blk = (int)(t % nblk);
-  return true;
-}
-
 // Row stride (elements) of matrices read with lds_read_transposed: the byte stride must be
 // 32 or 96 (mod 128) so that the 4 rows touched by a 16-lane group fall into distinct banks.
 #ifndef WM_PAD_TR

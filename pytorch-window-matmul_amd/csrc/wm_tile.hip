@@ -149,11 +149,13 @@ struct Rows {  // one batch element of a view
 
 // P1.  Block rows i0.., columns c0.. of X * Y^T for every 64-column chunk that meets the band.
 template <class T, bool X_FAST, bool Y_FAST>
-__global__ __launch_bounds__(THREADS) void tile_band_out_kernel(View xv, View yv, View cv, int64_t M, int64_t N,
-                                                                int64_t w, int64_t tiles) {
+__global__ __launch_bounds__(THREADS) void tile_band_out_kernel(View xv, View yv, View cv, int B, int64_t M,
+                                                                int64_t N, int64_t w, int64_t tiles) {
   typedef typename Acc<T>::type C;
   __shared__ Stage<C> t;
-  const int64_t b = blockIdx.x / tiles, i0 = (blockIdx.x % tiles) * TS;
+  int b, blk;
+  if (!decode_block((int)tiles, B, &b, &blk)) return;  // neighbouring tiles of a batch element share an XCD's L2
+  const int64_t i0 = (int64_t)blk * TS;
   const Rows<T> x(xv, b), y(yv, b), c(cv, b);
   const int64_t stages = (N + KS - 1) / KS;
   for (int64_t c0 = i0 - w; c0 <= i0 + TS - 1 + w; c0 += TS) {
@@ -179,11 +181,13 @@ __global__ __launch_bounds__(THREADS) void tile_band_out_kernel(View xv, View yv
 // that those rows' bands cover.  P3 (TRANSPOSED = true): output rows o0.., contraction over the
 // band rows lo..hi that reach them.  In both the band entry of (row r, column col) is A[r, col - r + w].
 template <class T, bool TRANSPOSED, bool A_FAST, bool Y_FAST>
-__global__ __launch_bounds__(THREADS) void tile_band_in_kernel(View av, View yv, View cv, int64_t M, int64_t N,
-                                                               int64_t w, int64_t tiles) {
+__global__ __launch_bounds__(THREADS) void tile_band_in_kernel(View av, View yv, View cv, int B, int64_t M,
+                                                               int64_t N, int64_t w, int64_t tiles) {
   typedef typename Acc<T>::type C;
   __shared__ Stage<C> t;
-  const int64_t b = blockIdx.x / tiles, o0 = (blockIdx.x % tiles) * TS, h0 = (int64_t)blockIdx.y * TS;
+  int b, blk;
+  if (!decode_block((int)tiles, B, &b, &blk)) return;
+  const int64_t o0 = (int64_t)blk * TS, h0 = (int64_t)blockIdx.y * TS;
   const Rows<T> a(av, b), y(yv, b), c(cv, b);
   const int64_t lo = o0 > w ? o0 - w : 0, hi = o0 + TS - 1 + w < M - 1 ? o0 + TS - 1 + w : M - 1;
   typename Mma<C>::acc_t acc[2][2] = {};
@@ -226,24 +230,24 @@ void with_flags(bool first, bool second, F launch) {
 template <class T>
 void launch_band_out(const Problem &p, const View &x, const View &y, const View &c) {
   const int64_t tiles = (p.M + TS - 1) / TS;
-  const dim3 grid((unsigned)(p.B * tiles)), block(THREADS);
+  const dim3 grid((unsigned)tiled_grid(p.B, tiles)), block(THREADS);
   with_flags(rows_closer(x), rows_closer(y), [&](auto x_fast, auto y_fast) {
     hipLaunchKernelGGL((tile_band_out_kernel<T, decltype(x_fast)::value, decltype(y_fast)::value>), grid, block, 0,
-                       p.stream, x, y, c, p.M, p.N, p.w, tiles);
+                       p.stream, x, y, c, (int)p.B, p.M, p.N, p.w, tiles);
   });
 }
 
 template <class T, bool TRANSPOSED>
 void launch_band_in(const Problem &p, const View &a, const View &y, const View &c) {
   const int64_t tiles = (p.M + TS - 1) / TS;
-  const dim3 grid((unsigned)(p.B * tiles), (unsigned)((p.N + TS - 1) / TS)), block(THREADS);
+  const dim3 grid((unsigned)tiled_grid(p.B, tiles), (unsigned)((p.N + TS - 1) / TS)), block(THREADS);
   // Band tile: neighbouring staged elements along the output rows lie sr - sc apart in memory
   // (band-in) or sc apart (transposed band-in); along the contraction sc or sr - sc.
   const int64_t along_m = TRANSPOSED ? llabs(a.sc) : llabs(a.sr - a.sc);
   const int64_t along_k = TRANSPOSED ? llabs(a.sr - a.sc) : llabs(a.sc);
   with_flags(along_m < along_k, !rows_closer(y), [&](auto a_fast, auto y_fast) {
     hipLaunchKernelGGL((tile_band_in_kernel<T, TRANSPOSED, decltype(a_fast)::value, decltype(y_fast)::value>), grid,
-                       block, 0, p.stream, a, y, c, p.M, p.N, p.w, tiles);
+                       block, 0, p.stream, a, y, c, (int)p.B, p.M, p.N, p.w, tiles);
   });
 }
 
