@@ -62,7 +62,7 @@ for _w in (1, 33, 1500):
                 B=7, M=3001, N=80, w=_w, dtype=_dt, qk_scale=1.0, backward=True,
                 label=f"B7 M3001 N80 w{_w} {_dt}, window->softmax->unwindow, fwd+bwd")
 # source files of the kernels whose HBM traffic profiles/config3_bf16_hbm_traffic.md records
-TRAFFIC_SOURCES = ("wm_mfma.hip", "wm_mfma_common.hpp")
+TRAFFIC_SOURCES = ("wm_mfma.hip", "wm_mfma_common.hpp", "wm_common.hpp")
 
 
 def band_unit_flops(B, M, N, w):
