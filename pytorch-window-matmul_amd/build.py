@@ -61,9 +61,12 @@ def build_hip_library(force=False):
         return HIP_LIB
     objs = []
     procs = []
+    headers = [d for d in deps if d not in sources]
     for src in sources:
         obj = os.path.join(CSRC, os.path.basename(src)[:-4] + ".o")
         objs.append(obj)
+        if not force and _newer(obj, [src] + headers):
+            continue  # this object is still current: only stale translation units are recompiled
         cmd = [os.path.join(ROCM, "bin", "hipcc"), *HIPCC_FLAGS, "-c", src, "-o", obj]
         print("+", " ".join(cmd), flush=True)
         procs.append((cmd, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)))
