@@ -203,8 +203,10 @@ int wm_window_attention_backward_static(const wm_operand *q, const wm_operand *k
  * replaces the copy the reference makes on entry (`B.transpose(-1, -2).contiguous()`, reference
  * cuda/window_matmul_cuda.cu:236, 285) and runs at memory speed (one read and one write of the
  * tensor).  Callers that hold key rows already (key.transpose(-1, -2) of a row-major tensor) skip it.
- * WM_ERR_UNSUPPORTED, nothing launched, unless k has unit column stride, rows is 16-byte aligned
- * and N is a multiple of 16 bytes (any M, any row stride). */
+ * WM_ERR_UNSUPPORTED, nothing launched, unless k has unit column stride, rows is 16-byte aligned,
+ * N is a multiple of 16 bytes, the row stride of k is at least M (rows may be padded, they may not
+ * overlap or run backwards), B <= 65535 and N <= 64 * 65535 (any M).  Callers fall back to their
+ * own copy on that status, as the PyTorch extension does. */
 int wm_key_rows(const wm_operand *k, void *rows, int64_t B, int64_t N, int64_t M, int dtype, void *stream);
 
 /* 1 if the fused kernels exist for this shape, dtype and scale (layout aside), else 0. */

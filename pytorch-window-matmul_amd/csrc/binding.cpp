@@ -13,6 +13,8 @@
 #include <torch/extension.h>
 
 #include <algorithm>
+#include <stdexcept>
+#include <string>
 #include <vector>
 
 #include <ATen/hip/impl/HIPGuardImplMasqueradingAsCUDA.h>
@@ -414,6 +416,13 @@ window_attention_backward(torch::Tensor q, torch::Tensor k, torch::Tensor v, tor
 
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.doc() = "MI355X banded matmul kernels behind the window_matmul package";
+  // The argument lists and workspace sizes of the C ABI change with WM_ABI_VERSION (version 4 doubled
+  // the float workspace of wm_window_attention_backward to 2 B M values): a library of another
+  // version next to this module would be called with the wrong contract, so refuse to load.
+  if (wm_abi_version() != WM_ABI_VERSION)
+    throw std::runtime_error("window_matmul_kernel was built against ABI " + std::to_string(WM_ABI_VERSION) +
+                             " of libwindow_matmul_hip.so, the library that was loaded reports " +
+                             std::to_string(wm_abi_version()));
   m.def("window_matmul_forward", &window_matmul_forward, "WindowMatmul forward");
   m.def("window_matmul_backward", &window_matmul_backward, "WindowMatmul backward", py::arg("src"), py::arg("other"),
         py::arg("window_size"), py::arg("grad_output"), py::arg("need_src") = true, py::arg("need_other") = true);

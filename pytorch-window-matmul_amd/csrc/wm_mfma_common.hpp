@@ -264,13 +264,13 @@ __device__ __forceinline__ u32x4 make_rsrc(const void *p, uint32_t bytes) {
 // compiler would make every later LDS read wait for all such loads in flight (it cannot tell the
 // tiles apart), which is exactly the wait a multi-stage pipeline must not have.  The kernels
 // count these loads themselves (wait_vmcnt) before the barrier that publishes a tile.  M0 is
-// written here and is not on the clobber list (it is a reserved register; the compiler sets it
-// right before each of its own uses, none of which these kernels contain).
+// written here and named as clobbered, so that a use of M0 the compiler makes itself (dynamic
+// register indexing, its own LDS-direct loads) is set up again after this statement.
 __device__ __forceinline__ void dma_piece(u32x4 rsrc, uint32_t lds_base, uint32_t voff, uint32_t soff) {
   asm volatile("s_mov_b32 m0, %3\n\ts_nop 0\n\tbuffer_load_dwordx4 %0, %1, %2 offen lds"
                :
                : "v"(voff), "s"(rsrc), "s"(soff), "s"(lds_base)
-               : "memory");
+               : "memory", "m0");
 }
 // The same marked non-temporal, for data that is read exactly once and in whole cache lines (a band
 // whose column groups are lines): it should not push the rows that neighbouring workgroups share out
@@ -279,14 +279,14 @@ __device__ __forceinline__ void dma_piece_streaming(u32x4 rsrc, uint32_t lds_bas
   asm volatile("s_mov_b32 m0, %3\n\ts_nop 0\n\tbuffer_load_dwordx4 %0, %1, %2 offen nt lds"
                :
                : "v"(voff), "s"(rsrc), "s"(soff), "s"(lds_base)
-               : "memory");
+               : "memory", "m0");
 }
 // The same with 4 bytes per lane: 256 consecutive bytes of LDS per wave-level load.
 __device__ __forceinline__ void dma_dword(u32x4 rsrc, uint32_t lds_base, uint32_t voff, uint32_t soff) {
   asm volatile("s_mov_b32 m0, %3\n\ts_nop 0\n\tbuffer_load_dword %0, %1, %2 offen lds"
                :
                : "v"(voff), "s"(rsrc), "s"(soff), "s"(lds_base)
-               : "memory");
+               : "memory", "m0");
 }
 __device__ __forceinline__ uint32_t lds_address(const void *p) {
   return (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const void *)p;

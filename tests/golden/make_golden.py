@@ -34,6 +34,8 @@ CASES = {
     "c5_ragged_w1_f32": dict(B=1, M=151, N=80, w=1, dtype="f32", zero_rows=True),
     "c5_ragged_w33_f32": dict(B=1, M=151, N=80, w=33, dtype="f32", zero_rows=True),
     "c5_ragged_w75_bf16": dict(B=1, M=151, N=80, w=75, dtype="bf16", zero_rows=True),
+    # float32 with a band that covers most of the sequence, over more than two 128-row tiles
+    "c5_ragged_w150_f32": dict(B=1, M=301, N=80, w=150, dtype="f32", zero_rows=True),
 }
 
 
@@ -83,6 +85,9 @@ def build(name, cfg, seed):
 
 
 if __name__ == "__main__":
+    only = sys.argv[1:]  # fixture names to (re)write; all of them when none is given
     for n, (name, cfg) in enumerate(CASES.items()):
+        if only and name not in only:
+            continue
         ok = build(name, cfg, seed=1000 + n)
         print(f"{name}: written (bit-identical to the compiled reference: {ok})")

@@ -27,7 +27,7 @@ def load(path):
 
 
 def test_fixtures_exist_and_were_checked_against_the_reference():
-    assert len(FIXTURES) == 7
+    assert len(FIXTURES) == 8
     for path in FIXTURES:
         assert load(path)[3], path
 

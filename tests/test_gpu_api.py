@@ -261,15 +261,17 @@ def test_views_at_a_misaligned_storage_offset(device, dtype):
                                       (torch.float32, 3), (torch.float32, 20), (torch.float32, 50), (torch.float32, 121),
                                       (torch.bfloat16, 160), (torch.float16, 256), (torch.bfloat16, 136), (torch.float32, 200)],
                          ids=lambda x: str(x).replace("torch.", ""))
-@pytest.mark.parametrize("w", [2, 9, 40])
+@pytest.mark.parametrize("w", [2, 9, 40, 300])
 def test_head_widths_between_the_tuned_ones(device, dtype, N, w):
     """A head width that is not a multiple of 16 (16-bit storage) or 8 (float32) is padded with zero
-    columns inside the extension, one beyond 128 is worked on in slices of 128 columns, and both run
-    on the tuned kernels; results, shapes, contiguity and all four gradients are those of the
-    operation on the whole tensors (CPU oracle)."""
+    columns inside the extension, one beyond 128 is worked on in slices of 128 columns (float32 band
+    gradients summed over the slices); results, shapes, contiguity and all four gradients are those of
+    the operation on the whole tensors (CPU oracle).  16-bit storage takes the padded and sliced route
+    at every window; float32 takes it above w = 256 (w = 300 here, with a longer sequence) and runs the
+    tile kernels, which need neither, at the narrower windows."""
     from window_matmul import unwindow_matmul, window_matmul
 
-    B, M = 3, 150
+    B, M = (3, 150) if w < 256 else (2, 700)
     tol = dict(rtol=1e-3, atol=1e-3) if dtype == torch.float32 else dict(rtol=2e-2, atol=2e-2)
     q, k, v = (seeded((B, M, N), 400 + s, dtype) for s in range(3))
     a = seeded((B, M, 2 * w + 1), 410, dtype, 0.25)

@@ -3,9 +3,10 @@
 The CPU oracle cannot finish these in seconds, so each is checked three ways:
   * exactly-computed row blocks: for sampled (batch, row range) the expected band rows and
     outputs are formed with small dense float64 matmuls on the GPU (library routines only);
-  * size-independent properties: row sums of the band against a cumulative-sum closed form,
-    the adjoint identities between forward and backward, exact +0.0 outside the sequence,
-    zero rows of q giving exact zero band rows;
+  * size-independent properties: row sums of the band against a cumulative-sum closed form
+    (bounded by the rounding of the stored values themselves, so that one dropped band entry
+    or one dropped value row fails), the adjoint identities between forward and backward,
+    exact +0.0 outside the sequence, zero rows of q giving exact zero band rows;
   * the golden fixtures cover the same workloads at reduced size against the CPU oracle.
 Tolerances: float32 1e-3, bfloat16 / float16 2e-2 (relative and absolute), as stated for the path.
 """
@@ -68,6 +69,18 @@ def check(got, want, tol, what):
     torch.testing.assert_close(got.double(), want, rtol=tol, atol=tol, msg=lambda s: f"{what}: {s}")
 
 
+def storage_eps(dtype):
+    """Largest relative error of rounding a float32 accumulator to `dtype` (float32 results are not
+    rounded again; what differs from an exact sum there is the order of the float32 accumulation)."""
+    return {torch.bfloat16: 2.0 ** -8, torch.float16: 2.0 ** -11, torch.float32: 2.0 ** -24}[dtype]
+
+
+def check_bounded(got, want, bound, what):
+    excess = (got.double() - want).abs() - bound
+    worst = float(excess.max())
+    assert worst <= 0.0, f"{what}: error exceeds its rounding bound by {worst:.3e} (bound there {float(bound.flatten()[excess.argmax()]):.3e})"
+
+
 def run_config(device, B, M, N, w, dtype, tol, qk_scale=1.0, backward=True, zero_rows=False, blocks=3, rows=192,
                uniform_band=False):
     from window_matmul import unwindow_matmul, window_matmul
@@ -103,11 +116,24 @@ def run_config(device, B, M, N, w, dtype, tol, qk_scale=1.0, backward=True, zero
         assert not att.detach()[:, zr].view(torch.int16 if att.element_size() == 2 else torch.int32).any()
 
     # closed forms over the whole tensor: row sums of the band, and unwindow with a band of ones
+    # Bounds from the stored values: each band entry is a float32 accumulation (error at most
+    # N 2^-24 sum_h |q_h k_h|, taken as 4 N 2^-24 |q| . window_sum(|k|) over a row) rounded once to the
+    # storage type (relative error eps, independent from entry to entry: 8 eps times the 2-norm of the
+    # row is beyond ten standard deviations of their sum, and far below one typical entry).
+    eps = storage_eps(dtype)
     ksum = window_sum(k.detach().double(), w)  # (B, M, N)
-    check(att.detach().double().sum(-1), (q.detach().double() * ksum).sum(-1), tol * (2 * w + 1) ** 0.5 * 4, "band row sums")
+    kabs = window_sum(k.detach().double().abs(), w)
+    a64 = att.detach().double()
+    bound = 8 * eps * a64.pow(2).sum(-1).sqrt() + 4 * N * 2.0 ** -24 * (q.detach().double().abs() * kabs).sum(-1) + 1e-6
+    check_bounded(a64.sum(-1), (q.detach().double() * ksum).sum(-1), bound, "band row sums")
+    del a64, kabs, ksum
     ones = torch.ones(B, M, 2 * w + 1, dtype=dtype, device=device)
     ones[:, ~mask] = float("nan")  # must be ignored
-    check(unwindow_matmul(ones, v.detach(), w), window_sum(v.detach().double(), w), tol * (2 * w + 1) ** 0.5 * 4, "sliding sums")
+    # one float32 accumulation of up to 2w+1 value rows, rounded once
+    want = window_sum(v.detach().double(), w)
+    bound = 2 * eps * want.abs() + 4 * (2 * w + 1) * 2.0 ** -24 * window_sum(v.detach().double().abs(), w) + 1e-6
+    check_bounded(unwindow_matmul(ones, v.detach(), w), want, bound, "sliding sums")
+    del ones, want, bound
 
     gA = gV = gQ = gK = None
     if backward:
@@ -124,11 +150,17 @@ def run_config(device, B, M, N, w, dtype, tol, qk_scale=1.0, backward=True, zero
         assert abs(float(lhs - (k.detach().double() * gK.double()).sum())) <= tol * scale + 1e-6
 
     # exactly-computed row blocks
+    # per sampled batch element: both ends of the sequence, a block at a random offset, one that has a
+    # seam between two 128-row tiles in its middle and one around a 64-row chunk seam that is not a tile seam
     gen = torch.Generator().manual_seed(3)
     for _ in range(blocks):
         b = int(torch.randint(B, (1,), generator=gen))
         r0 = int(torch.randint(max(M - rows, 1), (1,), generator=gen))
-        for r0 in (0, r0, max(M - rows, 0)):
+        tile = 128 * int(torch.randint(1, max(M // 128, 2), (1,), generator=gen))
+        chunk = 128 * int(torch.randint(0, max(M // 128, 1), (1,), generator=gen)) + 64
+        starts = {0, r0, max(M - rows, 0), min(max(tile - rows // 2, 0), max(M - rows, 0)),
+                  min(max(chunk - rows // 2, 0), max(M - rows, 0))}
+        for r0 in sorted(starts):
             r1 = min(r0 + rows, M)
             check(att.detach()[b, r0:r1], band_rows_expected(q.detach(), k.detach(), w, b, r0, r1), tol, "window fwd")
             check(out.detach()[b, r0:r1], unwindow_rows_expected(probs.detach(), v.detach(), w, b, r0, r1), tol, "unwindow fwd")
@@ -144,11 +176,11 @@ def test_config2_small_window_bf16(device):
 
 
 def test_config3_local_attention_bf16(device):
-    run_config(device, B=96, M=4096, N=64, w=256, dtype=torch.bfloat16, tol=2e-2, qk_scale=0.125)
+    run_config(device, B=96, M=4096, N=64, w=256, dtype=torch.bfloat16, tol=2e-2, qk_scale=0.125, blocks=6)
 
 
 def test_config4_wide_head_fp16(device):
-    run_config(device, B=16, M=32768, N=128, w=512, dtype=torch.float16, tol=2e-2, blocks=2, uniform_band=True)
+    run_config(device, B=16, M=32768, N=128, w=512, dtype=torch.float16, tol=2e-2, blocks=4, uniform_band=True)
 
 
 @pytest.mark.parametrize("w", [1, 33, 1500])

@@ -37,6 +37,8 @@ EDGE = [
     (2, 300, 64, 40), (3, 201, 32, 63), (2, 150, 48, 57), (1, 700, 16, 33),
     # float32 at N <= 64, w = 12..28: narrow-band MFMA kernels for all three products
     (3, 201, 64, 12), (2, 333, 48, 17), (3, 140, 16, 28), (2, 90, 32, 21),
+    # band that covers the whole sequence over many 128-row tiles (few tiles for the CUs: split tiles)
+    (1, 1100, 80, 1200), (2, 777, 80, 776), (1, 1500, 64, 750),
 ]
 CASES = REF_GRID + EDGE
 DTYPES = [torch.float32, torch.bfloat16, torch.float16, torch.float64]
