@@ -28,6 +28,7 @@
 // output band are stored as +0.0 whatever the operands hold.
 #include "wm_mfma_common.hpp"
 
+#include <algorithm>
 #include <type_traits>
 
 namespace wm {
@@ -369,8 +370,24 @@ __global__ __launch_bounds__(kThreads, RING && NK <= 4 ? 3 : 2) void mfma_p1_ker
   const int i0 = blk * TM;
   const int rows = min(TM, M - i0);
   const int c_lo = i0 - w, c_hi = i0 + rows - 1 + w;  // not clipped: out-of-sequence entries are written as zeros
-  const int c_start = ALIGNED ? c_lo - (int)(((int64_t)c_lo + (int64_t)b * csb + w) & (galign - 1)) : c_lo;
-  const int nk = (c_hi - c_start + KC) / KC;
+  int c_start = ALIGNED ? c_lo - (int)(((int64_t)c_lo + (int64_t)b * csb + w) & (galign - 1)) : c_lo;
+  int nk = (c_hi - c_start + KC) / KC;
+  // A launch with too few tiles for the chip gives every tile to gridDim.y workgroups, each with a
+  // contiguous share of the tile's chunks; the shares write disjoint column ranges of the band rows.
+  // Without the ring nothing is computed twice.  With it a row's line k spans chunks k - 1 and k, so a
+  // share that owns lines [first, last) also computes chunk first - 1, stores nothing after it (the
+  // rows' valid ranges below begin at the share's first line) and leaves the closing step, line
+  // `last`, to the next share.
+  const bool shared_tile = gridDim.y > 1;
+  bool first_share = true, last_share = true;
+  if (shared_tile) {
+    const int total = RING ? nk + 1 : nk;  // lines (the closing step stores line nk) or chunks
+    const int first = (int)((int64_t)total * blockIdx.y / gridDim.y), last = (int)((int64_t)total * (blockIdx.y + 1) / gridDim.y);
+    first_share = first == 0, last_share = last == total;
+    const int k0 = RING && !first_share ? first - 1 : first;
+    c_start += k0 * KC;
+    nk = (RING && last_share ? last - 1 : last) - k0;
+  }
   const uint16_t *Yb = Y + (int64_t)b * ysb;
   uint16_t *Cb = C + (int64_t)b * csb;
   // Head and tail pieces of neighbouring rows meet through the seam buffer when both rows belong
@@ -378,7 +395,9 @@ __global__ __launch_bounds__(kThreads, RING && NK <= 4 ? 3 : 2) void mfma_p1_ker
   // the two tiles (the tail is produced 2w-1 columns after the head: at least two chunks later).
   // (ring: a row's tail line is stored (2w + d' - d) / 64 steps after the head line of the row below,
   // d, d' <= kMaxShift the rows' line offsets: at least one step from 2w - kMaxShift >= 64 on)
-  const bool seam_across_waves = ALIGNED && (RING ? 2 * w - kMaxShift >= KC : 2 * w - 1 >= 2 * KC);
+  // In a shared tile head and tail fall into different workgroups: both leave element by element.
+  const bool seam_in_tile = ALIGNED && !shared_tile;
+  const bool seam_across_waves = seam_in_tile && (RING ? 2 * w - kMaxShift >= KC : 2 * w - 1 >= 2 * KC);
 
   // B-operand: this wave's 32 rows of X, all of N, kept in registers
   u32x4 xop[NK];
@@ -441,6 +460,8 @@ __global__ __launch_bounds__(kThreads, RING && NK <= 4 ? 3 : 2) void mfma_p1_ker
     // element address of (i, c_start) modulo a line: the line that contains it begins that many columns earlier
     st_shift[s] = RING ? (int)((0 - (reinterpret_cast<uintptr_t>(Cb + (int64_t)i * W + (w - i) + c_start) >> 1)) & 63) : 0;
     st_piece[s] = (st_shift[s] >> 3) + g;
+    // a later share of a tile owns the row from the line that its second chunk completes
+    if (RING && !first_share) st_lo[s] = max(i - w, c_start + st_shift[s]) - 8 * g;
   }
   uint16_t *stage_wr = stage + (lane & 31) * SS + 4 * (lane >> 5);
   const int y_rd_off = (lane & 31) * SY + 8 * (lane >> 5);
@@ -466,7 +487,8 @@ __global__ __launch_bounds__(kThreads, RING && NK <= 4 ? 3 : 2) void mfma_p1_ker
       if (RING) return *reinterpret_cast<const u32x4 *>(st_src[s] + ((((st_piece[s] + 8 * ((k + 1) & 1)) & 15) ^ (r & 15)) << 3));
       return *reinterpret_cast<const u32x4 *>(st_src[s]);
     };
-    if (cb - (RING ? KC : 0) >= iw_first + 31 - w && cb + (RING ? kMaxShift : KC) - 1 <= iw_first + w && iw_first + 31 < M) {
+    if (cb - (RING ? KC : 0) >= iw_first + 31 - w && cb + (RING ? kMaxShift : KC) - 1 <= iw_first + w && iw_first + 31 < M &&
+        (!RING || first_share || k > 0)) {
       // every chunk of the wave's tile lies inside the band: nothing to decide, and each group of 8
       // lanes writes one whole 128-byte line, which is what makes the streaming store pay
 #pragma unroll
@@ -493,7 +515,7 @@ __global__ __launch_bounds__(kThreads, RING && NK <= 4 ? 3 : 2) void mfma_p1_ker
           if (e_lo <= 0 && e_hi >= 7) {
             store_chunk<ALIGNED>(dst, v[s]);  // (plain: lines of edge tiles are completed piecewise)
           } else if (e_lo > 0) {  // head piece: elements e_lo..7 (W >= 17, so it reaches the chunk's end)
-            if (ALIGNED && rw > 0 && (r > 0 || seam_across_waves))
+            if (seam_in_tile && rw > 0 && (r > 0 || seam_across_waves))
               *reinterpret_cast<u32x4 *>(&seam[rw * 8]) = v[s];
             else
               store_chunk_elements(dst, v[s], e_lo, 7);
@@ -509,7 +531,7 @@ __global__ __launch_bounds__(kThreads, RING && NK <= 4 ? 3 : 2) void mfma_p1_ker
         if (tail_hi[s] >= 0) {
           const int rw = wave * 32 + (lane >> 3) + 8 * s, r = rw & 31;
           uint16_t *dst = st_dst[s] + cb_of(s);
-          if (ALIGNED && rw + 1 < TM && i0 + rw + 1 < M && (r < 31 || seam_across_waves)) {
+          if (seam_in_tile && rw + 1 < TM && i0 + rw + 1 < M && (r < 31 || seam_across_waves)) {
             const u32x4 head = *reinterpret_cast<const u32x4 *>(&seam[(rw + 1) * 8]);
             const u32x4 mine_part = keep_range(v[s], 0, tail_hi[s]);
             const u32x4 head_part = keep_range(head, tail_hi[s] + 1, 7);
@@ -587,7 +609,7 @@ __global__ __launch_bounds__(kThreads, RING && NK <= 4 ? 3 : 2) void mfma_p1_ker
     slot(k + 1, y_reg[1], y_reg[0]);
   }
   if (k < nk) slot(k, y_reg[0], y_reg[1]);
-  if (RING) store_lines(nk);  // every wavefront is past the last barrier; lines that end after the last chunk
+  if (RING && last_share) store_lines(nk);  // every wavefront is past the last barrier; lines that end after the last chunk
 }
 
 // ------------------------------------------------------------------------------------------
@@ -827,7 +849,9 @@ constexpr int kShallowChunksBelow = WM_P3_SHALLOW_BELOW;  // window sizes below 
 template <typename T, int NK, int KCH, int STAGES>
 __global__ __launch_bounds__(kThreads, (160 * 1024 / (STAGES * KCH * (2 * TM + (NK <= 4 ? 128 : 256))) >= 4
                                            ? 4
-                                           : 160 * 1024 / (STAGES * KCH * (2 * TM + (NK <= 4 ? 128 : 256))) >= 3 ? 3 : 2)) void mfma_p3_dma_kernel(
+                                           : 160 * 1024 / (STAGES * KCH * (2 * TM + (NK <= 4 ? 128 : 256))) >= 3
+                                                 ? 3
+                                                 : 160 * 1024 / (STAGES * KCH * (2 * TM + (NK <= 4 ? 128 : 256))) >= 2 ? 2 : 1)) void mfma_p3_dma_kernel(
     const uint16_t *__restrict__ A, const uint16_t *__restrict__ Y, uint16_t *__restrict__ C, int B, int M, int w,
     int nblk, int galign, int64_t asb, int64_t ysb, int64_t ysr, int64_t csb, int64_t csr) {
   constexpr int N = 16 * NK, NT = (NK + 1) / 2, CH = KCH, DEPTH = STAGES - 1;
@@ -944,7 +968,9 @@ __global__ __launch_bounds__(kThreads, (160 * 1024 / (STAGES * KCH * (2 * TM + (
 // begin before dense column 0: its position goes into the lanes' offsets, so that exactly the
 // pieces before the buffer read as zeros.
 template <typename T, int NK, int STAGES>
-__global__ __launch_bounds__(kThreads, (160 * 1024 / (STAGES * KC * (2 * TM + (NK <= 4 ? 128 : 256))) >= 3 ? 3 : 2)) void mfma_p2_dma_kernel(
+__global__ __launch_bounds__(kThreads, (160 * 1024 / (STAGES * KC * (2 * TM + (NK <= 4 ? 128 : 256))) >= 3
+                                           ? 3
+                                           : 160 * 1024 / (STAGES * KC * (2 * TM + (NK <= 4 ? 128 : 256))) >= 2 ? 2 : 1)) void mfma_p2_dma_kernel(
     const uint16_t *__restrict__ A, const uint16_t *__restrict__ Y, uint16_t *__restrict__ C, int B, int M, int w,
     int nblk, int galign, int64_t asb, int64_t ysb, int64_t ysr, int64_t csb, int64_t csr) {
   constexpr int N = 16 * NK, NT = (NK + 1) / 2, DEPTH = STAGES - 1;
@@ -1072,6 +1098,16 @@ int band_group(const View &v, int64_t w) { return (w % 32 == 0 && ((uintptr_t)v.
 
 unsigned grid_size(int64_t B, int64_t nblk) { return (unsigned)tiled_grid(B, nblk); }
 
+// Workgroups per tile for a launch of `tiles` tiles whose chunk loops are `chunks` long: one while
+// the tiles fill the chip's 256 CUs, otherwise enough to keep about three per CU resident, each with
+// at least four chunks.
+constexpr int kCUs = 256;
+unsigned tile_shares(int64_t tiles, int64_t chunks) {
+  if (tiles >= kCUs || chunks < 8) return 1;
+  const int64_t want = (3 * kCUs + tiles - 1) / tiles;
+  return (unsigned)std::max<int64_t>(1, std::min<int64_t>({want, chunks / 4, 64}));
+}
+
 // Shapes the kernels that load their tiles straight into LDS accept (band-in products): 32-bit byte
 // offsets inside a batch element of the band and of Y (chunks past the end included), and band rows
 // that can be cut into 16-byte pieces at 4-byte aligned addresses.  Returns the column-group
@@ -1100,14 +1136,15 @@ hipError_t launch_p2(const Problem &p, const View &a, const View &y, const View 
   // the band outgrows the last-level cache the kernel below, with two chunks per workgroup in flight,
   // is 2-4 % faster at N = 64 (B = 384 at w = 256; B = 32, M = 32768 at w = 512): not worth a rule.
   if (const int g = lds_direct_group<ALIGNED>(p, a, y)) {
-#define WM_P2_DMA(NK)                                                                                          \
+#define WM_P2_DMA(NK, STAGES)                                                                                  \
   case NK:                                                                                                     \
-    hipLaunchKernelGGL((mfma_p2_dma_kernel<T, NK, 2>), grid, block, 0, p.stream, (const uint16_t *)a.data,     \
+    hipLaunchKernelGGL((mfma_p2_dma_kernel<T, NK, STAGES>), grid, block, 0, p.stream, (const uint16_t *)a.data, \
                        (const uint16_t *)y.data, (uint16_t *)c.data, (int)p.B, (int)p.M, (int)p.w, nblk, g,    \
                        a.sb, y.sb, y.sr, c.sb, c.sr);                                                          \
     break;
     switch (p.N / 16) {
-      WM_P2_DMA(1) WM_P2_DMA(2) WM_P2_DMA(3) WM_P2_DMA(4) WM_P2_DMA(5) WM_P2_DMA(6) WM_P2_DMA(7) WM_P2_DMA(8)
+      WM_P2_DMA(1, 2) WM_P2_DMA(2, 2) WM_P2_DMA(3, 2) WM_P2_DMA(4, 2) WM_P2_DMA(5, 2) WM_P2_DMA(6, 2) WM_P2_DMA(7, 2)
+      WM_P2_DMA(8, 2)
     }
 #undef WM_P2_DMA
     return hipGetLastError();
@@ -1179,15 +1216,25 @@ template <typename T, bool ALIGNED>
 hipError_t launch_p1(const Problem &p, const View &x, const View &y, const View &c) {
   const int nblk = (int)((p.M + TM - 1) / TM);
   const int galign = band_group(c, p.w);
-  const dim3 grid(grid_size(p.B, nblk)), block(kThreads);
+  const dim3 block(kThreads);
+  dim3 grid(grid_size(p.B, nblk));
   // 16-byte column groups: every row is stored as two partial lines per chunk.  While the band fits
   // the last-level cache (256 MB) the halves meet there and plain stores do (B96 M4096 N64 w = 100,
   // 158 MB: 62 us, against 67 us with the ring of whole lines); beyond it the ring wins: 91 against
   // 116 us at w = 164 (259 MB), 119 against 200 us at w = 260, 327 against 747 us at w = 1028.
-  const bool ring_pays = p.B * p.M * (2 * p.w + 1) * 2 >= (int64_t)220 << 20;
+  // Fewer tiles than CUs (a wide band over a short sequence, few batch elements): a workgroup alone
+  // on its CU is bound by the latency of its chunk loop, about 1.3 us per chunk whatever runs beside
+  // it, so the tiles are shared out until about three workgroups per CU are resident, each with at
+  // least four chunks (B7 M3001 N80 w1500 bf16, 168 tiles: 65 -> 40 us).
+  // A launch with fewer tiles than CUs shares its tiles out and then runs several times as many
+  // workgroups as before, whose partial lines no longer meet in the caches: ring there as well
+  // (B7 M3001 N80 w1500, 126 MB: 40 against 45 us into one buffer, 40 against 65 us into a rotation of nine).
+  const unsigned shares = tile_shares(p.B * nblk, (TM + 2 * p.w) / KC + 1);
+  const bool ring_pays = p.B * p.M * (2 * p.w + 1) * 2 >= (int64_t)220 << 20 || shares > 1;
   // windows that are not a multiple of 4: the same with lines at any even column offset, which needs
   // the band 4-byte aligned (138-150 against 205 us at B96 M4096 N64, w = 255, 257, 258)
   const bool ring_unaligned = !(p.flags & WM_FLAG_NO_ALIGNED_BAND) && ((uintptr_t)c.data % 4) == 0;
+  grid.y = shares;
 #define WM_P1_LAUNCH(NK, AL, RING, LINES, G)                                                                 \
   hipLaunchKernelGGL((mfma_p1_kernel<T, NK, AL, RING, LINES>), grid, block, 0, p.stream,                     \
                      (const uint16_t *)x.data, (const uint16_t *)y.data, (uint16_t *)c.data, (int)p.B,       \
@@ -1208,7 +1255,8 @@ hipError_t launch_p1(const Problem &p, const View &x, const View &y, const View 
       (p.M + 2 * KC) * y.sr * 2 < 0x7fffffff && p.N == 128) {
     // (at N = 64, where the kernel above already places four workgroups on a CU, this variant measured
     // equal at w = 256 and 512 and 8 % slower at w = 64)
-    hipLaunchKernelGGL((mfma_p1_dma_kernel<T, 8, ALIGNED>), grid, block, 0, p.stream, (const uint16_t *)x.data,
+    // (one workgroup per tile: this kernel does not share tiles out)
+    hipLaunchKernelGGL((mfma_p1_dma_kernel<T, 8, ALIGNED>), dim3(grid.x), block, 0, p.stream, (const uint16_t *)x.data,
                        (const uint16_t *)y.data, (uint16_t *)c.data, (int)p.B, (int)p.M, (int)p.w, nblk, galign, x.sb,
                        x.sr, y.sb, y.sr, c.sb);
     return hipGetLastError();
