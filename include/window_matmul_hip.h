@@ -62,6 +62,7 @@ typedef enum wm_status {
 #define WM_FLAG_NO_ALIGNED_BAND 0x2u /* MFMA kernels: never use the 16-byte aligned band variant */
 #define WM_FLAG_NO_NARROW_BAND 0x4u  /* never use the narrow-band kernels (MFMA, w <= 63; vector ALU, w <= 14; fused attention, w <= 64) */
 #define WM_FLAG_NO_LDS_DIRECT 0x8u   /* never use the kernels that load chunks straight into LDS (fused attention; band-out product at N = 128) */
+#define WM_FLAG_NO_SPLIT_F32 0x10u   /* float32: never use the kernels that run on the bf16 matrix instruction through an exact three-way split */
 
 /* Rank-3 operand: element (b, r, c) lives at data + b*stride_b + r*stride_r + c*stride_c. */
 typedef struct wm_operand {

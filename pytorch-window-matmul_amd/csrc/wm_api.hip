@@ -33,7 +33,7 @@ int static_scratch(float **out) {
 
 int check_common(int64_t B, int64_t M, int64_t N, int64_t w, int dtype, unsigned flags) {
   if (dtype < WM_DTYPE_F32 || dtype > WM_DTYPE_F64) return WM_ERR_BAD_DTYPE;
-  if (flags & ~(WM_FLAG_FORCE_STRIDED | WM_FLAG_NO_ALIGNED_BAND | WM_FLAG_NO_NARROW_BAND | WM_FLAG_NO_LDS_DIRECT)) return WM_ERR_BAD_FLAGS;
+  if (flags & ~(WM_FLAG_FORCE_STRIDED | WM_FLAG_NO_ALIGNED_BAND | WM_FLAG_NO_NARROW_BAND | WM_FLAG_NO_LDS_DIRECT | WM_FLAG_NO_SPLIT_F32)) return WM_ERR_BAD_FLAGS;
   const int64_t lim = 0x7fffffff;
   if (B < 0 || M < 0 || N < 0 || w < 0) return WM_ERR_BAD_SHAPE;
   if (B > lim || M > lim || N > lim || w > (lim - 1) / 2) return WM_ERR_BAD_SHAPE;
@@ -257,6 +257,10 @@ const char *wm_kernel_choice(int op, int64_t B, int64_t M, int64_t N, int64_t w,
     }
     if (mfma_supports(op, B, M, N, w, dtype)) {
       static const char *names[] = {"mfma_p1", "mfma_p2", "mfma_p3"};
+      return names[op - 1];
+    }
+    if (f32_split_supports(op, M, N, w, dtype, flags)) {
+      static const char *names[] = {"f32_split_p1", "f32_split_p2", "f32_split_p3"};
       return names[op - 1];
     }
     if (f32_supports(op, M, N, w, dtype)) {

@@ -89,6 +89,12 @@ bool try_launch_f32_p1(const Problem &p, const View &x, const View &y, const Vie
 bool try_launch_f32_p2(const Problem &p, const View &a, const View &y, const View &c, hipError_t *err);
 bool try_launch_f32_p3(const Problem &p, const View &a, const View &y, const View &c, hipError_t *err);
 bool f32_supports(int op, int64_t M, int64_t N, int64_t w, int dtype);
+// The same products on the bf16 matrix instruction through an exact three-way split of every float32
+// value (wm_f32_split.hip); taken ahead of the kernels above from a window size on.
+bool try_launch_f32_split_p1(const Problem &p, const View &x, const View &y, const View &c, hipError_t *err);
+bool try_launch_f32_split_p2(const Problem &p, const View &a, const View &y, const View &c, hipError_t *err);
+bool try_launch_f32_split_p3(const Problem &p, const View &a, const View &y, const View &c, hipError_t *err);
+bool f32_split_supports(int op, int64_t M, int64_t N, int64_t w, int dtype, unsigned flags);
 // Tile family: float64, and whatever the families above decline in 16-bit and float32 storage;
 // 64 x 64 tiles on the 16x16x4 matrix instructions, any strides, any N and w.
 bool try_launch_tile_p1(const Problem &p, const View &x, const View &y, const View &c, hipError_t *err);

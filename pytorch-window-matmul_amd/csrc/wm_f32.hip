@@ -502,18 +502,21 @@ bool f32_supports(int op, int64_t M, int64_t N, int64_t w, int dtype) {
 }
 
 bool try_launch_f32_p1(const Problem &p, const View &x, const View &y, const View &c, hipError_t *err) {
+  if (try_launch_f32_split_p1(p, x, y, c, err)) return true;
   if (!f32_shape_ok(p.M, p.N, p.w, p.dtype)) return false;
   if (!fast_layout(x, p.dtype) || !fast_layout(y, p.dtype) || !f32_band_ok(c, 2 * p.w + 1)) return false;
   *err = launch_band_out(p, x, y, c);
   return true;
 }
 bool try_launch_f32_p2(const Problem &p, const View &a, const View &y, const View &c, hipError_t *err) {
+  if (try_launch_f32_split_p2(p, a, y, c, err)) return true;
   if (!f32_shape_ok(p.M, p.N, p.w, p.dtype)) return false;
   if (!f32_band_ok(a, 2 * p.w + 1) || !fast_layout(y, p.dtype) || !fast_layout(c, p.dtype)) return false;
   *err = launch_band_in<false>(p, a, y, c);
   return true;
 }
 bool try_launch_f32_p3(const Problem &p, const View &a, const View &y, const View &c, hipError_t *err) {
+  if (try_launch_f32_split_p3(p, a, y, c, err)) return true;
   if (!f32_shape_ok(p.M, p.N, p.w, p.dtype)) return false;
   if (!f32_band_ok(a, 2 * p.w + 1) || !fast_layout(y, p.dtype) || !fast_layout(c, p.dtype)) return false;
   *err = launch_band_in<true>(p, a, y, c);

@@ -20,6 +20,7 @@ FORCE_STRIDED = 0x1
 NO_ALIGNED_BAND = 0x2
 NO_NARROW_BAND = 0x4
 NO_LDS_DIRECT = 0x8
+NO_SPLIT_F32 = 0x10
 
 
 class Operand(ctypes.Structure):

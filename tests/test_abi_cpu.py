@@ -56,7 +56,11 @@ def test_kernel_choice_names():
     assert L.wm_kernel_choice(2, 2, 128, 64, 4, 3, 1, abi.FORCE_STRIDED) == b"strided_p2"
     assert L.wm_kernel_choice(9, 2, 128, 64, 4, 0, 1, 0) == b"invalid"
     # per family: float32 MFMA, 16-bit wide band, 16-bit narrow band (P1 any w <= 32, P2 and P3 for w % 4 == 0)
-    assert L.wm_kernel_choice(1, 7, 3001, 80, 1500, 0, 1, 0) == b"f32_mfma_p1"
+    assert L.wm_kernel_choice(1, 7, 3001, 80, 1500, 0, 1, 0) == b"f32_split_p1"  # float32 on the bf16 matrix instruction
+    assert L.wm_kernel_choice(1, 7, 3001, 80, 1500, 0, 1, abi.NO_SPLIT_F32) == b"f32_mfma_p1"
+    assert L.wm_kernel_choice(3, 7, 3001, 80, 15, 0, 1, 0) == b"f32_mfma_p3"     # below w = 16: the float32 instruction
+    assert L.wm_kernel_choice(2, 96, 4096, 32, 64, 0, 1, 0) == b"f32_mfma_p2"    # one 32-column block: no gain from the split
+    assert L.wm_kernel_choice(3, 96, 4096, 32, 64, 0, 1, 0) == b"f32_split_p3"
     assert L.wm_kernel_choice(2, 96, 4096, 64, 256, 2, 1, 0) == b"mfma_p2"
     assert L.wm_kernel_choice(1, 96, 16384, 64, 8, 2, 1, 0) == b"narrow_p1"
     assert L.wm_kernel_choice(2, 96, 16384, 64, 8, 1, 1, 0) == b"narrow_p2"
@@ -96,7 +100,7 @@ def test_kernel_choice_names():
     assert L.wm_kernel_choice(2, 96, 16384, 64, 3, 0, 1, 0) == b"vector_p2"
     assert L.wm_kernel_choice(1, 2, 128, 64, 4, 0, 1, 0) == b"narrow_p1"
     assert L.wm_kernel_choice(1, 2, 128, 48, 31, 0, 1, 0) == b"narrow_p1"
-    assert L.wm_kernel_choice(1, 2, 128, 64, 32, 0, 1, 0) == b"f32_mfma_p1"
+    assert L.wm_kernel_choice(1, 2, 128, 64, 32, 0, 1, 0) == b"f32_split_p1"
     assert L.wm_kernel_choice(1, 2, 128, 128, 4, 0, 1, 0) == b"vector_p1"
     assert L.wm_kernel_choice(1, 2, 128, 24, 4, 0, 1, 0) == b"vector_p1"
     assert L.wm_kernel_choice(3, 96, 16384, 64, 11, 0, 1, 0) == b"vector_p3"
@@ -106,7 +110,8 @@ def test_kernel_choice_names():
     assert L.wm_kernel_choice(3, 96, 16384, 64, 12, 0, 1, 0) == b"narrow_p3"
     assert L.wm_kernel_choice(2, 96, 16384, 32, 15, 0, 1, 0) == b"narrow_p2"
     assert L.wm_kernel_choice(2, 96, 16384, 16, 28, 0, 1, 0) == b"narrow_p2"
-    assert L.wm_kernel_choice(2, 96, 16384, 64, 29, 0, 1, 0) == b"f32_mfma_p2"
+    assert L.wm_kernel_choice(2, 96, 16384, 64, 29, 0, 1, 0) == b"f32_split_p2"
+    assert L.wm_kernel_choice(2, 96, 16384, 64, 29, 0, 1, abi.NO_SPLIT_F32) == b"f32_mfma_p2"
     assert L.wm_kernel_choice(1, 96, 16384, 64, 8, 0, 1, abi.NO_NARROW_BAND) == b"f32_mfma_p1"
     assert L.wm_kernel_choice(1, 2, 128, 3, 4, 0, 1, 0) == b"tile_p1"  # N not a multiple of 8
     assert L.wm_kernel_choice(1, 2, 128, 64, 4, 2, 0, 0) == b"tile_p1"  # layout not vector friendly

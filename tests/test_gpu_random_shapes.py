@@ -106,11 +106,13 @@ def test_every_narrow_window(device, dtype, B, M, N, w):
 
 
 # one shape per float32 kernel family, against the CPU oracle itself (kernel_choice names the family)
-F32_FAMILIES = [("vector_p2", 3, 300, 80, 4), ("narrow_p2", 2, 333, 64, 16), ("f32_mfma_p2", 2, 400, 80, 64),
-                ("narrow_p1", 3, 257, 48, 24), ("f32_mfma_p1", 1, 515, 128, 100), ("vector_p3", 2, 129, 24, 9)]
+F32_FAMILIES = [("vector_p2", 3, 300, 80, 4), ("narrow_p2", 2, 333, 64, 16), ("f32_mfma_p2", 2, 400, 80, 15),
+                ("narrow_p1", 3, 257, 48, 24), ("f32_mfma_p1", 1, 515, 128, 15), ("vector_p3", 2, 129, 24, 9),
+                ("f32_split_p2", 2, 400, 80, 64), ("f32_split_p1", 1, 515, 128, 100), ("f32_split_p3", 2, 300, 32, 40),
+                ("f32_mfma_p2", 2, 300, 32, 40), ("f32_split_p1", 2, 260, 24, 130), ("f32_split_p3", 1, 700, 72, 350)]
 
 
-@pytest.mark.parametrize("family,B,M,N,w", F32_FAMILIES, ids=[f[0] for f in F32_FAMILIES])
+@pytest.mark.parametrize("family,B,M,N,w", F32_FAMILIES, ids=[f"{f[0]}-N{f[3]}-w{f[4]}" for f in F32_FAMILIES])
 def test_float32_families_match_the_oracle(device, family, B, M, N, w):
     op = int(family[-1])
     assert abi.lib().wm_kernel_choice(op, B, M, N, w, abi.DTYPES[torch.float32], 1, 0).decode() == family
@@ -156,3 +158,32 @@ def test_fused_attention_agrees_with_chain_of_ops(device, dtype, B, M, N, w):
     _assert_close_in_scale(gq, gq_ref, 2e-2, "grad_q")
     _assert_close_in_scale(gk, gk_ref.transpose(1, 2), 2e-2, "grad_k")
     _assert_close_in_scale(gv, gv_ref, 2e-2, "grad_v")
+
+
+@pytest.mark.parametrize("B,M,N,w", [(2, 700, 80, 300), (1, 515, 128, 100), (2, 300, 32, 40), (3, 200, 8, 16), (1, 1100, 64, 1200)])
+def test_split_float32_kernels_keep_float32_accuracy(device, B, M, N, w):
+    """The float32 products that run on the bf16 matrix instruction (every value cut into three bf16
+    parts, six of the nine partial products kept) against the dense float64 formulation: their largest
+    error may be no more than four times that of the kernels on the float32 matrix instruction
+    (WM_FLAG_NO_SPLIT_F32) on the same inputs, i.e. rounding noise of float32 accumulation, nothing
+    that scales with the 2^-8 of a bf16 operand or the 2^-16 of a two-part split."""
+    g = torch.Generator().manual_seed(7 * N + w)
+    q, k, v, go = (torch.randn(B, M, N, generator=g) * 3.0 for _ in range(4))
+    a, ga = (torch.randn(B, M, 2 * w + 1, generator=g) for _ in range(2))
+    kt = k.transpose(1, 2).contiguous()
+    want = dict(att=oracle.dense_window_matmul(q, kt, w), out=oracle.dense_unwindow_matmul(a, v, w))
+    want["grad_a"], want["grad_v"] = oracle.dense_unwindow_matmul_backward(a, v, w, go)
+    want["grad_q"], gkt = oracle.dense_window_matmul_backward(q, kt, w, ga)
+    want["grad_k"] = gkt.transpose(1, 2)
+    dq, dk, dv, dgo, da, dga = (t.to(device) for t in (q, k, v, go, a, ga))
+    worst = {}
+    for flags in (0, abi.NO_SPLIT_F32):
+        got = dict(att=abi.window_forward(dq, dk.transpose(1, 2), w, flags), out=abi.unwindow_forward(da, dv, w, flags))
+        got["grad_a"], got["grad_v"] = abi.unwindow_backward(da, dv, w, dgo, flags)
+        got["grad_q"], gk = abi.window_backward(dq, dk.transpose(1, 2), w, dga, flags)
+        got["grad_k"] = gk.transpose(1, 2)  # the entry point returns grad_k in the (B, N, M) layout of k
+        worst[flags] = {n: float((got[n].cpu().double() - want[n].double()).abs().max()) for n in want}
+    for n in want:
+        scale = float(want[n].double().abs().max())
+        assert worst[0][n] <= 4 * worst[abi.NO_SPLIT_F32][n] + 1e-7 * scale, (n, worst[0][n], worst[abi.NO_SPLIT_F32][n])
+        assert worst[0][n] <= 2e-5 * scale, (n, worst[0][n], scale)
