@@ -19,16 +19,20 @@ from .band_softmax import band_softmax
 from .window_matmul import unwindow_matmul, window_matmul
 
 
-def _chain_is_faster(window_size: int, width: int) -> bool:
-    """Windows at which a training step is faster through the separate ops than through the fused
-    kernels.  Up to N = 64 the fused backward is one kernel at windows up to 32 and the chain only wins
-    at the very narrowest windows of the narrow heads; above N = 64 the recomputing two-kernel backward
-    costs the same at every narrow window.  Measured on bf16 tensors of 100 M elements with M = 16384
-    (chain / fused, ms per step): N = 16: 0.67 / 0.69 at w = 2, 0.72 / 0.72 at w = 3; N = 32: 0.48 /
-    0.48 at w = 2, 0.50 / 0.48 at w = 3; N = 48: 0.51 / 0.46 at w = 1; N = 64: 0.47 / 0.47 at w = 1,
-    0.48 / 0.45 at w = 2, 0.52 / 0.44 at w = 8, 0.88 / 0.52 at w = 32; N = 96: 0.81 / 0.86 at w = 32,
-    0.96 / 0.92 at w = 40; N = 128: 0.72 / 0.79 at w = 32, 0.86 / 0.84 at w = 40."""
-    return window_size <= (2 if width <= 32 else 0 if width <= 64 else 36)
+def _chain_is_faster(window_size: int, width: int, elements: int) -> bool:
+    """Whether a training step is faster through the separate ops than through the fused kernels.
+    Up to N = 64 the fused backward is one kernel at narrow windows and the fused step wins or ties at
+    every window (N = 16, 32 at w <= 2: 0.67 / 0.69 and 0.48 / 0.48 ms, chain / fused, on 100 M elements:
+    a tie, left to the fused kernels).  Above N = 64 the recomputing two-kernel backward costs the same
+    at every narrow window, and the chain wins up to w = 32 at N = 128 (B16 M32768: 0.374 / 0.535 ms at
+    w = 4, 0.510 / 0.543 at w = 32, 0.588 / 0.580 at w = 36; B96 M4096: 0.378 / 0.395 at w = 32, 0.435 /
+    0.426 at w = 36) and up to about w = 24 at N = 96 (B96 M4096: 0.251 / 0.294 at w = 16, 0.332 / 0.308 at
+    w = 32).  Small problems are bound by the host, which issues seven launches for the chain and three
+    for the fused step: at B7 M3001 the chain takes 0.21 ms and the fused step 0.085-0.09 ms whatever the
+    window and head width, so below about 32 M elements per tensor the fused kernels are always taken."""
+    if width <= 64 or elements < (32 << 20):
+        return False
+    return window_size <= (24 if width <= 96 else 32)
 
 
 class WindowAttentionFunc(torch.autograd.Function):
@@ -73,7 +77,7 @@ def window_attention(query: torch.Tensor, key: torch.Tensor, value: torch.Tensor
     # With a very narrow band the recomputing backward of the fused kernels costs more than the
     # band it avoids writing, so training there goes through the separate ops.
     training = torch.is_grad_enabled() and any(t.requires_grad for t in (q, k, v))
-    if _native.window_attention_supported(q, window_size, scale) and not (training and _chain_is_faster(window_size, q.shape[-1])):
+    if _native.window_attention_supported(q, window_size, scale) and not (training and _chain_is_faster(window_size, q.shape[-1], q.numel())):
         out = WindowAttentionFunc.apply(q, k, v, window_size, scale, bool(mask_out_of_range))
     else:
         att = window_matmul(q, k.transpose(-1, -2), window_size)
