@@ -256,6 +256,13 @@ class Bench:
                 })
             kb = kernel_bytes(B, M, N, w, es)
             per_kernel = {}
+            if cfg["backward"] and B * M <= (1 << 16):
+                # a problem this small pays for launches, not arithmetic: the two backward ops as their callers
+                # issue them (both gradients from one call; the library makes that one launch where it can)
+                launches.update({
+                    "unwindow_bwd(both)": lambda: abi.unwindow_backward(probs, v, w, go, fam),
+                    "window_bwd(both)": lambda: abi.window_backward(q, kt, w, ga, fam),
+                })
             for name, fn in launches.items():
                 ms = single = time_gpu(fn, iters, 3, settle_ms)
                 if single < 0.05:
@@ -298,6 +305,9 @@ class Bench:
             copy_ms = time_gpu(lambda: scratch.copy_(att), iters, 3, settle_ms)
             out["copy_yardstick_GBps"] = round(2 * att.numel() * es / copy_ms / 1e6, 1)
             out["copy_bytes_each_way"] = att.numel() * es
+        both = {n: per_kernel.pop(n) for n in list(per_kernel) if n.endswith("(both)")}
+        if both:
+            out["backward_ops"] = {n: {"ms": x["ms"], "single_launch_ms": x.get("single_launch_ms", x["ms"])} for n, x in both.items()}
         dom = max(per_kernel, key=lambda n: per_kernel[n]["ms"])
         out["slowest_kernel"] = dom
         if per_kernel[dom]["ms"] < 0.03:
@@ -362,6 +372,7 @@ def main():
     if args.kernels_only:
         k = bench.kernels(iters, settle_ms=0.0)
         print(json.dumps({"workload": cfg["label"], "family": args.family, "kernels": k["kernels"],
+                          "backward_ops": k.get("backward_ops"),
                           "fused_attention": k.get("fused_attention"), "band_softmax": k["band_softmax"],
                           "copy_yardstick_GBps": k["copy_yardstick_GBps"],
                           "copy_bytes_each_way": k["copy_bytes_each_way"]}), flush=True)

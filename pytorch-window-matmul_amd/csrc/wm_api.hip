@@ -73,6 +73,11 @@ int run_primitive(mfma_fn narrow, mfma_fn vector, mfma_fn fast, mfma_fn f32, mfm
   return to_status(slow(p, a, y, c));
 }
 
+// The one-launch backward of the vector-ALU kernels stands aside for every flag that selects kernels by hand.
+bool fused_backward_allowed(const Problem &p) {
+  return !(p.flags & (WM_FLAG_FORCE_STRIDED | WM_FLAG_NO_NARROW_BAND)) && tiled_grid_fits(p.B, p.M);
+}
+
 int p1(const Problem &p, const View &x, const View &y, const View &c) {
   return run_primitive(try_launch_small_p1, try_launch_vector_p1, try_launch_mfma_p1, try_launch_f32_p1,
                        try_launch_tile_p1, launch_strided_p1, p, x, y, c);
@@ -112,6 +117,12 @@ int wm_window_matmul_backward(const wm_operand *q, const wm_operand *k, const wm
   if (missing(q) || missing(k) || missing(grad_a)) return WM_ERR_NULL_POINTER;
   if ((grad_q && !grad_q->data) || (grad_k && !grad_k->data)) return WM_ERR_NULL_POINTER;
   const Problem p{B, M, N, w, dtype, flags, (hipStream_t)stream};
+  if (grad_q && grad_k && fused_backward_allowed(p)) {  // small problems: both products in one launch
+    hipError_t err = hipSuccess;
+    if (try_launch_vector_window_backward(p, make_view(grad_a), transposed(make_view(k)), make_view(q), make_view(grad_q),
+                                          transposed(make_view(grad_k)), &err))
+      return to_status(err);
+  }
   if (grad_q)
     if (int st = p2(p, make_view(grad_a), transposed(make_view(k)), make_view(grad_q))) return st;
   if (grad_k)
@@ -136,6 +147,12 @@ int wm_unwindow_matmul_backward(const wm_operand *a, const wm_operand *v, const 
   if ((grad_a && !grad_a->data) || (grad_v && !grad_v->data)) return WM_ERR_NULL_POINTER;
   if (N > 0 && (missing(a) || missing(v) || missing(grad_o))) return WM_ERR_NULL_POINTER;
   const Problem p{B, M, N, w, dtype, flags, (hipStream_t)stream};
+  if (grad_a && grad_v && N > 0 && fused_backward_allowed(p)) {  // small problems: both products in one launch
+    hipError_t err = hipSuccess;
+    if (try_launch_vector_unwindow_backward(p, make_view(a), make_view(v), make_view(grad_o), make_view(grad_a),
+                                            make_view(grad_v), &err))
+      return to_status(err);
+  }
   if (grad_a) {
     const wm_operand none{grad_a->data, 0, 0, 0};  // N == 0: grad_a is all +0.0
     if (int st = p1(p, make_view(N > 0 ? grad_o : &none), make_view(N > 0 ? v : &none), make_view(grad_a)))

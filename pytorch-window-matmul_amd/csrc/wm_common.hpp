@@ -84,6 +84,12 @@ bool try_launch_vector_p1(const Problem &p, const View &x, const View &y, const 
 bool try_launch_vector_p2(const Problem &p, const View &a, const View &y, const View &c, hipError_t *err);
 bool try_launch_vector_p3(const Problem &p, const View &a, const View &y, const View &c, hipError_t *err);
 bool vector_supports(int op, int64_t M, int64_t N, int64_t w, int dtype);
+// Both gradients of an op in one launch of the vector-ALU kernels, for small problems (false: not taken,
+// nothing launched; the caller then launches the two products separately).
+bool try_launch_vector_window_backward(const Problem &p, const View &ga, const View &k, const View &q, const View &gq,
+                                       const View &gk, hipError_t *err);
+bool try_launch_vector_unwindow_backward(const Problem &p, const View &a, const View &v, const View &go, const View &ga,
+                                         const View &gv, hipError_t *err);
 // float32 MFMA family (N multiple of 8 up to 128, w >= 4).
 bool try_launch_f32_p1(const Problem &p, const View &x, const View &y, const View &c, hipError_t *err);
 bool try_launch_f32_p2(const Problem &p, const View &a, const View &y, const View &c, hipError_t *err);

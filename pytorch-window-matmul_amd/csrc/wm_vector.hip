@@ -20,6 +20,8 @@
 // in LDS, one thread per band entry, consecutive threads on consecutive entries of the flat band.  One barrier per workgroup; no atomics.
 #include "wm_mfma_common.hpp"
 
+#include <algorithm>
+
 namespace wm {
 namespace {
 
@@ -71,11 +73,11 @@ struct Elem<f32_t> {
 // TRANSPOSED false: P2 (rows = band rows i).  TRANSPOSED true: P3 (rows = output rows c, the
 // contraction runs over the band rows r = c-w .. c+w).
 template <typename T, int NK, bool TRANSPOSED>  // N = 16 NK (16-bit) or 8 NK (float32): 2 NK pieces per row
-__global__ __launch_bounds__(kThreads) void vector_band_in_kernel(const typename Elem<T>::type *__restrict__ A,
-                                                                  const typename Elem<T>::type *__restrict__ Y,
-                                                                  typename Elem<T>::type *__restrict__ C, int B,
-                                                                  int M, int w, int nblk, int vrows, int64_t asb,
-                                                                  int64_t ysb, int64_t ysr, int64_t csb, int64_t csr) {
+__device__ __forceinline__ void vector_band_in_body(const typename Elem<T>::type *__restrict__ A,
+                                                    const typename Elem<T>::type *__restrict__ Y,
+                                                    typename Elem<T>::type *__restrict__ C, int B, int M, int w,
+                                                    int nblk, int vrows, int64_t asb, int64_t ysb, int64_t ysr,
+                                                    int64_t csb, int64_t csr) {
   typedef typename Elem<T>::type E;
   constexpr int VEC = 16 / sizeof(E);       // elements per 16-byte piece
   constexpr int NCG = 2 * NK, N = NCG * VEC;  // 16-byte column groups per row
@@ -196,6 +198,30 @@ __global__ __launch_bounds__(kThreads) void vector_band_in_kernel(const typename
   }
 }
 
+template <typename T, int NK, bool TRANSPOSED>
+__global__ __launch_bounds__(kThreads) void vector_band_in_kernel(const typename Elem<T>::type *__restrict__ A,
+                                                                  const typename Elem<T>::type *__restrict__ Y,
+                                                                  typename Elem<T>::type *__restrict__ C, int B,
+                                                                  int M, int w, int nblk, int vrows, int64_t asb,
+                                                                  int64_t ysb, int64_t ysr, int64_t csb, int64_t csr) {
+  vector_band_in_body<T, NK, TRANSPOSED>(A, Y, C, B, M, w, nblk, vrows, asb, ysb, ysr, csb, csr);
+}
+
+// Both products of window_matmul's backward in one launch: blockIdx.y = 0 forms grad_q = P2(grad_a, K rows),
+// blockIdx.y = 1 forms grad_k = P3(grad_a, Q).  Same tiles, same LDS images, half the launches: what a small
+// problem pays for is the launch, not the arithmetic.
+template <typename T, int NK>
+__global__ __launch_bounds__(kThreads) void vector_window_backward_kernel(
+    const typename Elem<T>::type *__restrict__ GA, const typename Elem<T>::type *__restrict__ K,
+    const typename Elem<T>::type *__restrict__ Q, typename Elem<T>::type *__restrict__ GQ,
+    typename Elem<T>::type *__restrict__ GK, int B, int M, int w, int nblk, int vrows, int64_t asb, int64_t ksb,
+    int64_t ksr, int64_t qsb, int64_t qsr, int64_t gqsb, int64_t gqsr, int64_t gksb, int64_t gksr) {
+  if (blockIdx.y == 0)
+    vector_band_in_body<T, NK, false>(GA, K, GQ, B, M, w, nblk, vrows, asb, ksb, ksr, gqsb, gqsr);
+  else
+    vector_band_in_body<T, NK, true>(GA, Q, GK, B, M, w, nblk, vrows, asb, qsb, qsr, gksb, gksr);
+}
+
 // x.lo * y.lo + x.hi * y.hi + acc on packed pairs of 16-bit values (v_dot2_f32_bf16 / v_dot2_f32_f16).
 template <typename T>
 __device__ __forceinline__ float dot2(uint32_t x, uint32_t y, float acc);
@@ -212,11 +238,11 @@ __device__ __forceinline__ float dot2<f16_t>(uint32_t x, uint32_t y, float acc) 
 // P1: band[b,i,j] = sum_h X[b,i,h] Y[b,i+j-w,h]  (+0.0 where i+j-w is outside the sequence).
 // One thread per band entry, consecutive threads on consecutive entries of the flat band.
 template <typename T, int NK>  // 2 NK 16-byte pieces per row: N = 16 NK (16-bit) or 8 NK (float32)
-__global__ __launch_bounds__(kThreads) void vector_band_out_kernel(const typename Elem<T>::type *__restrict__ X,
-                                                                   const typename Elem<T>::type *__restrict__ Y,
-                                                                   typename Elem<T>::type *__restrict__ C, int B,
-                                                                   int M, int w, int nblk, int vrows, int64_t xsb,
-                                                                   int64_t xsr, int64_t ysb, int64_t ysr, int64_t csb) {
+__device__ __forceinline__ void vector_band_out_body(const typename Elem<T>::type *__restrict__ X,
+                                                     const typename Elem<T>::type *__restrict__ Y,
+                                                     typename Elem<T>::type *__restrict__ C, int B, int M, int w,
+                                                     int nblk, int vrows, int64_t xsb, int64_t xsr, int64_t ysb,
+                                                     int64_t ysr, int64_t csb) {
   typedef typename Elem<T>::type E;
   constexpr int VEC = 16 / sizeof(E);
   constexpr int NCG = 2 * NK, N = NCG * VEC;
@@ -282,6 +308,30 @@ __global__ __launch_bounds__(kThreads) void vector_band_out_kernel(const typenam
     else
       Cb[item] = sum;
   }
+}
+
+template <typename T, int NK>
+__global__ __launch_bounds__(kThreads) void vector_band_out_kernel(const typename Elem<T>::type *__restrict__ X,
+                                                                   const typename Elem<T>::type *__restrict__ Y,
+                                                                   typename Elem<T>::type *__restrict__ C, int B,
+                                                                   int M, int w, int nblk, int vrows, int64_t xsb,
+                                                                   int64_t xsr, int64_t ysb, int64_t ysr, int64_t csb) {
+  vector_band_out_body<T, NK>(X, Y, C, B, M, w, nblk, vrows, xsb, xsr, ysb, ysr, csb);
+}
+
+// Both products of unwindow_matmul's backward in one launch: blockIdx.y = 0 forms grad_a = P1(grad_o, V) on
+// tiles of `orows` rows, blockIdx.y = 1 forms grad_v = P3(A, grad_o) on tiles of `irows` rows (the two
+// products tile the sequence differently; a workgroup beyond its product's tiles returns at once).
+template <typename T, int NK>
+__global__ __launch_bounds__(kThreads) void vector_unwindow_backward_kernel(
+    const typename Elem<T>::type *__restrict__ A, const typename Elem<T>::type *__restrict__ V,
+    const typename Elem<T>::type *__restrict__ GO, typename Elem<T>::type *__restrict__ GA,
+    typename Elem<T>::type *__restrict__ GV, int B, int M, int w, int oblk, int orows, int iblk, int irows,
+    int64_t asb, int64_t vsb, int64_t vsr, int64_t gosb, int64_t gosr, int64_t gasb, int64_t gvsb, int64_t gvsr) {
+  if (blockIdx.y == 0)
+    vector_band_out_body<T, NK>(GO, V, GA, B, M, w, oblk, orows, gosb, gosr, vsb, vsr, gasb);
+  else
+    vector_band_in_body<T, NK, true>(A, GO, GV, B, M, w, iblk, irows, asb, gosb, gosr, gvsb, gvsr);
 }
 
 // Output rows per workgroup: as many as keep the LDS images of the widest supported window small.
@@ -363,6 +413,93 @@ bool vector_supports(int op, int64_t M, int64_t N, int64_t w, int dtype) {
   if (N < 16 || N > 128 || N % 16 != 0) return false;
   if (op == 1) return false;  // 16-bit band-out: the narrow-band MFMA kernel is faster at every w
   return w <= VECTOR_MAX_W && vector_lds(w, N, dtype) <= 65536;
+}
+
+// One launch for both gradients of an op, for problems so small that the second launch is what they
+// would pay for (at most kFusedTiles tiles per product: a few workgroups per CU).
+constexpr int64_t kFusedTiles = 1024;
+bool vector_16bit_out_ok(int64_t N, int64_t w, int dtype) {  // band-out product in 16-bit storage, fused launches only
+  return (dtype == WM_DTYPE_BF16 || dtype == WM_DTYPE_F16) && N >= 16 && N <= 128 && N % 16 == 0 && w <= VECTOR_MAX_W &&
+         vector_out_lds(w, N, dtype) <= 65536;
+}
+
+bool try_launch_vector_window_backward(const Problem &p, const View &ga, const View &k, const View &q, const View &gq,
+                                       const View &gk, hipError_t *err) {
+  if (!vector_supports(2, p.M, p.N, p.w, p.dtype) || !vector_supports(3, p.M, p.N, p.w, p.dtype)) return false;
+  if (!band_contiguous(ga, 2 * p.w + 1) || !fast_layout(k, p.dtype) || !fast_layout(q, p.dtype) ||
+      !fast_layout(gq, p.dtype) || !fast_layout(gk, p.dtype))
+    return false;
+  const int vrows = vector_rows(p.N, p.dtype);
+  const int nblk = (int)((p.M + vrows - 1) / vrows);
+  if (p.B * nblk > kFusedTiles) return false;
+  const dim3 grid(vector_grid(p.B, nblk), 2), block(kThreads);
+  const size_t lds = vector_lds(p.w, p.N, p.dtype);
+  const int pieces = (int)(p.N * dtype_size(p.dtype) / 16);
+#define WM_VWB(T, NK)                                                                                            \
+  case NK:                                                                                                       \
+    hipLaunchKernelGGL((vector_window_backward_kernel<T, NK>), grid, block, lds, p.stream,                       \
+                       (const typename Elem<T>::type *)ga.data, (const typename Elem<T>::type *)k.data,          \
+                       (const typename Elem<T>::type *)q.data, (typename Elem<T>::type *)gq.data,                \
+                       (typename Elem<T>::type *)gk.data, (int)p.B, (int)p.M, (int)p.w, nblk, vrows, ga.sb, k.sb, \
+                       k.sr, q.sb, q.sr, gq.sb, gq.sr, gk.sb, gk.sr);                                             \
+    break;
+#define WM_VWB_ALL(T)                                                                                  \
+  switch (pieces / 2) {                                                                                \
+    WM_VWB(T, 1) WM_VWB(T, 2) WM_VWB(T, 3) WM_VWB(T, 4) WM_VWB(T, 5) WM_VWB(T, 6) WM_VWB(T, 7) WM_VWB(T, 8)   \
+    WM_VWB(T, 9) WM_VWB(T, 10) WM_VWB(T, 11) WM_VWB(T, 12) WM_VWB(T, 13) WM_VWB(T, 14) WM_VWB(T, 15) WM_VWB(T, 16) \
+    default: return false;                                                                             \
+  }
+  if (p.dtype == WM_DTYPE_BF16) {
+    WM_VWB_ALL(bf16_t)
+  } else if (p.dtype == WM_DTYPE_F16) {
+    WM_VWB_ALL(f16_t)
+  } else {
+    WM_VWB_ALL(f32_t)
+  }
+#undef WM_VWB_ALL
+#undef WM_VWB
+  *err = hipGetLastError();
+  return true;
+}
+
+bool try_launch_vector_unwindow_backward(const Problem &p, const View &a, const View &v, const View &go, const View &ga,
+                                         const View &gv, hipError_t *err) {
+  const bool out_ok = p.dtype == WM_DTYPE_F32 ? vector_supports(1, p.M, p.N, p.w, p.dtype) : vector_16bit_out_ok(p.N, p.w, p.dtype);
+  if (!out_ok || !vector_supports(3, p.M, p.N, p.w, p.dtype)) return false;
+  if (!band_contiguous(a, 2 * p.w + 1) || !band_contiguous(ga, 2 * p.w + 1) || !fast_layout(v, p.dtype) ||
+      !fast_layout(go, p.dtype) || !fast_layout(gv, p.dtype))
+    return false;
+  const int orows = vector_out_rows(p.N, p.dtype), irows = vector_rows(p.N, p.dtype);
+  const int oblk = (int)((p.M + orows - 1) / orows), iblk = (int)((p.M + irows - 1) / irows);
+  if (p.B * oblk > kFusedTiles) return false;
+  const dim3 grid(std::max(vector_grid(p.B, oblk), vector_grid(p.B, iblk)), 2), block(kThreads);
+  const size_t lds = std::max(vector_out_lds(p.w, p.N, p.dtype), vector_lds(p.w, p.N, p.dtype));
+  const int pieces = (int)(p.N * dtype_size(p.dtype) / 16);
+#define WM_VUB(T, NK)                                                                                            \
+  case NK:                                                                                                       \
+    hipLaunchKernelGGL((vector_unwindow_backward_kernel<T, NK>), grid, block, lds, p.stream,                     \
+                       (const typename Elem<T>::type *)a.data, (const typename Elem<T>::type *)v.data,           \
+                       (const typename Elem<T>::type *)go.data, (typename Elem<T>::type *)ga.data,               \
+                       (typename Elem<T>::type *)gv.data, (int)p.B, (int)p.M, (int)p.w, oblk, orows, iblk, irows, \
+                       a.sb, v.sb, v.sr, go.sb, go.sr, ga.sb, gv.sb, gv.sr);                                      \
+    break;
+#define WM_VUB_ALL(T)                                                                                  \
+  switch (pieces / 2) {                                                                                \
+    WM_VUB(T, 1) WM_VUB(T, 2) WM_VUB(T, 3) WM_VUB(T, 4) WM_VUB(T, 5) WM_VUB(T, 6) WM_VUB(T, 7) WM_VUB(T, 8)   \
+    WM_VUB(T, 9) WM_VUB(T, 10) WM_VUB(T, 11) WM_VUB(T, 12) WM_VUB(T, 13) WM_VUB(T, 14) WM_VUB(T, 15) WM_VUB(T, 16) \
+    default: return false;                                                                             \
+  }
+  if (p.dtype == WM_DTYPE_BF16) {
+    WM_VUB_ALL(bf16_t)
+  } else if (p.dtype == WM_DTYPE_F16) {
+    WM_VUB_ALL(f16_t)
+  } else {
+    WM_VUB_ALL(f32_t)
+  }
+#undef WM_VUB_ALL
+#undef WM_VUB
+  *err = hipGetLastError();
+  return true;
 }
 
 bool try_launch_vector_p1(const Problem &p, const View &x, const View &y, const View &c, hipError_t *err) {
