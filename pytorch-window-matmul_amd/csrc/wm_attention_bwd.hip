@@ -447,6 +447,9 @@ __global__ __launch_bounds__(kThreads) void attention_backward_stats_kernel(
   }
 }
 
+// (Three workgroups per CU up to N = 64: the kernel needs about 157 registers.  Forced into the 128 of a
+// fourth workgroup it spills 35 of them and takes 237 instead of 104 us at B96 M4096 N64 w256; with
+// three workgroups two stages do as well as three, 101 against 104 us, and are what it uses.)
 template <typename T, int NK>
 __global__ __launch_bounds__(kThreads, NK <= 4 ? 3 : 2) void attention_backward_query_dma_kernel(
     const uint16_t *__restrict__ Q, const uint16_t *__restrict__ K, const uint16_t *__restrict__ V,
@@ -456,10 +459,10 @@ __global__ __launch_bounds__(kThreads, NK <= 4 ? 3 : 2) void attention_backward_
     int64_t dqsb, int64_t dqsr) {
   typedef BwdTile<NK> TL;
   constexpr int N = TL::N, NB = TL::NB, PPR = TL::PPR, ROWB = TL::ROWB, TILE = TL::TILE;
-  constexpr int STAGES = TL::STAGES, DEPTH = TL::DEPTH;
+  constexpr int STAGES = 2, DEPTH = STAGES - 1;
   constexpr int LOADS = 2 * (PPR / 4);  // loads per wavefront and chunk (K and V)
-  __shared__ __attribute__((aligned(1024))) uint16_t k_lds[STAGES][TILE];
-  __shared__ __attribute__((aligned(1024))) uint16_t v_lds[STAGES][TILE];
+  __shared__ __attribute__((aligned(1024))) uint16_t kv_lds[2 * STAGES][TILE];  // key tiles, then value tiles
+  uint16_t (*const k_lds)[TILE] = kv_lds, (*const v_lds)[TILE] = kv_lds + STAGES;
 
   int b, blk;
   if (!decode_block(nblk, B, &b, &blk)) return;
@@ -593,7 +596,7 @@ __global__ __launch_bounds__(kThreads, NK <= 4 ? 3 : 2) void attention_backward_
 
   wait_vmcnt<0>();
   __builtin_amdgcn_s_barrier();
-  static_assert(4 * RowStage<NB>::ELEMS <= STAGES * TILE, "the four staging areas must fit the key tiles");
+  static_assert(4 * RowStage<NB>::ELEMS <= 2 * STAGES * TILE, "the four staging areas must fit the tiles");
   store_wave_rows<T, NB>(&k_lds[0][0] + wave * RowStage<NB>::ELEMS, dq, scale, dQ + (int64_t)b * dqsb, dqsr, qw0, M, N,
                          lane);
 }

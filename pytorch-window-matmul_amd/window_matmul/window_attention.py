@@ -19,6 +19,10 @@ from .band_softmax import band_softmax
 from .window_matmul import unwindow_matmul, window_matmul
 
 
+# tensors below this many elements: the step is bound by the host's launches, of which the fused path has fewer
+_HOST_BOUND_ELEMENTS = 32 << 20
+
+
 def _chain_is_faster(window_size: int, width: int, elements: int) -> bool:
     """Whether a training step is faster through the separate ops than through the fused kernels.
     Up to N = 64 the fused backward is one kernel at narrow windows and the fused step wins or ties at
@@ -30,7 +34,7 @@ def _chain_is_faster(window_size: int, width: int, elements: int) -> bool:
     w = 32).  Small problems are bound by the host, which issues seven launches for the chain and three
     for the fused step: at B7 M3001 the chain takes 0.21 ms and the fused step 0.085-0.09 ms whatever the
     window and head width, so below about 32 M elements per tensor the fused kernels are always taken."""
-    if width <= 64 or elements < (32 << 20):
+    if width <= 64 or elements < _HOST_BOUND_ELEMENTS:
         return False
     return window_size <= (24 if width <= 96 else 32)
 

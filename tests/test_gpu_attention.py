@@ -259,27 +259,39 @@ def _graph_nodes(t):
     return {type(fn).__name__ for fn in seen}
 
 
-def test_narrow_window_training_goes_through_the_separate_ops(device):
+def test_narrow_window_training_goes_through_the_separate_ops(device, monkeypatch):
     """Same values either way; the choice only shows in which autograd nodes produced the result.
-    Heads up to 64 wide have a one-kernel backward at narrow windows and stay fused (but for the very
-    narrowest windows of heads up to 32 wide); wider heads train through the separate ops up to w = 36."""
+    Heads up to 64 wide stay fused at every window; wider heads train through the separate ops at narrow
+    windows (up to w = 24 at N = 96, up to w = 32 at N = 128) once the tensors are large enough for the
+    kernels, not the host's launches, to set the pace.  The tensors here are small, so the size rule is
+    switched off for the first pass and checked on its own in the second."""
+    import sys
+
     from window_matmul import window_attention
 
-    for N, w_chain, w_fused in ((96, (8, 36), (40,)), (32, (1, 2), (3, 8, 20)), (64, (), (1, 8, 12, 16, 20))):
-        q, k, v, go = (seeded((2, 200, N), s, torch.bfloat16).to(device) for s in (131, 132, 133, 134))
-        for w in w_chain + w_fused:
-            with torch.no_grad():
-                want = window_attention(q, k, v, w)      # fused forward (one pass up to w = 16 / 32)
-            qq, kk, vv = (t.clone().requires_grad_(True) for t in (q, k, v))
-            out = window_attention(qq, kk, vv, w)
-            nodes = _graph_nodes(out)
-            assert ("UnwindowMatmulFuncBackward" in nodes) == (w in w_chain), (N, w)
-            assert ("WindowAttentionFuncBackward" in nodes) == (w in w_fused), (N, w)
-            torch.testing.assert_close(out.float(), want.float(), **TOL)
-            out.backward(go)
-            want_g = ao.window_attention_backward(q.cpu(), k.cpu(), v.cpu(), w, go.cpu(), 1.0 / math.sqrt(N))
-            for x, y in zip((qq.grad, kk.grad, vv.grad), want_g):
-                close(x, y)
+    module = sys.modules["window_matmul.window_attention"]
+    assert module._chain_is_faster(8, 96, 100 << 20) and not module._chain_is_faster(8, 96, 1 << 20)
+    assert module._chain_is_faster(32, 128, 100 << 20) and not module._chain_is_faster(33, 128, 100 << 20)
+    assert not module._chain_is_faster(1, 64, 100 << 20) and not module._chain_is_faster(2, 32, 100 << 20)
+    for host_bound, cases in ((0, ((96, (8, 24), (25, 40)), (128, (16, 32), (33,)), (32, (), (1, 2, 3, 8, 20)),
+                                   (64, (), (1, 8, 12, 16, 20)))),
+                              (module._HOST_BOUND_ELEMENTS, ((96, (), (8, 24, 40)), (128, (), (16, 33))))):
+        monkeypatch.setattr(module, "_HOST_BOUND_ELEMENTS", host_bound)
+        for N, w_chain, w_fused in cases:
+            q, k, v, go = (seeded((2, 200, N), s, torch.bfloat16).to(device) for s in (131, 132, 133, 134))
+            for w in w_chain + w_fused:
+                with torch.no_grad():
+                    want = window_attention(q, k, v, w)      # fused forward (one pass up to w = 16 / 32)
+                qq, kk, vv = (t.clone().requires_grad_(True) for t in (q, k, v))
+                out = window_attention(qq, kk, vv, w)
+                nodes = _graph_nodes(out)
+                assert ("UnwindowMatmulFuncBackward" in nodes) == (w in w_chain), (N, w)
+                assert ("WindowAttentionFuncBackward" in nodes) == (w in w_fused), (N, w)
+                torch.testing.assert_close(out.float(), want.float(), **TOL)
+                out.backward(go)
+                want_g = ao.window_attention_backward(q.cpu(), k.cpu(), v.cpu(), w, go.cpu(), 1.0 / math.sqrt(N))
+                for x, y in zip((qq.grad, kk.grad, vv.grad), want_g):
+                    close(x, y)
 
 
 @pytest.mark.parametrize("dtype", DTYPES, ids=lambda d: str(d).split(".")[-1])
