@@ -413,7 +413,7 @@ __global__ __launch_bounds__(kThreads, NK <= 4 ? 4 : 2) void attention_forward_d
 
   const u32x4 k_rsrc = make_rsrc(K + (int64_t)b * ksb, (uint32_t)((M - 1) * ksr * 2 + 2 * N));
   const u32x4 v_rsrc = make_rsrc(V + (int64_t)b * vsb, (uint32_t)((M - 1) * vsr * 2 + 2 * N));
-  const bool piece_in_row = (((64 * wave + lane) % PPR) ^ swz((64 * wave + lane) / PPR)) < N / 8;
+  const bool piece_in_row = (((64 * wave + lane) % PPR) ^ swz<PPR>((64 * wave + lane) / PPR)) < N / 8;
   const uint32_t k_voff = piece_in_row ? dma_lane_offset<PPR>(wave, lane, ksr) : 0x80000000u;
   const uint32_t v_voff = piece_in_row ? dma_lane_offset<PPR>(wave, lane, vsr) : 0x80000000u;
   const uint32_t k_step = (uint32_t)(256 / PPR * ksr * 2), v_step = (uint32_t)(256 / PPR * vsr * 2);
@@ -441,17 +441,18 @@ __global__ __launch_bounds__(kThreads, NK <= 4 ? 4 : 2) void attention_forward_d
   // 8 bytes at column 32 hb + 16 (grp % 2) + 4 (s % 4).  The swizzle only touches address bits
   // that the ks / hb terms do not carry into, so those terms are XORed in at the point of use.
   const int r32 = lane & 31;
-  const uint32_t k_at = (uint32_t)(r32 * ROWB + ((half ^ swz(r32)) << 4));
+  const uint32_t k_at = (uint32_t)(r32 * ROWB + ((half ^ swz<PPR>(r32)) << 4));
   const int s16 = lane & 15, grp = lane >> 4, rowl = 4 * (grp >> 1) + (s16 >> 2);
-  const uint32_t v_at = (uint32_t)(rowl * ROWB + (((2 * (grp & 1) + ((s16 & 3) >> 1)) ^ swz(rowl)) << 4) + 8 * (s16 & 1));
+  const uint32_t v_at = (uint32_t)(rowl * ROWB + (((2 * (grp & 1) + ((s16 & 3) >> 1)) ^ swz<PPR>(rowl)) << 4) + 8 * (s16 & 1));
   typedef s16x4 __attribute__((address_space(3))) * lds_tr_ptr;
   auto key_operand = [&](const uint16_t *tile, int kb, int ks) {
     return *reinterpret_cast<const u32x4 *>(reinterpret_cast<const char *>(tile) + 32 * kb * ROWB + (k_at ^ (32 * ks)));
   };
   auto value_operand = [&](const uint16_t *tile, int kb, int t, int hb) {
-    const char *p = reinterpret_cast<const char *>(tile) + (32 * kb + 16 * t) * ROWB + (v_at ^ (64 * hb));
-    const u32x2 lo = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr_ptr)(p)));
-    const u32x2 hi = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr_ptr)(p + 8 * ROWB)));
+    const char *p = reinterpret_cast<const char *>(tile) + (32 * kb + 16 * t) * ROWB;
+    const u32x2 lo = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr_ptr)(p + (v_at ^ (64 * hb)))));
+    const u32x2 hi = __builtin_bit_cast(  // eight rows further down the swizzle differs in bit 1
+        u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr_ptr)(p + 8 * ROWB + (v_at ^ 32 ^ (64 * hb)))));
     const u32x4 r = {lo[0], lo[1], hi[0], hi[1]};
     return r;
   };

@@ -396,18 +396,18 @@ struct BwdTile {
   // byte offset of the lane's piece for the loads of a chunk (dma_chunk), out of range for pieces beyond N
   static __device__ __forceinline__ uint32_t load_offset(int wave, int lane, int64_t row_stride) {
     const int slot = 64 * wave + lane;
-    return ((slot % PPR) ^ swz(slot / PPR)) < N / 8 ? dma_lane_offset<PPR>(wave, lane, row_stride) : 0x80000000u;
+    return ((slot % PPR) ^ swz<PPR>(slot / PPR)) < N / 8 ? dma_lane_offset<PPR>(wave, lane, row_stride) : 0x80000000u;
   }
   static constexpr int STAGES = NK <= 4 ? 3 : 2, DEPTH = STAGES - 1;
   typedef s16x4 __attribute__((address_space(3))) * lds_tr_ptr;
   // byte offsets inside a tile for the two ways a tile is read (see attention_forward_dma_kernel)
   static __device__ __forceinline__ uint32_t row_at(int lane) {
     const int r32 = lane & 31, half = lane >> 5;
-    return (uint32_t)(r32 * ROWB + ((half ^ swz(r32)) << 4));
+    return (uint32_t)(r32 * ROWB + ((half ^ swz<PPR>(r32)) << 4));
   }
   static __device__ __forceinline__ uint32_t tr_at(int lane) {
     const int s16 = lane & 15, grp = lane >> 4, rowl = 4 * (grp >> 1) + (s16 >> 2);
-    return (uint32_t)(rowl * ROWB + (((2 * (grp & 1) + ((s16 & 3) >> 1)) ^ swz(rowl)) << 4) + 8 * (s16 & 1));
+    return (uint32_t)(rowl * ROWB + (((2 * (grp & 1) + ((s16 & 3) >> 1)) ^ swz<PPR>(rowl)) << 4) + 8 * (s16 & 1));
   }
   // rows 32 blk + lane % 32 of the tile, pieces 2 ks + half: A operand of a product contracted over N
   static __device__ __forceinline__ u32x4 rows(const uint16_t *tile, uint32_t at, int blk, int ks) {
@@ -415,9 +415,10 @@ struct BwdTile {
   }
   // columns 32 hb .. + 31 of rows 32 blk + 16 t .. + 15, transposed: A operand of a product contracted over rows
   static __device__ __forceinline__ u32x4 cols(const uint16_t *tile, uint32_t at, int blk, int t, int hb) {
-    const char *p = reinterpret_cast<const char *>(tile) + (32 * blk + 16 * t) * ROWB + (at ^ (64 * hb));
-    const u32x2 lo = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr_ptr)(p)));
-    const u32x2 hi = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr_ptr)(p + 8 * ROWB)));
+    const char *p = reinterpret_cast<const char *>(tile) + (32 * blk + 16 * t) * ROWB;
+    const u32x2 lo = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr_ptr)(p + (at ^ (64 * hb)))));
+    const u32x2 hi = __builtin_bit_cast(  // eight rows further down the swizzle differs in bit 1
+        u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr_ptr)(p + 8 * ROWB + (at ^ 32 ^ (64 * hb)))));
     const u32x4 r = {lo[0], lo[1], hi[0], hi[1]};
     return r;
   }
@@ -840,7 +841,7 @@ __global__ __launch_bounds__(kThreads, NKB >= 4 || (NK >= 3 && NKB == 3) ? 2 : 3
   const float ninf = -__builtin_huge_valf();
   const int r32 = lane & 31;
   const bool want_kv = dK != nullptr || dV != nullptr;
-  // a group of 32 tile rows that starts at row `first` (a multiple of 8) as B operand: row lane % 32,
+  // a group of 32 tile rows that starts at row `first` (a multiple of 16) as B operand: row lane % 32,
   // pieces 2 ks + lane / 32
   auto own_rows = [&](const uint16_t *tile, int first, uint32_t at, int ks) __attribute__((always_inline)) {
     return *reinterpret_cast<const u32x4 *>(reinterpret_cast<const char *>(tile) + first * TL::ROWB + (at ^ (32 * ks)));

@@ -680,7 +680,7 @@ __global__ __launch_bounds__(kThreads, 3) void mfma_p1_dma_kernel(const uint16_t
       const uint32_t base = lds_address(y_lds[k & 1]) + 1024 * wave_s;
 #pragma unroll
       for (int j = 0; j < LOADS; ++j) {
-        const int slot = 64 * (wave_s + 4 * j) + lane, row = slot / PPR, piece = (slot % PPR) ^ swz(row);
+        const int slot = 64 * (wave_s + 4 * j) + lane, row = slot / PPR, piece = (slot % PPR) ^ swz<PPR>(row);
         dma_piece(y_rsrc, base + 4096 * j, (uint32_t)max(cb + row, 0) * y_row_bytes + 16 * piece, 0);
       }
     }
@@ -702,7 +702,7 @@ __global__ __launch_bounds__(kThreads, 3) void mfma_p1_dma_kernel(const uint16_t
     st_src[s] = stage + r * SS + 8 * g;
   }
   uint16_t *stage_wr = stage + (lane & 31) * SS + 4 * (lane >> 5);
-  const uint32_t y_at = (uint32_t)((lane & 31) * ROWB + (((lane >> 5) ^ swz(lane & 31)) << 4));  // byte offset, piece of ks = 0
+  const uint32_t y_at = (uint32_t)((lane & 31) * ROWB + (((lane >> 5) ^ swz<PPR>(lane & 31)) << 4));  // byte offset, piece of ks = 0
 
   // One slot: multiply chunk k, stage the 32 x 64 result and store it.  Returns whether the slot
   // issued exactly the four whole-line stores per lane of a chunk inside the band.
@@ -710,6 +710,8 @@ __global__ __launch_bounds__(kThreads, 3) void mfma_p1_dma_kernel(const uint16_t
     const int buf = k & 1;
     const int cb = c_start + k * KC;
     bool four_stores = false;
+    // chunks of the workgroup's column range that no row of this wavefront reaches
+    if (cb + KC - 1 < iw_first - w || cb > iw_first + 31 + w) return false;
     // multiply and stage; the version for chunks with columns outside the sequence forces those
     // columns to +0.0 (by definition, whatever X holds) and is kept out of the common path
     auto multiply_and_stage = [&](auto edge) {

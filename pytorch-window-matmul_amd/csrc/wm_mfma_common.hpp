@@ -234,10 +234,24 @@ __device__ __forceinline__ void store_wave_rows(uint16_t *stage, const f32x16 (&
 // One wave-level load moves 64 pieces of 16 bytes; lane l's piece lands at LDS base + 16 l, so a
 // tile of R rows x PPR pieces is a flat, unpadded row-major array of 16-byte slots and WHICH piece
 // a lane fetches is the only freedom.  Rows of 128 or 256 bytes (PPR 8 or 16) would put a column of
-// the tile into one bank group, so the piece that lives in slot p of row r is piece p ^ swz(r):
-//   rows r..r+7, same piece (ds_read_b128 by 8 consecutive lanes)       -> 8 distinct bank groups
-//   rows 4n..4n+3, same 32-byte block (ds_read_b64_tr_b16, 16 lanes)     -> 4 distinct blocks
-__device__ __forceinline__ int swz(int r) { return ((r & 3) << 1) | ((r >> 2) & 1); }
+// the tile into one bank group, so the piece that lives in slot p of row r is piece p ^ swz<PPR>(r).
+// LDS reads are served 256 bytes per cycle from 64 banks (ds_read_b128: 16 lanes a cycle,
+// ds_read_b64_tr_b16: 32 lanes a cycle), and a cycle's lanes must fall into 16 different 16-byte
+// bank groups:
+//   rows r..r+15, same piece (ds_read_b128 of an operand with the contraction along the row)
+//   rows 4n..4n+3, the four pieces of a 64-byte block (ds_read_b64_tr_b16, two 16-lane groups)
+// 256-byte rows start in the same bank, so the swizzle alone tells 16 rows apart: row bits 0-1 go
+// to piece bits 2-3 (the rows of a transposing read), row bits 2-3 to piece bits 0-1.  128-byte
+// rows alternate between the two halves of the banks, which takes care of row bit 0: row bit 1
+// goes to piece bit 2, row bits 2-3 to piece bits 0-1.  In both, a row 4 further down has bit 0 of
+// the swizzle flipped and a row 8 further down bit 1; 16 rows further down nothing changes.
+// (Measured per instruction with the swizzle (r & 3) << 1 | (r >> 2) & 1, which tells only 8 rows
+// apart: 8 instead of 4 cycles per ds_read_b128, and 4 instead of 2 per transposing read of 256-byte rows.)
+template <int PPR>
+__device__ __forceinline__ int swz(int r) {
+  static_assert(PPR == 8 || PPR == 16, "rows of 128 or 256 bytes");
+  return PPR == 16 ? ((r & 3) << 2) | ((r >> 2) & 3) : (((r >> 1) & 1) << 2) | (((r >> 3) & 1) << 1) | ((r >> 2) & 1);
+}
 
 // s_waitcnt vmcnt(n) alone (gfx9 encoding: vmcnt in bits 3:0 and 15:14, expcnt 6:4, lgkmcnt 11:8).
 template <int N>
@@ -307,7 +321,7 @@ __device__ __forceinline__ void dma_chunk(u32x4 rsrc, const uint16_t *tile, int 
 // The lane's offset for the above: slot 64 wave + lane of the tile -> row, logical piece.
 template <int PPR>
 __device__ __forceinline__ uint32_t dma_lane_offset(int wave, int lane, int64_t row_stride_elems) {
-  const int slot = 64 * wave + lane, row = slot / PPR, piece = (slot % PPR) ^ swz(row);
+  const int slot = 64 * wave + lane, row = slot / PPR, piece = (slot % PPR) ^ swz<PPR>(row);
   return (uint32_t)(row * row_stride_elems * 2 + piece * 16);
 }
 
@@ -329,7 +343,7 @@ struct LdsTile {
   static __device__ __forceinline__ int load_row(int wave, int lane, int j) { return (64 * wave + lane) / PPR + 256 / PPR * j; }
   static __device__ __forceinline__ int load_piece(int wave, int lane) {
     const int slot = 64 * wave + lane;
-    return (slot % PPR) ^ swz(slot / PPR);
+    return (slot % PPR) ^ swz<PPR>(slot / PPR);
   }
   // bytes in memory between two of the wave's loads (256 / PPR rows)
   static __device__ __forceinline__ uint32_t step(int64_t row_stride_elems) {
@@ -361,7 +375,7 @@ struct LdsTile {
   // 32 ks for pieces 2 ks + lane / 32): operand with the contraction along the row.
   static __device__ __forceinline__ uint32_t row_at(int lane) {
     const int r32 = lane & 31, half = lane >> 5;
-    return (uint32_t)(r32 * ROWB + ((half ^ swz(r32)) << 4));
+    return (uint32_t)(r32 * ROWB + ((half ^ swz<PPR>(r32)) << 4));
   }
   static __device__ __forceinline__ u32x4 rows(const uint16_t *tile, uint32_t at, int blk, int ks) {
     return *reinterpret_cast<const u32x4 *>(reinterpret_cast<const char *>(tile) + 32 * blk * ROWB + (at ^ (32 * ks)));
@@ -371,12 +385,14 @@ struct LdsTile {
   // r0 a multiple of 16.
   static __device__ __forceinline__ uint32_t tr_at(int lane) {
     const int s16 = lane & 15, grp = lane >> 4, rowl = 4 * (grp >> 1) + (s16 >> 2);
-    return (uint32_t)(rowl * ROWB + (((2 * (grp & 1) + ((s16 & 3) >> 1)) ^ swz(rowl)) << 4) + 8 * (s16 & 1));
+    return (uint32_t)(rowl * ROWB + (((2 * (grp & 1) + ((s16 & 3) >> 1)) ^ swz<PPR>(rowl)) << 4) + 8 * (s16 & 1));
   }
   static __device__ __forceinline__ u32x4 cols(const uint16_t *tile, uint32_t at, int r0, int cb) {
-    const char *p = reinterpret_cast<const char *>(tile) + r0 * ROWB + (at ^ (64 * cb));
-    const u32x2 lo = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr_ptr)(p)));
-    const u32x2 hi = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr_ptr)(p + 8 * ROWB)));
+    const char *p = reinterpret_cast<const char *>(tile) + r0 * ROWB;
+    // eight rows further down the swizzle differs in bit 1
+    const u32x2 lo = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr_ptr)(p + (at ^ (64 * cb)))));
+    const u32x2 hi = __builtin_bit_cast(
+        u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr_ptr)(p + 8 * ROWB + (at ^ 32 ^ (64 * cb)))));
     const u32x4 r = {lo[0], lo[1], hi[0], hi[1]};
     return r;
   }
@@ -384,7 +400,7 @@ struct LdsTile {
   // r0 + 8 (lane / 32) + {0 .. 7}: the order in which `rows` of another tile delivers its pieces.
   static __device__ __forceinline__ uint32_t tr_at_seq(int lane) {
     const int s16 = lane & 15, grp = lane >> 4, rowl = 8 * (grp >> 1) + (s16 >> 2);
-    return (uint32_t)(rowl * ROWB + (((2 * (grp & 1) + ((s16 & 3) >> 1)) ^ swz(rowl)) << 4) + 8 * (s16 & 1));
+    return (uint32_t)(rowl * ROWB + (((2 * (grp & 1) + ((s16 & 3) >> 1)) ^ swz<PPR>(rowl)) << 4) + 8 * (s16 & 1));
   }
   static __device__ __forceinline__ u32x4 cols_seq(const uint16_t *tile, uint32_t at, int r0, int cb) {
     const char *p = reinterpret_cast<const char *>(tile) + r0 * ROWB;
