@@ -71,6 +71,10 @@ hipError_t launch_strided_p3(const Problem &p, const View &a, const View &y, con
 bool try_launch_mfma_p1(const Problem &p, const View &x, const View &y, const View &c, hipError_t *err);
 bool try_launch_mfma_p2(const Problem &p, const View &a, const View &y, const View &c, hipError_t *err);
 bool try_launch_mfma_p3(const Problem &p, const View &a, const View &y, const View &c, hipError_t *err);
+// Whether the band-in kernels of that family that load their tiles straight into LDS accept the
+// layout of band `a` and operand `y` (the shape aside): what the narrow-band family asks before it
+// leaves a window to them.
+bool lds_direct_layout_ok(const Problem &p, const View &a, const View &y);
 // Narrow-band family (w <= 32; P2 and P3 while their LDS images fit 64 KB; float32 at N <= 64).
 bool try_launch_small_p1(const Problem &p, const View &x, const View &y, const View &c, hipError_t *err);
 bool try_launch_small_p2(const Problem &p, const View &a, const View &y, const View &c, hipError_t *err);

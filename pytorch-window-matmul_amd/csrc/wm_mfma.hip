@@ -1116,8 +1116,7 @@ unsigned tile_shares(int64_t tiles, int64_t chunks) {
 // alignment to launch with (64, 8 or 2 elements), 0 if the shape is not accepted.
 template <bool ALIGNED>
 int lds_direct_group(const Problem &p, const View &a, const View &y) {
-  if ((p.flags & WM_FLAG_NO_LDS_DIRECT) || y.sr <= 0 || ((uintptr_t)a.data % 4) != 0) return 0;
-  if ((p.M + 4 * KC) * (2 * p.w + 1) * 2 + 256 >= 0x7fffffff || (p.M + 4 * KC) * y.sr * 2 >= 0x7fffffff) return 0;
+  if (!lds_direct_layout_ok(p, a, y)) return 0;
   return ALIGNED ? band_group(a, p.w) : 2;
 }
 
@@ -1291,6 +1290,11 @@ hipError_t by_dtype(int op, const Problem &p, const View &a, const View &y, cons
 }
 
 }  // namespace
+
+bool lds_direct_layout_ok(const Problem &p, const View &a, const View &y) {
+  if ((p.flags & WM_FLAG_NO_LDS_DIRECT) || y.sr <= 0 || ((uintptr_t)a.data % 4) != 0) return false;
+  return (p.M + 4 * KC) * (2 * p.w + 1) * 2 + 256 < 0x7fffffff && (p.M + 4 * KC) * y.sr * 2 < 0x7fffffff;
+}
 
 bool mfma_supports(int op, int64_t B, int64_t M, int64_t N, int64_t w, int dtype) {
   (void)op;

@@ -975,7 +975,10 @@ bool try_launch_small_p1(const Problem &p, const View &x, const View &y, const V
 }
 
 bool try_launch_small_p2(const Problem &p, const View &a, const View &y, const View &c, hipError_t *err) {
-  if (!small_supports(2, p.M, p.N, p.w, p.dtype, p.flags)) return false;
+  // a window is left to the wide-band kernels only where the ones that were measured faster, those
+  // with tiles straight into LDS, take this layout
+  const unsigned flags = lds_direct_layout_ok(p, a, y) ? p.flags : p.flags | WM_FLAG_NO_LDS_DIRECT;
+  if (!small_supports(2, p.M, p.N, p.w, p.dtype, flags)) return false;
   if (!band_contiguous(a, 2 * p.w + 1) || !fast_layout(y, p.dtype) || !fast_layout(c, p.dtype)) return false;
   if (p.dtype == WM_DTYPE_F32) {
     *err = launch_small_in_f32<false>(p, a, y, c);
@@ -986,7 +989,10 @@ bool try_launch_small_p2(const Problem &p, const View &a, const View &y, const V
 }
 
 bool try_launch_small_p3(const Problem &p, const View &a, const View &y, const View &c, hipError_t *err) {
-  if (!small_supports(3, p.M, p.N, p.w, p.dtype, p.flags)) return false;
+  // a window is left to the wide-band kernels only where the ones that were measured faster, those
+  // with tiles straight into LDS, take this layout
+  const unsigned flags = lds_direct_layout_ok(p, a, y) ? p.flags : p.flags | WM_FLAG_NO_LDS_DIRECT;
+  if (!small_supports(3, p.M, p.N, p.w, p.dtype, flags)) return false;
   if (!band_contiguous(a, 2 * p.w + 1) || !fast_layout(y, p.dtype) || !fast_layout(c, p.dtype)) return false;
   if (p.dtype == WM_DTYPE_F32) {
     *err = launch_small_in_f32<true>(p, a, y, c);

@@ -139,11 +139,12 @@ def test_band_out_ring_of_lines(device, B, M, N, w, dtype):
             torch.testing.assert_close(want[b, rows].float().cpu(), ref, **TOL)
 
 
-@pytest.mark.parametrize("w", [40, 41, 64])
+@pytest.mark.parametrize("w", [16, 24, 40, 41, 64])
 def test_band_at_an_odd_element_offset(device, w):
     """A band whose first element sits at an odd element offset is only 2-byte aligned: neither the
     16-byte pieces of the LDS-direct kernels nor the whole-line stores apply, the products take the
-    kernels for unaligned bands and give the numbers of the aligned call."""
+    kernels for unaligned bands (at w = 16 and 24 the narrow-band ones, which leave those windows
+    to the LDS-direct kernels only for layouts those accept) and give the numbers of the aligned call."""
     B, M, N, dtype = 3, 700, 64, torch.bfloat16
     W = 2 * w + 1
     q, k, v, go = (seeded((B, M, N), 350 + s, dtype).to(device) for s in range(4))
