@@ -1252,11 +1252,14 @@ hipError_t launch_p1(const Problem &p, const View &x, const View &y, const View 
   // N = 128 with whole-line band stores: Y chunks straight into LDS, three workgroups per CU (32-bit
   // byte offsets inside a batch element).  With 16-byte column groups most slots take the piecewise
   // store path, whose stores this kernel waits for: 10 % slower there than the kernel above.
+  // It runs one workgroup per tile: with few tiles the kernel above, which shares them out, is ahead
+  // (fp16/bf16, this kernel / the one above: B1 M8192 w2048, 64 tiles: 72 / 28 us; B2 M4096 w1024: 41 /
+  // 18; B4 M4096 w256, 128 tiles: 17.9 / 14.6; B6 M4096 w128, 192 tiles: 14.0 / 15.0; B7 M4096 w512,
+  // 224 tiles: 25.9 / 26.5).
   if (ALIGNED && galign == 64 && !(p.flags & WM_FLAG_NO_LDS_DIRECT) && y.sr > 0 &&
-      (p.M + 2 * KC) * y.sr * 2 < 0x7fffffff && p.N == 128) {
+      (p.M + 2 * KC) * y.sr * 2 < 0x7fffffff && p.N == 128 && (shares == 1 || p.B * nblk >= 160)) {
     // (at N = 64, where the kernel above already places four workgroups on a CU, this variant measured
     // equal at w = 256 and 512 and 8 % slower at w = 64)
-    // (one workgroup per tile: this kernel does not share tiles out)
     hipLaunchKernelGGL((mfma_p1_dma_kernel<T, 8, ALIGNED>), dim3(grid.x), block, 0, p.stream, (const uint16_t *)x.data,
                        (const uint16_t *)y.data, (uint16_t *)c.data, (int)p.B, (int)p.M, (int)p.w, nblk, galign, x.sb,
                        x.sr, y.sb, y.sr, c.sb);
