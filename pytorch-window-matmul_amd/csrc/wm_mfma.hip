@@ -29,6 +29,7 @@
 #include "wm_mfma_common.hpp"
 
 #include <algorithm>
+#include <cstdlib>
 #include <type_traits>
 
 namespace wm {
@@ -886,7 +887,10 @@ __global__ __launch_bounds__(kThreads, (160 * 1024 / (STAGES * KCH * (2 * TM + (
   const bool lines = galign == 64;
   const uint32_t t_voff = TT::lane_offset(wave, lane, 2 * w), t_step = TT::step(2 * w);
   const uint32_t t_col0 = (uint32_t)(a_rem + c0 + w) * 2, t_row = (uint32_t)(4 * w);  // bytes
-  const u32x4 y_rsrc = make_rsrc(Y + (int64_t)b * ysb, (uint32_t)(((int64_t)(M - 1) * ysr + N) * 2));
+  // blockIdx.y selects which N columns of Y and C this workgroup works on (launches with few tiles
+  // give every block of columns workgroups of its own; otherwise there is one block)
+  const int h0 = N * (int)blockIdx.y;
+  const u32x4 y_rsrc = make_rsrc(Y + (int64_t)b * ysb + h0, (uint32_t)(((int64_t)(M - 1) * ysr + N) * 2));
   // (pieces of the Y tile beyond column N are requested out of range: zeros, no memory traffic)
   const uint32_t y_voff = YT::load_piece(wave, lane) < N / 8 ? YT::lane_offset(wave, lane, ysr) : 0x80000000u;
   const uint32_t y_step = YT::step(ysr), y_row = (uint32_t)(ysr * 2);
@@ -958,8 +962,8 @@ __global__ __launch_bounds__(kThreads, (160 * 1024 / (STAGES * KCH * (2 * TM + (
   wait_vmcnt<0>();
   __syncthreads();
   static_assert(4 * RowStage<NT>::ELEMS <= STAGES * TT::ELEMS, "the four staging areas must fit the band tile buffers");
-  store_wave_rows<T, NT>(&t_lds[0][0] + wave * RowStage<NT>::ELEMS, acc, 1.0f, C + (int64_t)b * csb, csr, cw0, M, N,
-                         lane);
+  store_wave_rows<T, NT>(&t_lds[0][0] + wave * RowStage<NT>::ELEMS, acc, 1.0f, C + (int64_t)b * csb + h0, csr, cw0, M,
+                         N, lane);
 }
 
 // ------------------------------------------------------------------------------------------
@@ -1003,7 +1007,10 @@ __global__ __launch_bounds__(kThreads, (160 * 1024 / (STAGES * KC * (2 * TM + (N
   const bool lines = galign == 64;  // whole-line column groups: the band is streamed (non-temporal)
   const uint32_t t_voff = TT::lane_offset(wave, lane, 2 * w) + (uint32_t)(a_rem + (int64_t)i0 * 2 * w + w) * 2;
   const uint32_t t_step = TT::step(2 * w);
-  const u32x4 y_rsrc = make_rsrc(Y + (int64_t)b * ysb, (uint32_t)(((int64_t)(M - 1) * ysr + N) * 2));
+  // blockIdx.y selects which N columns of Y and C this workgroup works on (launches with few tiles
+  // give every block of columns workgroups of its own; otherwise there is one block)
+  const int h0 = N * (int)blockIdx.y;
+  const u32x4 y_rsrc = make_rsrc(Y + (int64_t)b * ysb + h0, (uint32_t)(((int64_t)(M - 1) * ysr + N) * 2));
   const bool y_piece = YT::load_piece(wave, lane) < N / 8;  // else: beyond column N, requested out of range
   const uint32_t y_voff = YT::lane_offset(wave, lane, ysr), y_step = YT::step(ysr), y_row = (uint32_t)(ysr * 2);
   // pieces of the band tile that hold no entry of the band (8 columns from c8 of row i with c8 - i
@@ -1075,8 +1082,8 @@ __global__ __launch_bounds__(kThreads, (160 * 1024 / (STAGES * KC * (2 * TM + (N
   wait_vmcnt<0>();
   __syncthreads();
   static_assert(4 * RowStage<NT>::ELEMS <= STAGES * TT::ELEMS, "the four staging areas must fit the band tile buffers");
-  store_wave_rows<T, NT>(&t_lds[0][0] + wave * RowStage<NT>::ELEMS, acc, 1.0f, C + (int64_t)b * csb, csr, iw0, M, N,
-                         lane);
+  store_wave_rows<T, NT>(&t_lds[0][0] + wave * RowStage<NT>::ELEMS, acc, 1.0f, C + (int64_t)b * csb + h0, csr, iw0, M,
+                         N, lane);
 }
 
 // ------------------------------------------------------------------------------------------
@@ -1110,6 +1117,17 @@ unsigned tile_shares(int64_t tiles, int64_t chunks) {
   return (unsigned)std::max<int64_t>(1, std::min<int64_t>({want, chunks / 4, 64}));
 }
 
+// Column blocks of the band-in kernels that load their tiles straight into LDS.  A workgroup alone on
+// its CU is bound by its own chunk step (operand reads, then the MFMAs of every column block, one
+// wavefront per SIMD with nothing to overlap them), not by its bytes, so a launch with no more tiles
+// than half the CUs gives every 32 or 64 columns of Y workgroups of their own; the band tile is then
+// fetched once per block, from L2 after the first.  Returns the width of a block in units of 16.
+int band_in_column_block(int64_t tiles, int64_t N) {
+  static const bool off = getenv("WM_NO_COLUMN_BLOCKS") != nullptr;
+  if (off || 2 * tiles > kCUs || N % 32 != 0 || N < 64) return (int)(N / 16);
+  return (N % 64 == 0 && 4 * tiles > kCUs) ? 4 : 2;
+}
+
 // Shapes the kernels that load their tiles straight into LDS accept (band-in products): 32-bit byte
 // offsets inside a batch element of the band and of Y (chunks past the end included), and band rows
 // that can be cut into 16-byte pieces at 4-byte aligned addresses.  Returns the column-group
@@ -1137,13 +1155,15 @@ hipError_t launch_p2(const Problem &p, const View &a, const View &y, const View 
   // the band outgrows the last-level cache the kernel below, with two chunks per workgroup in flight,
   // is 2-4 % faster at N = 64 (B = 384 at w = 256; B = 32, M = 32768 at w = 512): not worth a rule.
   if (const int g = lds_direct_group<ALIGNED>(p, a, y)) {
+    const int nkb = band_in_column_block(p.B * nblk, p.N);
+    const dim3 grid_c(grid.x, (unsigned)(p.N / 16 / nkb));
 #define WM_P2_DMA(NK, STAGES)                                                                                  \
   case NK:                                                                                                     \
-    hipLaunchKernelGGL((mfma_p2_dma_kernel<T, NK, STAGES>), grid, block, 0, p.stream, (const uint16_t *)a.data, \
+    hipLaunchKernelGGL((mfma_p2_dma_kernel<T, NK, STAGES>), grid_c, block, 0, p.stream, (const uint16_t *)a.data, \
                        (const uint16_t *)y.data, (uint16_t *)c.data, (int)p.B, (int)p.M, (int)p.w, nblk, g,    \
                        a.sb, y.sb, y.sr, c.sb, c.sr);                                                          \
     break;
-    switch (p.N / 16) {
+    switch (nkb) {
       WM_P2_DMA(1, 2) WM_P2_DMA(2, 2) WM_P2_DMA(3, 2) WM_P2_DMA(4, 2) WM_P2_DMA(5, 2) WM_P2_DMA(6, 2) WM_P2_DMA(7, 2)
       WM_P2_DMA(8, 2)
     }
@@ -1174,8 +1194,9 @@ hipError_t launch_p3(const Problem &p, const View &a, const View &y, const View 
   // 23 % at B = 32, M = 32768, w = 64; 9-13 % at config 4; 4 % at B = 384, w = 256; equal at B = 32,
   // M = 32768, w = 512.
   if (const int g = lds_direct_group<ALIGNED>(p, a, y)) {
-    const dim3 grid_g(grid_size(p.B, (p.M + g - 1 + TM - 1) / TM));
     const int nblk_g = (int)((p.M + g - 1 + TM - 1) / TM);
+    const int nkb = band_in_column_block(p.B * ((p.M + TM - 1) / TM), p.N);
+    const dim3 grid_g(grid_size(p.B, nblk_g), (unsigned)(p.N / 16 / nkb));
 #define WM_P3_DMA(NK, KCH, STAGES)                                                                             \
   case NK:                                                                                                     \
     hipLaunchKernelGGL((mfma_p3_dma_kernel<T, NK, KCH, STAGES>), grid_g, block, 0, p.stream,                   \
@@ -1187,9 +1208,9 @@ hipError_t launch_p3(const Problem &p, const View &a, const View &y, const View 
     // against 140 us at w = 33, 130 against 145 at w = 48, 175 against 188 at w = 96, 206 against 216
     // at w = 128, 349 against 329 at w = 200).
     if (p.N <= 64 && p.w < kShallowChunksBelow) {
-      switch (p.N / 16) { WM_P3_DMA(1, 32, 3) WM_P3_DMA(2, 32, 3) WM_P3_DMA(3, 32, 3) WM_P3_DMA(4, 32, 3) }
+      switch (nkb) { WM_P3_DMA(1, 32, 3) WM_P3_DMA(2, 32, 3) WM_P3_DMA(3, 32, 3) WM_P3_DMA(4, 32, 3) }
     } else {
-      switch (p.N / 16) {
+      switch (nkb) {
         WM_P3_DMA(1, WM_P3_DMA_KC, WM_P3_DMA_STAGES) WM_P3_DMA(2, WM_P3_DMA_KC, WM_P3_DMA_STAGES)
         WM_P3_DMA(3, WM_P3_DMA_KC, WM_P3_DMA_STAGES) WM_P3_DMA(4, WM_P3_DMA_KC, WM_P3_DMA_STAGES)
         WM_P3_DMA(5, WM_P3_DMA_KC, WM_P3_DMA_STAGES) WM_P3_DMA(6, WM_P3_DMA_KC, WM_P3_DMA_STAGES)

@@ -6,7 +6,8 @@ head width, for any window as long as the band is 4-byte aligned).  ``WM_FLAG_NO
 switches them off, so every shape here runs both ways: the results must agree within the 16-bit
 tolerance (rtol = atol = 2e-2; bit for bit where the order of the sums is the same: band-out
 product, and band-in product when the window is a multiple of 4), and both must match the CPU
-oracle.  Shapes cover ragged sequence ends, sequences shorter than a tile, batch elements whose band does not start on a 128-byte line, operands with padded rows and
+oracle.  Every shape here has fewer tiles than half the CUs, so the band-in products with N a multiple
+of 32 run with one workgroup per block of 32 or 64 columns of Y.  Shapes cover ragged sequence ends, sequences shorter than a tile, batch elements whose band does not start on a 128-byte line, operands with padded rows and
 batches, and invalid band entries filled with NaN.
 """
 import pytest
