@@ -29,7 +29,6 @@
 #include "wm_mfma_common.hpp"
 
 #include <algorithm>
-#include <cstdlib>
 #include <type_traits>
 
 namespace wm {
@@ -1123,8 +1122,7 @@ unsigned tile_shares(int64_t tiles, int64_t chunks) {
 // than half the CUs gives every 32 or 64 columns of Y workgroups of their own; the band tile is then
 // fetched once per block, from L2 after the first.  Returns the width of a block in units of 16.
 int band_in_column_block(int64_t tiles, int64_t N) {
-  static const bool off = getenv("WM_NO_COLUMN_BLOCKS") != nullptr;
-  if (off || 2 * tiles > kCUs || N % 32 != 0 || N < 64) return (int)(N / 16);
+  if (2 * tiles > kCUs || N % 32 != 0 || N < 64) return (int)(N / 16);
   return (N % 64 == 0 && 4 * tiles > kCUs) ? 4 : 2;
 }
 
