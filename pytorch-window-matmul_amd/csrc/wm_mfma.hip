@@ -854,7 +854,7 @@ __global__ __launch_bounds__(kThreads, (160 * 1024 / (STAGES * KCH * (2 * TM + (
                                            : 160 * 1024 / (STAGES * KCH * (2 * TM + (NK <= 4 ? 128 : 256))) >= 3
                                                  ? 3
                                                  : 160 * 1024 / (STAGES * KCH * (2 * TM + (NK <= 4 ? 128 : 256))) >= 2 ? 2 : 1)) void mfma_p3_dma_kernel(
-    const uint16_t *__restrict__ A, const uint16_t *__restrict__ Y, uint16_t *__restrict__ C, int B, int M, int w,
+    const uint16_t *__restrict__ A, const uint16_t *__restrict__ Y, uint16_t *__restrict__ C, int B, int M, int n_total, int w,
     int nblk, int galign, int64_t asb, int64_t ysb, int64_t ysr, int64_t csb, int64_t csr) {
   constexpr int N = 16 * NK, NT = (NK + 1) / 2, CH = KCH, DEPTH = STAGES - 1;
   using TT = LdsTile<CH, TM / 8>;            // [CH rows r][TM columns c]
@@ -889,9 +889,10 @@ __global__ __launch_bounds__(kThreads, (160 * 1024 / (STAGES * KCH * (2 * TM + (
   // blockIdx.y selects which N columns of Y and C this workgroup works on (launches with few tiles
   // give every block of columns workgroups of its own; otherwise there is one block)
   const int h0 = N * (int)blockIdx.y;
-  const u32x4 y_rsrc = make_rsrc(Y + (int64_t)b * ysb + h0, (uint32_t)(((int64_t)(M - 1) * ysr + N) * 2));
+  const int n_cols = min(N, n_total - h0);  // (the last block of a width that is no multiple of N is narrower)
+  const u32x4 y_rsrc = make_rsrc(Y + (int64_t)b * ysb + h0, (uint32_t)(((int64_t)(M - 1) * ysr + n_cols) * 2));
   // (pieces of the Y tile beyond column N are requested out of range: zeros, no memory traffic)
-  const uint32_t y_voff = YT::load_piece(wave, lane) < N / 8 ? YT::lane_offset(wave, lane, ysr) : 0x80000000u;
+  const uint32_t y_voff = YT::load_piece(wave, lane) < n_cols / 8 ? YT::lane_offset(wave, lane, ysr) : 0x80000000u;
   const uint32_t y_step = YT::step(ysr), y_row = (uint32_t)(ysr * 2);
   // A piece of the band tile (8 columns from c8 of band row r) holds an entry of the band only if
   // c8 - r lies in [-w - 7, w]; the others are requested beyond the end of the buffer, which costs no
@@ -962,7 +963,7 @@ __global__ __launch_bounds__(kThreads, (160 * 1024 / (STAGES * KCH * (2 * TM + (
   __syncthreads();
   static_assert(4 * RowStage<NT>::ELEMS <= STAGES * TT::ELEMS, "the four staging areas must fit the band tile buffers");
   store_wave_rows<T, NT>(&t_lds[0][0] + wave * RowStage<NT>::ELEMS, acc, 1.0f, C + (int64_t)b * csb + h0, csr, cw0, M,
-                         N, lane);
+                         n_cols, lane);
 }
 
 // ------------------------------------------------------------------------------------------
@@ -976,7 +977,7 @@ template <typename T, int NK, int STAGES>
 __global__ __launch_bounds__(kThreads, (160 * 1024 / (STAGES * KC * (2 * TM + (NK <= 4 ? 128 : 256))) >= 3
                                            ? 3
                                            : 160 * 1024 / (STAGES * KC * (2 * TM + (NK <= 4 ? 128 : 256))) >= 2 ? 2 : 1)) void mfma_p2_dma_kernel(
-    const uint16_t *__restrict__ A, const uint16_t *__restrict__ Y, uint16_t *__restrict__ C, int B, int M, int w,
+    const uint16_t *__restrict__ A, const uint16_t *__restrict__ Y, uint16_t *__restrict__ C, int B, int M, int n_total, int w,
     int nblk, int galign, int64_t asb, int64_t ysb, int64_t ysr, int64_t csb, int64_t csr) {
   constexpr int N = 16 * NK, NT = (NK + 1) / 2, DEPTH = STAGES - 1;
   using TT = LdsTile<TM, KC / 8>;            // [TM rows i][KC dense columns c]
@@ -1009,8 +1010,9 @@ __global__ __launch_bounds__(kThreads, (160 * 1024 / (STAGES * KC * (2 * TM + (N
   // blockIdx.y selects which N columns of Y and C this workgroup works on (launches with few tiles
   // give every block of columns workgroups of its own; otherwise there is one block)
   const int h0 = N * (int)blockIdx.y;
-  const u32x4 y_rsrc = make_rsrc(Y + (int64_t)b * ysb + h0, (uint32_t)(((int64_t)(M - 1) * ysr + N) * 2));
-  const bool y_piece = YT::load_piece(wave, lane) < N / 8;  // else: beyond column N, requested out of range
+  const int n_cols = min(N, n_total - h0);  // (the last block of a width that is no multiple of N is narrower)
+  const u32x4 y_rsrc = make_rsrc(Y + (int64_t)b * ysb + h0, (uint32_t)(((int64_t)(M - 1) * ysr + n_cols) * 2));
+  const bool y_piece = YT::load_piece(wave, lane) < n_cols / 8;  // else: beyond the block's columns, requested out of range
   const uint32_t y_voff = YT::lane_offset(wave, lane, ysr), y_step = YT::step(ysr), y_row = (uint32_t)(ysr * 2);
   // pieces of the band tile that hold no entry of the band (8 columns from c8 of row i with c8 - i
   // outside [-w - 7, w]) are requested beyond the end of the buffer: no memory traffic for them
@@ -1082,7 +1084,7 @@ __global__ __launch_bounds__(kThreads, (160 * 1024 / (STAGES * KC * (2 * TM + (N
   __syncthreads();
   static_assert(4 * RowStage<NT>::ELEMS <= STAGES * TT::ELEMS, "the four staging areas must fit the band tile buffers");
   store_wave_rows<T, NT>(&t_lds[0][0] + wave * RowStage<NT>::ELEMS, acc, 1.0f, C + (int64_t)b * csb + h0, csr, iw0, M,
-                         N, lane);
+                         n_cols, lane);
 }
 
 // ------------------------------------------------------------------------------------------
@@ -1118,12 +1120,19 @@ unsigned tile_shares(int64_t tiles, int64_t chunks) {
 
 // Column blocks of the band-in kernels that load their tiles straight into LDS.  A workgroup alone on
 // its CU is bound by its own chunk step (operand reads, then the MFMAs of every column block, one
-// wavefront per SIMD with nothing to overlap them), not by its bytes, so a launch with no more tiles
-// than half the CUs gives every 32 or 64 columns of Y workgroups of their own; the band tile is then
-// fetched once per block, from L2 after the first.  Returns the width of a block in units of 16.
+// wavefront per SIMD with nothing to overlap them), not by its bytes, so a launch with few tiles gives
+// every two to four 16-column groups of Y workgroups of their own (`blockIdx.y`; the last block may be
+// narrower); the band tile is then fetched once per block, from L2 after the first.  Measured under
+// graph replay, bf16, band-in / transposed, us, with / without: 32 tiles N128 w256 9.4 / 14.7 and 10.3 /
+// 14.4; 128 tiles N128 w1024 31.5 / 38.5; 160 tiles N128 w512 19.5 / 22.7; 168 tiles N80 w1500 38.6 /
+// 43.9 and 37.1 / 43.0; 192 tiles N128 w256 13.5 / 15.4; level at 224 tiles N128 w512; at N = 64 level up
+// to 192 tiles and 13 % slower at 224 tiles w1024, 40 % slower at 384.  Returns the width of a block in
+// units of 16 columns.
 int band_in_column_block(int64_t tiles, int64_t N) {
-  if (2 * tiles > kCUs || N % 32 != 0 || N < 64) return (int)(N / 16);
-  return (N % 64 == 0 && 4 * tiles > kCUs) ? 4 : 2;
+  const int nk = (int)(N / 16);
+  if (tiles > (N > 64 ? 200 : kCUs / 2) || nk < 4) return nk;
+  const int blocks = 4 * tiles > kCUs ? 2 : 4;
+  return std::max(2, (nk + blocks - 1) / blocks);
 }
 
 // Shapes the kernels that load their tiles straight into LDS accept (band-in products): 32-bit byte
@@ -1154,12 +1163,12 @@ hipError_t launch_p2(const Problem &p, const View &a, const View &y, const View 
   // is 2-4 % faster at N = 64 (B = 384 at w = 256; B = 32, M = 32768 at w = 512): not worth a rule.
   if (const int g = lds_direct_group<ALIGNED>(p, a, y)) {
     const int nkb = band_in_column_block(p.B * nblk, p.N);
-    const dim3 grid_c(grid.x, (unsigned)(p.N / 16 / nkb));
+    const dim3 grid_c(grid.x, (unsigned)((p.N / 16 + nkb - 1) / nkb));
 #define WM_P2_DMA(NK, STAGES)                                                                                  \
   case NK:                                                                                                     \
     hipLaunchKernelGGL((mfma_p2_dma_kernel<T, NK, STAGES>), grid_c, block, 0, p.stream, (const uint16_t *)a.data, \
-                       (const uint16_t *)y.data, (uint16_t *)c.data, (int)p.B, (int)p.M, (int)p.w, nblk, g,    \
-                       a.sb, y.sb, y.sr, c.sb, c.sr);                                                          \
+                       (const uint16_t *)y.data, (uint16_t *)c.data, (int)p.B, (int)p.M, (int)p.N, (int)p.w,   \
+                       nblk, g, a.sb, y.sb, y.sr, c.sb, c.sr);                                                 \
     break;
     switch (nkb) {
       WM_P2_DMA(1, 2) WM_P2_DMA(2, 2) WM_P2_DMA(3, 2) WM_P2_DMA(4, 2) WM_P2_DMA(5, 2) WM_P2_DMA(6, 2) WM_P2_DMA(7, 2)
@@ -1194,12 +1203,12 @@ hipError_t launch_p3(const Problem &p, const View &a, const View &y, const View 
   if (const int g = lds_direct_group<ALIGNED>(p, a, y)) {
     const int nblk_g = (int)((p.M + g - 1 + TM - 1) / TM);
     const int nkb = band_in_column_block(p.B * ((p.M + TM - 1) / TM), p.N);
-    const dim3 grid_g(grid_size(p.B, nblk_g), (unsigned)(p.N / 16 / nkb));
+    const dim3 grid_g(grid_size(p.B, nblk_g), (unsigned)((p.N / 16 + nkb - 1) / nkb));
 #define WM_P3_DMA(NK, KCH, STAGES)                                                                             \
   case NK:                                                                                                     \
     hipLaunchKernelGGL((mfma_p3_dma_kernel<T, NK, KCH, STAGES>), grid_g, block, 0, p.stream,                   \
                        (const uint16_t *)a.data, (const uint16_t *)y.data, (uint16_t *)c.data, (int)p.B,       \
-                       (int)p.M, (int)p.w, nblk_g, g, a.sb, y.sb, y.sr, c.sb, c.sr);                           \
+                       (int)p.M, (int)p.N, (int)p.w, nblk_g, g, a.sb, y.sb, y.sr, c.sb, c.sr);                 \
     break;
     // A band of a few chunks only: chunks of 32 rows, three deep, fit four workgroups on a CU up to
     // N = 64 and overfetch less at the band's edges (B96 M16384 N64, 32- against 64-row chunks: 119
