@@ -61,6 +61,12 @@ for _w in (1, 33, 1500):
             WORKLOADS[f"c5_w{_w}_{_dt}"] = dict(
                 B=7, M=3001, N=80, w=_w, dtype=_dt, qk_scale=1.0, backward=True,
                 label=f"B7 M3001 N80 w{_w} {_dt}, window->softmax->unwindow, fwd+bwd")
+# a single long sequence and a single short one (launches with far fewer tiles than CUs; --kernels-only
+# runs for the kernel trace in profiles/, not part of the default run)
+WORKLOADS["one_sequence_16k"] = dict(B=1, M=16384, N=128, w=1024, dtype="bf16", qk_scale=1.0, backward=True,
+                                     label="B1 M16384 N128 w1024 bf16, window->softmax->unwindow, fwd+bwd")
+WORKLOADS["one_sequence_4k"] = dict(B=1, M=4096, N=128, w=256, dtype="bf16", qk_scale=1.0, backward=True,
+                                    label="B1 M4096 N128 w256 bf16, window->softmax->unwindow, fwd+bwd")
 # source files the dominant kernel of the headline configuration can come from (the wide-band 16-bit
 # family, its shared headers and the dispatcher that picks it): the digest of these guards the HBM
 # traffic figure stored in profiles/config3_bf16_hbm_traffic.md
